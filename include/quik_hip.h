@@ -1,0 +1,130 @@
+/* C ABI of libquik_hip.so: the MI355X (gfx950) implementation of the forward path of
+ * QUIK's MixedQLinear.  Plain pointers and sizes only; every pointer is DEVICE memory on
+ * the current HIP device unless stated otherwise, every output buffer is allocated by the
+ * caller, `stream` is a hipStream_t passed as void* (NULL = the default stream), and all
+ * calls are asynchronous with respect to the host.  Every function returns QUIK_OK (0) or
+ * a negative quik_status; quik_status_string() gives the message the Python layer raises.
+ *
+ * Each entry point names the interface of the reference it replaces (paths relative to
+ * the reference checkout).  The reference returns freshly allocated tensors; here the
+ * thin host layer (quik_amd/_ops.py) allocates and this library only fills.
+ */
+#ifndef QUIK_HIP_H_
+#define QUIK_HIP_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum quik_status {
+  QUIK_OK = 0,
+  QUIK_ERR_BITS = -1,      /* bits argument must be either 4 or 8 (or 8/16/32 for symmetric dequantize) */
+  QUIK_ERR_SHAPE = -2,     /* sizes inconsistent with each other */
+  QUIK_ERR_DTYPE = -3,     /* dtype id not QUIK_F16 / QUIK_BF16, or not supported by this op */
+  QUIK_ERR_ALIGN = -4,     /* K or a pointer violates the alignment the op needs */
+  QUIK_ERR_NULL = -5,      /* required pointer is NULL */
+  QUIK_ERR_RANGE = -6,     /* size beyond what the kernel supports */
+  QUIK_ERR_LAUNCH = -7     /* HIP reported a launch error; hipGetLastError text via quik_last_hip_error() */
+} quik_status;
+
+typedef enum quik_dtype { QUIK_F16 = 0, QUIK_BF16 = 1 } quik_dtype;
+
+const char *quik_status_string(int status);
+const char *quik_last_hip_error(void);
+int quik_abi_version(void);
+
+/* ------------------------------------------------------------------------------------
+ * Column map: the outlier split of one layer in the compact form the quantize kernel
+ * reads.  Built once per layer (or per call by the stateless op) from the int64 index
+ * tensors the reference passes to every call (src/asymmetric/asymmetric.cu:449-453).
+ * Indices outside [0, cols) are clamped into range.
+ * quik_colmap_bytes: size of the workspace, 0 if the arguments are invalid. */
+int64_t quik_colmap_bytes(int64_t cols, int64_t num_int, int64_t num_fp);
+int quik_colmap_build(const int64_t *int_indices, int64_t num_int,
+                      const int64_t *fp_indices, int64_t num_fp, int64_t cols,
+                      void *colmap, void *stream);
+
+/* quik.asymmetric.quantize(src, int_indices, fp_indices, bits) -> (dst, meta, fp_x)
+ * replaces QUIK::asymmetric::quantize, src/asymmetric/asymmetric.cpp:16-25 and
+ * quantizeCUDA, src/asymmetric/asymmetric.cu:492-584.
+ *   x      [rows, cols] dtype, contiguous
+ *   dst    [rows, num_int/2] uint8 (bits=4, low nibble = even element) or [rows, num_int] int8
+ *   meta   [2*rows] dtype, interleaved (scale, zero)
+ *   fp_x   [rows, num_fp] dtype
+ * num_int + num_fp must equal cols and num_int must be even (asymmetric.cu:519-524).
+ * `colmap` comes from quik_colmap_build for the same (cols, num_int, num_fp). */
+int quik_asym_quantize(const void *x, int dtype, int64_t rows, int64_t cols,
+                       const void *colmap, int64_t num_int, int64_t num_fp, int bits,
+                       void *dst, void *meta, void *fp_x, void *stream);
+
+/* quik.asymmetric.find_meta(src, bits) -> meta [2*rows]; fp16 only, all columns.
+ * replaces findMaxMinMetaCUDA, src/asymmetric/asymmetric.cu:320-338. */
+int quik_asym_find_meta(const void *x, int64_t rows, int64_t cols, int bits,
+                        void *meta, void *stream);
+
+/* quik.asymmetric.quantizeOld(src, meta, bits) -> dst; fp16 only, every column.
+ * replaces quantizeCUDAOld, src/asymmetric/asymmetric.cu:68-117.
+ * dst is [rows, ceil(cols/2)] uint8 for bits=4 (flat pairing over the whole array as the
+ * reference kernel does, :25-43) or [rows, cols] int8. */
+int quik_asym_quantize_old(const void *x, const void *meta, int64_t rows, int64_t cols,
+                           int bits, void *dst, void *stream);
+
+/* quik.asymmetric.dequantize(x, meta, scale_col, wReduced, y, bits) -> out
+ * replaces dequantizeCUDA, src/asymmetric/asymmetric.cu:175-233 (kernel :119-173).
+ *   acc [rows, cols] int32; meta [2*rows]; scale_col [cols]; w_reduced [cols];
+ *   y, out [rows, cols] dtype.  fp32 arithmetic, one rounding to dtype. */
+int quik_asym_dequantize(const int32_t *acc, const void *meta, const void *scale_col,
+                         const void *w_reduced, const void *y, int dtype, int64_t rows,
+                         int64_t cols, int bits, void *out, void *stream);
+
+/* quik.symmetric.quantize(src, scale, bits) -> dst; fp16 only.
+ * replaces int4QuantizationCUDA / int8QuantizationCUDA, src/symmetric/symmetric.cu:6-79.
+ *   x [rows, cols] fp16; scale [rows] fp16; dst [rows, ceil(cols/2)] uint8 or [rows, cols] int8.
+ * No clamp: int4 keeps the low four bits, int8 wraps (C conversion). */
+int quik_sym_quantize(const void *x, const void *scale, int64_t rows, int64_t cols,
+                      int bits, void *dst, void *stream);
+
+/* quik.symmetric.dequantize(x, scale_row, scale_col, y, bits) -> out; fp16 chain.
+ * replaces dequantizationCUDA<T>, src/symmetric/symmetric.cu:91-152;
+ * x_bits selects the element type of x: 8 int8, 16 fp16, 32 int32 (symmetric.cpp:32-41). */
+int quik_sym_dequantize(const void *x, int x_bits, const void *scale_row,
+                        const void *scale_col, const void *y, int64_t rows, int64_t cols,
+                        void *out, void *stream);
+
+/* quik.matmul.int4Matmul(A, B) -> C int32 [M, N]
+ * replaces int4MatmulCUDA, src/matmul/matmul.cu:17-55.
+ *   A [M, K/2], B [N, K/2] uint8 nibble-packed, K = number of int4 elements per row.
+ * K % 32 == 0 (the reference's 128-bit operand alignment); K < 131072. */
+int quik_int4_matmul(const uint8_t *A, const uint8_t *B, int32_t *C, int64_t M, int64_t N,
+                     int64_t K, void *stream);
+
+/* quik.matmul.int8Matmul(A, B) -> C int32 [M, N]
+ * replaces int8MatmulCUDA, src/matmul/matmul.cu:98-136.  K % 16 == 0. */
+int quik_int8_matmul(const int8_t *A, const int8_t *B, int32_t *C, int64_t M, int64_t N,
+                     int64_t K, void *stream);
+
+/* One-launch replacement for the tail of MixedQLinear.forward
+ * (experiments/qlinear.py:122-145): outlier GEMM (+bias), integer GEMM and dequantize.
+ *   out[m,n] = dtype( f32(acc[m,n]) * (s_row[m]*s_col[n])
+ *                     + (zero[m] + 2^(bits-1) * s_row[m]) * w_reduced[n]
+ *                     + sum_f fp_x[m,f]*fp_w[n,f] + bias[n] )
+ *   qx      [M, K/2] uint8 (bits=4) or [M, K] int8 (bits=8)     (quantize output)
+ *   qw      [N, K/2] uint8 or [N, K] int8                       (MixedQLinear.int_weight)
+ *   meta    [2*M] dtype (scale, zero) pairs; for the symmetric variant pass
+ *           w_reduced = NULL and meta = per-row scales [M] (no zero-point term)
+ *   s_col   [N] dtype (weights_scales), w_reduced [N] dtype or NULL
+ *   fp_x    [M, F] dtype, fp_w [N, F] dtype, F % 8 == 0 (F may be 0 with NULL pointers)
+ *   bias    [N] dtype or NULL
+ * The integer accumulators are exact; the rest is fp32 with one rounding to dtype. */
+int quik_mixed_linear_fwd(const void *qx, const void *qw, const void *meta,
+                          const void *s_col, const void *w_reduced, const void *fp_x,
+                          const void *fp_w, const void *bias, int dtype, int64_t M,
+                          int64_t N, int64_t K, int64_t F, int bits, void *out,
+                          void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* QUIK_HIP_H_ */

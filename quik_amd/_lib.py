@@ -1,0 +1,98 @@
+"""ctypes binding of libquik_hip.so (declarations: include/quik_hip.h)."""
+from __future__ import annotations
+
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libquik_hip.so")
+
+QUIK_F16, QUIK_BF16 = 0, 1
+
+_vp, _i64, _int = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
+
+# name -> (restype, argtypes); one entry per symbol declared in include/quik_hip.h
+SIGNATURES = {
+    "quik_status_string": (ctypes.c_char_p, [_int]),
+    "quik_last_hip_error": (ctypes.c_char_p, []),
+    "quik_abi_version": (_int, []),
+    "quik_colmap_bytes": (_i64, [_i64, _i64, _i64]),
+    "quik_colmap_build": (_int, [_vp, _i64, _vp, _i64, _i64, _vp, _vp]),
+    "quik_asym_quantize": (_int, [_vp, _int, _i64, _i64, _vp, _i64, _i64, _int, _vp, _vp, _vp, _vp]),
+    "quik_asym_find_meta": (_int, [_vp, _i64, _i64, _int, _vp, _vp]),
+    "quik_asym_quantize_old": (_int, [_vp, _vp, _i64, _i64, _int, _vp, _vp]),
+    "quik_asym_dequantize": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _int, _vp, _vp]),
+    "quik_sym_quantize": (_int, [_vp, _vp, _i64, _i64, _int, _vp, _vp]),
+    "quik_sym_dequantize": (_int, [_vp, _int, _vp, _vp, _vp, _i64, _i64, _vp, _vp]),
+    "quik_int4_matmul": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
+    "quik_int8_matmul": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
+    "quik_mixed_linear_fwd": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _i64, _int,
+                                     _vp, _vp]),
+}
+
+_lib = None
+
+
+def load():
+    """Load the HIP library; there is no fallback when it is missing."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with `make -C quik_amd/csrc` (or __graft_entry__.build()); "
+                "quik_amd has no CPU or PyTorch fallback")
+        lib = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = lib
+    return _lib
+
+
+def check(status: int, op: str):
+    if status != 0:
+        lib = load()
+        msg = lib.quik_status_string(status).decode()
+        if status == -7:
+            msg += ": " + lib.quik_last_hip_error().decode()
+        raise RuntimeError(f"{op}: {msg}")
+
+
+def ptr(t):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def dtype_id(t: torch.Tensor, op: str, allow_bf16: bool) -> int:
+    if t.dtype == torch.float16:
+        return QUIK_F16
+    if t.dtype == torch.bfloat16 and allow_bf16:
+        return QUIK_BF16
+    want = "float16 or bfloat16" if allow_bf16 else "float16"
+    raise RuntimeError(f"{op}: expected a {want} tensor but got {t.dtype}")
+
+
+def check_cuda_contiguous(op: str, **tensors):
+    """The checks the reference's host functions make before launching:
+    torch::checkAllContiguous and torch::checkDeviceType(..., CUDA)."""
+    dev = None
+    for name, t in tensors.items():
+        if not isinstance(t, torch.Tensor):
+            raise TypeError(f"{op}(): argument '{name}' must be a torch.Tensor, not {type(t).__name__}")
+        if not t.is_cuda:
+            raise RuntimeError(f"{op}: expected tensor for argument '{name}' to be on a CUDA (HIP) device, "
+                               f"but it is on {t.device}")
+        if not t.is_contiguous():
+            raise RuntimeError(f"{op}: expected tensor for argument '{name}' to be contiguous")
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            raise RuntimeError(f"{op}: expected all tensors on the same GPU, but '{name}' is on {t.device} "
+                               f"and another argument is on {dev}")
+    return dev

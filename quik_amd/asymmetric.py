@@ -1,0 +1,144 @@
+"""quik.asymmetric: per-token asymmetric quantize / dequantize ops on MI355X.
+
+Same names, argument order and keyword names as the reference's pybind module
+(src/asymmetric/asymmetric.cpp:134-180 of the reference): quantize, dequantize, find_meta,
+quantizeOld.  Every op allocates and returns new tensors on the device of its first argument
+and runs on torch's current stream.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _lib as L
+
+__all__ = ["quantize", "dequantize", "find_meta", "quantizeOld", "build_colmap", "quantize_mapped"]
+
+
+def _check_bits(bits):
+    if bits not in (4, 8):
+        raise RuntimeError("bits argument must be either 4 or 8")
+
+
+def build_colmap(int_indices: torch.Tensor, fp_indices: torch.Tensor, cols: int) -> torch.Tensor:
+    """Compact column map for quantize_mapped (uint8 blob on the indices' device).
+
+    Build it once per layer; it depends only on the two index tensors."""
+    L.check_cuda_contiguous("quantize", int_indices=int_indices, fp_indices=fp_indices)
+    if int_indices.dtype != torch.int64 or fp_indices.dtype != torch.int64:
+        raise RuntimeError("quantize: int_indices and fp_indices must be int64 tensors")
+    lib = L.load()
+    num_int, num_fp = int_indices.numel(), fp_indices.numel()
+    if num_fp + num_int != cols:
+        raise RuntimeError("Quantize: number of fp and int columns is not equal to total number of columns")
+    nbytes = lib.quik_colmap_bytes(cols, num_int, num_fp)
+    with torch.cuda.device(int_indices.device):
+        cm = torch.empty(nbytes, dtype=torch.uint8, device=int_indices.device)
+        L.check(lib.quik_colmap_build(L.ptr(int_indices), num_int, L.ptr(fp_indices) if num_fp else None, num_fp,
+                                      cols, L.ptr(cm), L.stream()), "quantize")
+    return cm
+
+
+def quantize_mapped(src: torch.Tensor, colmap: torch.Tensor, num_int: int, num_fp: int, bits: int):
+    """quantize() with a prebuilt column map: one kernel launch."""
+    _check_bits(bits)
+    L.check_cuda_contiguous("quantize", src=src, colmap=colmap)
+    if src.dim() != 2:
+        raise RuntimeError(f"quantize: expected a 2-D src but got {src.dim()} dimensions")
+    dt = L.dtype_id(src, "quantize", allow_bf16=True)
+    rows, cols = src.shape
+    if num_fp + num_int != cols:
+        raise RuntimeError("Quantize: number of fp and int columns is not equal to total number of columns")
+    if num_int % 2 != 0:
+        raise RuntimeError("Quantize: number of int columns has to be even (implementation detail)")
+    lib = L.load()
+    with torch.cuda.device(src.device):
+        if bits == 4:
+            dst = torch.empty((rows, num_int // 2), dtype=torch.uint8, device=src.device)
+        else:
+            dst = torch.empty((rows, num_int), dtype=torch.int8, device=src.device)
+        meta = torch.empty((2 * rows,), dtype=src.dtype, device=src.device)
+        fp_x = torch.empty((rows, num_fp), dtype=src.dtype, device=src.device)
+        L.check(lib.quik_asym_quantize(L.ptr(src), dt, rows, cols, L.ptr(colmap), num_int, num_fp, bits, L.ptr(dst),
+                                       L.ptr(meta), L.ptr(fp_x), L.stream()), "quantize")
+    return dst, meta, fp_x
+
+
+def quantize(src: torch.Tensor, int_indices: torch.Tensor, fp_indices: torch.Tensor, bits: int):
+    """(dst, meta, fp_x) = quantize(src [M, in], int_indices [K] int64, fp_indices [F] int64, bits).
+
+    dst: uint8 [M, K/2] (bits=4, low nibble = even element) or int8 [M, K]; meta: [2M]
+    interleaved (scale, zero) in src's dtype; fp_x[r, j] = src[r, fp_indices[j]]."""
+    _check_bits(bits)
+    L.check_cuda_contiguous("quantize", src=src)
+    L.check_cuda_contiguous("quantize", int_indices=int_indices)
+    L.check_cuda_contiguous("quantize", fp_indices=fp_indices)
+    if src.dim() != 2:
+        raise RuntimeError(f"quantize: expected a 2-D src but got {src.dim()} dimensions")
+    colmap = build_colmap(int_indices, fp_indices, src.shape[1])
+    return quantize_mapped(src, colmap, int_indices.numel(), fp_indices.numel(), bits)
+
+
+def dequantize(x: torch.Tensor, meta: torch.Tensor, scale_col: torch.Tensor, wReduced: torch.Tensor,
+               y: torch.Tensor, bits: int) -> torch.Tensor:
+    """out = dtype(f32(x) * (s_row * s_col) + ((zero + 2^(bits-1) * s_row) * wReduced + y)).
+
+    x int32 [M, N]; meta [2M]; scale_col with size(0) == N; wReduced with size(1) == N; y [M, N]."""
+    L.check_cuda_contiguous("dequantize", x=x, meta=meta, scale_col=scale_col, y=y)
+    L.check_cuda_contiguous("dequantize", wReduced=wReduced.contiguous())
+    _check_bits(bits)
+    if x.dtype != torch.int32:
+        raise RuntimeError(f"dequantize: expected an int32 x but got {x.dtype}")
+    if x.numel() != y.numel():
+        raise RuntimeError(f"Expected tensor for x to have same number of elements as tensor for y; but "
+                           f"{x.numel()} does not equal {y.numel()} (while checking arguments for dequantize)")
+    rows, cols = x.shape
+    if meta.size(0) != 2 * rows:
+        raise RuntimeError(f"dequantize: expected meta to have size {2 * rows} at dimension 0, got {meta.size(0)}")
+    if scale_col.size(0) != cols:
+        raise RuntimeError(f"dequantize: expected scale_col to have size {cols} at dimension 0, "
+                           f"got {scale_col.size(0)}")
+    if wReduced.dim() < 2 or wReduced.size(1) != cols:
+        raise RuntimeError(f"dequantize: expected wReduced to have size {cols} at dimension 1")
+    dt = L.dtype_id(y, "dequantize", allow_bf16=True)
+    for name, t in (("meta", meta), ("scale_col", scale_col), ("wReduced", wReduced)):
+        if t.dtype != y.dtype:
+            raise RuntimeError(f"dequantize: expected {name} to have dtype {y.dtype} but got {t.dtype}")
+    lib = L.load()
+    with torch.cuda.device(x.device):
+        out = torch.empty_like(y)
+        L.check(lib.quik_asym_dequantize(L.ptr(x), L.ptr(meta), L.ptr(scale_col), L.ptr(wReduced.contiguous()),
+                                         L.ptr(y), dt, rows, cols, bits, L.ptr(out), L.stream()), "dequantize")
+    return out
+
+
+def find_meta(src: torch.Tensor, bits: int) -> torch.Tensor:
+    """meta [2M] fp16: per-row (scale, zero) over all columns of an fp16 src."""
+    L.check_cuda_contiguous("find_meta", src=src)
+    _check_bits(bits)
+    L.dtype_id(src, "find_meta", allow_bf16=False)
+    rows, cols = src.shape
+    lib = L.load()
+    with torch.cuda.device(src.device):
+        meta = torch.empty((2 * rows,), dtype=torch.float16, device=src.device)
+        L.check(lib.quik_asym_find_meta(L.ptr(src), rows, cols, bits, L.ptr(meta), L.stream()), "find_meta")
+    return meta
+
+
+def quantizeOld(src: torch.Tensor, meta: torch.Tensor, bits: int) -> torch.Tensor:
+    """Quantise every column of an fp16 src with given meta [2M]."""
+    L.check_cuda_contiguous("quantize", src=src, meta=meta)
+    _check_bits(bits)
+    L.dtype_id(src, "quantize", allow_bf16=False)
+    L.dtype_id(meta, "quantize", allow_bf16=False)
+    rows, cols = src.shape
+    if meta.size(0) != 2 * rows:
+        raise RuntimeError(f"quantize: expected meta to have size {2 * rows} at dimension 0, got {meta.size(0)}")
+    lib = L.load()
+    with torch.cuda.device(src.device):
+        if bits == 4:
+            dst = torch.empty((rows, (cols + 1) // 2), dtype=torch.uint8, device=src.device)
+        else:
+            dst = torch.empty((rows, cols), dtype=torch.int8, device=src.device)
+        L.check(lib.quik_asym_quantize_old(L.ptr(src), L.ptr(meta), rows, cols, bits, L.ptr(dst), L.stream()),
+                "quantize")
+    return dst

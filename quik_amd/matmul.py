@@ -1,0 +1,85 @@
+"""quik.matmul: exact integer GEMMs on MI355X matrix cores.
+
+Same names and keyword names as the reference's pybind module (src/matmul/matmul.cpp:78-109):
+int4Matmul(A, B), int8Matmul(A, B) -> int32 [M, N] = A @ B^T.  The 2:4-sparse and cuSPARSELt
+entry points of the reference are NVIDIA sparse-tensor-core formats and are not provided.
+mixed_linear is the one-launch fused tail of MixedQLinear.forward (no reference counterpart
+as a separate op; it computes what experiments/qlinear.py:122-145 computes in three ops).
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _lib as L
+
+__all__ = ["int4Matmul", "int8Matmul", "mixed_linear"]
+
+
+def _matmul(op, A, B, want_dtype, sym, kmul):
+    L.check_cuda_contiguous(op, A=A, B=B)
+    if A.dtype != want_dtype or B.dtype != want_dtype:
+        raise RuntimeError(f"{op}: expected {want_dtype} operands but got {A.dtype} and {B.dtype}")
+    if A.dim() != 2 or B.dim() != 2 or A.size(1) != B.size(1):
+        raise RuntimeError(f"{op}: A [M, K] and B [N, K] must agree in K, got {tuple(A.shape)} and {tuple(B.shape)}")
+    M, N, K = A.size(0), B.size(0), A.size(1) * kmul
+    lib = L.load()
+    with torch.cuda.device(A.device):
+        C = torch.empty((M, N), dtype=torch.int32, device=A.device)
+        L.check(getattr(lib, sym)(L.ptr(A), L.ptr(B), L.ptr(C), M, N, K, L.stream()), op)
+    return C
+
+
+def int4Matmul(A: torch.Tensor, B: torch.Tensor) -> torch.Tensor:
+    """A uint8 [M, K/2], B uint8 [N, K/2], nibble-packed int4 (low nibble = even element)."""
+    return _matmul("int4Matmul", A, B, torch.uint8, "quik_int4_matmul", 2)
+
+
+def int8Matmul(A: torch.Tensor, B: torch.Tensor) -> torch.Tensor:
+    """A int8 [M, K], B int8 [N, K]."""
+    return _matmul("int8Matmul", A, B, torch.int8, "quik_int8_matmul", 1)
+
+
+def mixed_linear(qx, int_weight, meta, weights_scales, reduced_w, fp_x, fp_weight, bias, bits, out_dtype):
+    """Fused outlier GEMM + integer GEMM + dequantize: returns [M, N] in out_dtype.
+
+    reduced_w=None selects the symmetric form (meta = per-row scales, no zero-point term)."""
+    if bits not in (4, 8):
+        raise RuntimeError("bits argument must be either 4 or 8")
+    tensors = dict(qx=qx, int_weight=int_weight, meta=meta, weights_scales=weights_scales)
+    for name, t in (("reduced_w", reduced_w), ("fp_x", fp_x), ("fp_weight", fp_weight), ("bias", bias)):
+        if t is not None and t.numel() > 0:
+            tensors[name] = t
+    L.check_cuda_contiguous("mixed_linear", **tensors)
+    want = torch.uint8 if bits == 4 else torch.int8
+    if qx.dtype != want or int_weight.dtype != want:
+        raise RuntimeError(f"mixed_linear: bits={bits} expects {want} operands")
+    if out_dtype == torch.float16:
+        dt = L.QUIK_F16
+    elif out_dtype == torch.bfloat16:
+        dt = L.QUIK_BF16
+    else:
+        raise RuntimeError(f"mixed_linear: unsupported dtype {out_dtype}")
+    for name, t in tensors.items():
+        if name not in ("qx", "int_weight") and t.dtype != out_dtype:
+            raise RuntimeError(f"mixed_linear: expected {name} of dtype {out_dtype} but got {t.dtype}")
+    M, N = qx.size(0), int_weight.size(0)
+    if qx.size(1) != int_weight.size(1):
+        raise RuntimeError("mixed_linear: qx and int_weight disagree in K")
+    K = qx.size(1) * (2 if bits == 4 else 1)
+    F = 0 if "fp_x" not in tensors else fp_x.size(1)
+    if F and (fp_weight.size(0) != N or fp_weight.size(1) != F or fp_x.size(0) != M):
+        raise RuntimeError("mixed_linear: fp_x [M, F] and fp_weight [N, F] sizes are inconsistent")
+    if meta.numel() != (2 * M if reduced_w is not None else M) or weights_scales.numel() != N:
+        raise RuntimeError("mixed_linear: meta / weights_scales sizes are inconsistent with M, N")
+    if reduced_w is not None and reduced_w.numel() != N:
+        raise RuntimeError("mixed_linear: reduced_w must have N elements")
+    if "bias" in tensors and bias.numel() != N:
+        raise RuntimeError("mixed_linear: bias must have N elements")
+    lib = L.load()
+    with torch.cuda.device(qx.device):
+        out = torch.empty((M, N), dtype=out_dtype, device=qx.device)
+        L.check(lib.quik_mixed_linear_fwd(L.ptr(qx), L.ptr(int_weight), L.ptr(meta), L.ptr(weights_scales),
+                                          L.ptr(reduced_w), L.ptr(fp_x) if F else None,
+                                          L.ptr(fp_weight) if F else None, L.ptr(tensors.get("bias")), dt, M, N, K,
+                                          F, bits, L.ptr(out), L.stream()), "mixed_linear")
+    return out

@@ -1,0 +1,246 @@
+"""MixedQLinear for MI355X: the module interface of the reference's experiments/qlinear.py.
+
+Same constructor, buffers, `from_float` signature and `SharedQuantizedInput` protocol as the
+reference (experiments/qlinear.py:21-199), so `llama_replace_with_kernels`
+(experiments/llama.py:394-440) can use it unchanged.  Differences, all deliberate:
+
+* forward runs two launches by default: one quantize kernel (cached column map) and one fused
+  GEMM kernel (integer GEMM + outlier GEMM + dequantize).  `fused=False` replays the
+  reference's op sequence (F.linear, int GEMM, dequantize) with the stand-alone ops.
+* a 3-D input (B, S, in) is flattened to (B*S, in) and the result has shape (B, S, N); the
+  reference keeps only batch element 0 (qlinear.py:89-90) and returns (1, S, N), which is
+  the same thing for B == 1.
+* the symmetric branch works: the reference calls the symmetric ops without their `bits`
+  argument and hands a [N, 1] scale where [1, N] is checked (qlinear.py:103,142), so it raises
+  at HEAD.  Its activation scale divisor `1 << (bits - 1) - 1` parses as 1 << ((bits-1)-1)
+  = 4 for bits=4; that value is kept (`sym_divisor`) so codes match what the expression says.
+"""
+from __future__ import annotations
+
+import torch
+from torch import Tensor
+
+from . import asymmetric, matmul, symmetric
+
+__all__ = ["MixedQLinear", "SharedQuantizedInput", "Linear4bit", "Linear8bit", "pack_to_i4", "two_compl"]
+
+
+def two_compl(x: Tensor, bits: int) -> Tensor:
+    return torch.where(x < 0, 2 ** bits + x, x)
+
+
+def pack_to_i4(X: Tensor) -> Tensor:
+    """Signed int4 codes [R, K] (K even) -> uint8 [R, K/2], even element in the low nibble."""
+    u = two_compl(X.to(dtype=torch.int8), 4).to(torch.uint8)
+    return u[:, 0::2] | (u[:, 1::2] << 4)
+
+
+class SharedQuantizedInput:
+    """Quantized activation shared by the layers of one group (q/k/v, gate/up): the first
+    member quantizes, the others reuse, the last one clears (qlinear.py:21-37)."""
+
+    def __init__(self, group_size):
+        self.qint_x = None
+        self.fp_x = None
+        self.qscale_x = None
+        self.meta = None
+        self.group_size = group_size
+        self.cur_group_elem = 0
+
+    def finish(self):
+        self.cur_group_elem += 1
+        if self.cur_group_elem == self.group_size:
+            self.qint_x = None
+            self.qscale_x = None
+            self.meta = None
+            self.fp_x = None
+            self.cur_group_elem = 0
+
+
+class MixedQLinear(torch.nn.Module):
+    def __init__(self, in_features, out_features, shared_input=None,
+                 fp_features_num=0, symm=False, bits=4, dtype=torch.float16, fused=True):
+        super().__init__()
+        self.fp_features_num = fp_features_num
+        self.int_features_num = in_features - fp_features_num
+        self.in_features = in_features
+        self.out_features = out_features
+        self.symmetric = symm
+        self.bits = bits
+        self.shared_input = shared_input
+        self.dtype = dtype
+        self.fused = fused
+        self.sym_divisor = 1 << ((bits - 1) - 1)
+        self.register_buffer('weights_scales', torch.zeros((out_features, 1), dtype=dtype))
+        if bits == 4:
+            self.register_buffer('int_weight', torch.zeros((out_features, self.int_features_num // 2),
+                                                           dtype=torch.uint8))
+        else:
+            self.register_buffer('int_weight', torch.zeros((out_features, self.int_features_num), dtype=torch.int8))
+        self.register_buffer('bias', torch.zeros((out_features,), dtype=dtype))
+        self.register_buffer('int_indices', torch.zeros((self.int_features_num,), dtype=torch.long))
+        self.register_buffer('fp_indices', torch.zeros((fp_features_num,), dtype=torch.long))
+        if fp_features_num > 0:
+            self.register_buffer('fp_weight', torch.zeros((out_features, fp_features_num), dtype=dtype))
+        if not symm:
+            self.register_buffer('reduced_w', torch.zeros((1, out_features), dtype=dtype))
+        self._colmap = None
+        self._colmap_key = None
+
+    # -- cached column map: rebuilt when the index buffers move or are written in place
+    def _column_map(self):
+        key = (self.int_indices.data_ptr(), self.fp_indices.data_ptr(), self.int_indices._version,
+               self.fp_indices._version, self.int_indices.device)
+        if self._colmap is None or self._colmap_key != key:
+            self._colmap = asymmetric.build_colmap(self.int_indices, self.fp_indices, self.in_features)
+            self._colmap_key = key
+        return self._colmap
+
+    def _quantize_input(self, x, shared_input):
+        if self.symmetric:
+            if self.fp_features_num > 0:
+                int_x = x[:, self.int_indices].contiguous()
+                shared_input.fp_x = x[:, self.fp_indices].contiguous()
+            else:
+                int_x = x
+                shared_input.fp_x = None
+            shared_input.qscale_x = (torch.max(torch.abs(int_x), dim=1)[0].unsqueeze(1) /
+                                     self.sym_divisor).to(torch.float16)
+            shared_input.qint_x = symmetric.quantize(int_x, shared_input.qscale_x, self.bits)
+        else:
+            shared_input.qint_x, shared_input.meta, shared_input.fp_x = asymmetric.quantize_mapped(
+                x, self._column_map(), self.int_features_num, self.fp_features_num, self.bits)
+
+    def forward(self, x):
+        if self.int_features_num <= 0:
+            return torch.nn.functional.linear(x, self.fp_weight, self.bias)
+        if not x.is_cuda:
+            raise RuntimeError("MixedQLinear.forward needs a tensor on the GPU; there is no CPU path")
+        lead = x.shape[:-1] if x.dim() == 3 else (1, x.shape[0])
+        x2 = x.reshape(-1, x.shape[-1])
+        if not x2.is_contiguous():
+            x2 = x2.contiguous()
+        shared_input = self.shared_input if self.shared_input is not None else SharedQuantizedInput(1)
+        with torch.cuda.device(x.device):
+            if shared_input.qint_x is None:
+                self._quantize_input(x2, shared_input)
+            if self.fused:
+                output = matmul.mixed_linear(
+                    shared_input.qint_x, self.int_weight,
+                    shared_input.qscale_x if self.symmetric else shared_input.meta,
+                    self.weights_scales, None if self.symmetric else self.reduced_w,
+                    shared_input.fp_x if self.fp_features_num > 0 else None,
+                    self.fp_weight if self.fp_features_num > 0 else None,
+                    self.bias, self.bits, self.dtype)
+            else:
+                output = self._forward_unfused(shared_input)
+        shared_input.finish()
+        return output.reshape(*lead, self.out_features)
+
+    def _forward_unfused(self, shared_input):
+        """The reference's op sequence (qlinear.py:122-145)."""
+        rows = shared_input.qint_x.shape[0]
+        if self.fp_features_num > 0:
+            fp_result = torch.nn.functional.linear(shared_input.fp_x, self.fp_weight, self.bias)
+        elif self.bias is not None:
+            fp_result = self.bias.repeat(rows, 1)
+        else:
+            fp_result = torch.zeros((rows, self.out_features), dtype=self.dtype, device=self.int_weight.device)
+        if self.bits == 4:
+            int_result = matmul.int4Matmul(shared_input.qint_x, self.int_weight)
+        else:
+            int_result = matmul.int8Matmul(shared_input.qint_x, self.int_weight)
+        if self.symmetric:
+            return symmetric.dequantize(int_result, shared_input.qscale_x,
+                                        self.weights_scales.reshape(1, -1).contiguous(), fp_result.contiguous(), 32)
+        return asymmetric.dequantize(int_result, shared_input.meta, self.weights_scales, self.reduced_w,
+                                     fp_result.contiguous(), self.bits)
+
+    @staticmethod
+    def from_float(module: torch.nn.Linear, weight_matrix, weights_scales, shared_input=None,
+                   fp_indices=None, symm=False, bits=4, fused=True):
+        """Build a MixedQLinear from a float Linear (qlinear.py:150-199).
+
+        `weight_matrix` [out, in] holds the fake-quantized weights (codes * scale on the int
+        columns), `weights_scales` [out, 1] the per-output-channel scales, `fp_indices` the
+        outlier input columns.  Integer columns are the ascending complement of fp_indices."""
+        assert weights_scales.shape == (module.out_features, 1), 'weights_scales should have shape (out_features, 1)'
+        assert weight_matrix.shape == (module.out_features, module.in_features)
+        assert (symm and bits == 4) or not symm, "Symmetric quantization with 8 bits is not supported"
+        int_indices = torch.arange(module.in_features)
+        if fp_indices is None or len(fp_indices) == 0:
+            fp_indices = torch.tensor([], dtype=int_indices.dtype)
+        else:
+            fp_indices = fp_indices.to(device='cpu', dtype=int_indices.dtype)
+            int_indices = int_indices[~torch.isin(int_indices, fp_indices)]
+        assert torch.numel(int_indices) + torch.numel(fp_indices) == module.in_features, \
+            'There are some duplication in the fp_indices!'
+
+        mod = MixedQLinear(module.in_features, module.out_features, shared_input,
+                           fp_features_num=torch.numel(fp_indices), symm=symm, bits=bits,
+                           dtype=weight_matrix.dtype, fused=fused)
+        if torch.cuda.is_available():
+            weight_matrix = weight_matrix.cuda()
+        dev = weight_matrix.device
+        mod.weights_scales.copy_(weights_scales.to(weight_matrix.dtype))
+        w_int = weight_matrix[:, int_indices.to(dev)]
+        rounded = (w_int / weights_scales.to(dev)).round()
+        if bits == 4:
+            mod.int_weight.copy_(pack_to_i4(rounded.to(torch.int8)).cpu())
+        else:
+            mod.int_weight.copy_(rounded.to(torch.int8).cpu())
+        if not symm:
+            reduced_w = torch.sum(w_int.float(), dim=1, keepdim=True).to(weight_matrix.dtype)
+            mod.reduced_w.copy_(reduced_w.t().cpu())
+        if module.bias is not None:
+            mod.bias.copy_(module.bias)
+        else:
+            mod.bias = None
+        mod.int_indices.copy_(int_indices)
+        mod.fp_indices.copy_(fp_indices)
+        if mod.fp_features_num > 0:
+            mod.fp_weight.copy_(weight_matrix[:, fp_indices.to(dev)].to(weight_matrix.dtype))
+        return mod
+
+
+class Linear8bit(torch.nn.Module):
+    """Plain int8 GEMM layer of the reference's benchmark scaffolding (qlinear.py:202-228)."""
+
+    def __init__(self, in_features, out_features, bias=None):
+        super().__init__()
+        self.in_features = in_features
+        self.out_features = out_features
+        self.register_buffer('int_weight', torch.zeros((out_features, in_features), dtype=torch.int8))
+        self.register_buffer('bias', torch.zeros((out_features,), dtype=torch.float16))
+        if bias is not None:
+            self.bias.copy_(bias)
+        else:
+            self.bias = None
+
+    def forward(self, x):
+        if x.dim() == 3:
+            x = x[0]
+        out = matmul.int8Matmul(x.to(torch.int8).contiguous(), self.int_weight).to(torch.float16)
+        return out if self.bias is None else out.add(self.bias)
+
+
+class Linear4bit(torch.nn.Module):
+    """Plain int4 GEMM layer of the reference's benchmark scaffolding (qlinear.py:231-256)."""
+
+    def __init__(self, in_features, out_features, bias=None):
+        super().__init__()
+        self.in_features = in_features
+        self.out_features = out_features
+        self.register_buffer('int_weight', torch.zeros((out_features, in_features // 2), dtype=torch.uint8))
+        self.register_buffer('bias', torch.zeros((out_features,), dtype=torch.float16))
+        if bias is not None:
+            self.bias.copy_(bias)
+        else:
+            self.bias = None
+
+    def forward(self, x):
+        if x.dim() == 3:
+            x = x[0]
+        x_int4 = x[:, :x.size(1) // 2].to(torch.uint8).contiguous()
+        out = matmul.int4Matmul(x_int4, self.int_weight).to(torch.float16)
+        return out if self.bias is None else out.add(self.bias)

@@ -1,0 +1,65 @@
+"""quik.symmetric: symmetric quantize / dequantize ops on MI355X.
+
+Same names and keyword names as the reference's pybind module
+(src/symmetric/symmetric.cpp:108-136).  The reference's own caller omits `bits`
+(experiments/qlinear.py:103,142) although the binding requires it; here `bits` defaults to
+the value that caller means (4 for quantize, 32 for dequantize), so both spellings work.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _lib as L
+
+__all__ = ["quantize", "dequantize"]
+
+
+def quantize(src: torch.Tensor, scale: torch.Tensor, bits: int = 4) -> torch.Tensor:
+    """q = rne_int(fp16(src / scale[row])); uint8 [M, ceil(K/2)] nibbles (bits=4, low four bits
+    kept, no clamp) or int8 [M, K] (bits=8, wraps)."""
+    L.check_cuda_contiguous("quantize", src=src, scale=scale)
+    if bits not in (4, 8):
+        raise RuntimeError("Unsupported data type")
+    L.dtype_id(src, "quantize", allow_bf16=False)
+    L.dtype_id(scale, "quantize", allow_bf16=False)
+    rows, cols = src.shape
+    if scale.size(0) != rows:
+        raise RuntimeError(f"quantize: expected scale to have size {rows} at dimension 0, got {scale.size(0)}")
+    lib = L.load()
+    with torch.cuda.device(src.device):
+        if bits == 4:
+            dst = torch.empty((rows, (cols + 1) // 2), dtype=torch.uint8, device=src.device)
+        else:
+            dst = torch.empty((rows, cols), dtype=torch.int8, device=src.device)
+        L.check(lib.quik_sym_quantize(L.ptr(src), L.ptr(scale), rows, cols, bits, L.ptr(dst), L.stream()), "quantize")
+    return dst
+
+
+_X_DTYPE = {8: torch.int8, 16: torch.float16, 32: torch.int32}
+
+
+def dequantize(x: torch.Tensor, scale_row: torch.Tensor, scale_col: torch.Tensor, y: torch.Tensor,
+               bits: int = 32) -> torch.Tensor:
+    """out = fp16(fp16(fp16(fp16(x) * scale_row) * scale_col) + y); `bits` names x's type:
+    8 int8, 16 float16, 32 int32.  scale_row has size(0) == M and scale_col size(1) == N."""
+    L.check_cuda_contiguous("dequantize", x=x, scale_row=scale_row, scale_col=scale_col, y=y)
+    if bits not in _X_DTYPE:
+        raise RuntimeError("Unsupported data type")
+    if x.dtype != _X_DTYPE[bits]:
+        raise RuntimeError(f"dequantize: bits={bits} expects x of dtype {_X_DTYPE[bits]} but got {x.dtype}")
+    if x.shape != y.shape:
+        raise RuntimeError(f"dequantize: expected x and y to have the same size, got {tuple(x.shape)} and "
+                           f"{tuple(y.shape)}")
+    rows, cols = x.shape
+    if scale_row.size(0) != rows:
+        raise RuntimeError(f"dequantize: expected scale_row to have size {rows} at dimension 0")
+    if scale_col.dim() < 2 or scale_col.size(1) != cols:
+        raise RuntimeError(f"dequantize: expected scale_col to have size {cols} at dimension 1")
+    for name, t in (("scale_row", scale_row), ("scale_col", scale_col), ("y", y)):
+        L.dtype_id(t, "dequantize", allow_bf16=False)
+    lib = L.load()
+    with torch.cuda.device(x.device):
+        out = torch.empty_like(y)
+        L.check(lib.quik_sym_dequantize(L.ptr(x), bits, L.ptr(scale_row), L.ptr(scale_col), L.ptr(y), rows, cols,
+                                        L.ptr(out), L.stream()), "dequantize")
+    return out

@@ -1,0 +1,130 @@
+"""CPU-side checks of the boundary: the library loads, exports every symbol that
+include/quik_hip.h declares, rejects bad arguments before touching the GPU, and the Python
+surface has the reference's names and keyword arguments.  No kernel is launched here."""
+import ctypes
+import inspect
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "quik_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(quik_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from quik_amd import _lib as L
+    lib = L.load()
+    names = _declared_symbols()
+    assert len(names) >= 14
+    for n in names:
+        assert hasattr(lib, n), n
+    assert sorted(L.SIGNATURES) == names
+    assert lib.quik_abi_version() == 1
+    assert lib.quik_status_string(-1) == b"bits argument must be either 4 or 8"
+
+
+def test_argument_validation_without_gpu():
+    """Every entry point validates before launching; these calls return before any HIP call."""
+    from quik_amd import _lib as L
+    lib = L.load()
+    null = ctypes.c_void_p(None)
+    one = ctypes.c_void_p(16)  # never dereferenced: validation fails first
+    assert lib.quik_colmap_bytes(8192, 7936, 256) > 0
+    assert lib.quik_colmap_bytes(8192, 7936, 255) == 0
+    # idx16 layout: 7936*2 + 256*2 + 8192/8 bytes, sections 16-byte aligned
+    assert lib.quik_colmap_bytes(8192, 7936, 256) == 7936 * 2 + 512 + 1024
+    assert lib.quik_colmap_bytes(70000, 69000, 1000) == 69000 * 4 + 4000 + ((70000 + 31) // 32 * 4 + 15) // 16 * 16
+    assert lib.quik_asym_quantize(one, 0, 4, 64, one, 62, 2, 5, one, one, one, null) == -1
+    assert lib.quik_asym_quantize(one, 0, 4, 64, one, 60, 2, 4, one, one, one, null) == -2
+    assert lib.quik_asym_quantize(one, 0, 4, 64, one, 61, 3, 4, one, one, one, null) == -4
+    assert lib.quik_asym_quantize(one, 7, 4, 64, one, 62, 2, 4, one, one, one, null) == -3
+    assert lib.quik_asym_quantize(null, 0, 4, 64, one, 62, 2, 4, one, one, one, null) == -5
+    assert lib.quik_asym_quantize(one, 0, 0, 64, one, 62, 2, 4, one, one, one, null) == 0     # empty batch
+    assert lib.quik_int4_matmul(one, one, one, 4, 4, 48, null) == -4      # K % 32
+    assert lib.quik_int4_matmul(one, one, one, 4, 4, 131072, null) == -6  # accumulator headroom
+    assert lib.quik_int8_matmul(one, one, one, 4, 4, 24, null) == -4      # K % 16
+    assert lib.quik_int8_matmul(null, one, one, 4, 4, 32, null) == -5
+    assert lib.quik_int4_matmul(one, one, one, 0, 4, 32, null) == 0
+    assert lib.quik_asym_dequantize(one, one, one, one, one, 0, 4, 4, 3, one, null) == -1
+    assert lib.quik_sym_dequantize(one, 4, one, one, one, 4, 4, one, null) == -1
+    assert lib.quik_sym_quantize(one, one, 4, 4, 16, one, null) == -1
+    assert lib.quik_mixed_linear_fwd(one, one, one, one, one, one, one, null, 0, 4, 4, 32, 12, 4, one, null) == -4
+    assert lib.quik_mixed_linear_fwd(one, one, null, one, one, one, one, null, 0, 4, 4, 32, 8, 4, one, null) == -5
+
+
+def test_python_surface_matches_reference_names():
+    """Names and keyword arguments of the pybind module (src/asymmetric/asymmetric.cpp:144-180,
+    src/symmetric/symmetric.cpp:120-136, src/matmul/matmul.cpp:85,109 of the reference)."""
+    import quik
+    from quik._C import asymmetric, matmul, symmetric
+    assert quik.__all__ == ['matmul', 'symmetric', 'asymmetric']
+    sig = lambda f: list(inspect.signature(f).parameters)
+    assert sig(asymmetric.quantize) == ["src", "int_indices", "fp_indices", "bits"]
+    assert sig(asymmetric.dequantize) == ["x", "meta", "scale_col", "wReduced", "y", "bits"]
+    assert sig(asymmetric.find_meta) == ["src", "bits"]
+    assert sig(asymmetric.quantizeOld) == ["src", "meta", "bits"]
+    assert sig(symmetric.quantize) == ["src", "scale", "bits"]
+    assert sig(symmetric.dequantize) == ["x", "scale_row", "scale_col", "y", "bits"]
+    assert sig(matmul.int4Matmul) == ["A", "B"] and sig(matmul.int8Matmul) == ["A", "B"]
+    from quik_amd import qlinear
+    assert sig(qlinear.MixedQLinear.from_float)[:7] == ["module", "weight_matrix", "weights_scales", "shared_input",
+                                                         "fp_indices", "symm", "bits"]
+    assert sig(qlinear.MixedQLinear.__init__)[1:8] == ["in_features", "out_features", "shared_input",
+                                                        "fp_features_num", "symm", "bits", "dtype"]
+
+
+def test_ops_reject_cpu_tensors_and_bad_bits():
+    import torch
+
+    import quik
+    x = torch.zeros(4, 64, dtype=torch.float16)
+    ii, fi = torch.arange(62), torch.tensor([62, 63])
+    with pytest.raises(RuntimeError, match="CUDA"):
+        quik.asymmetric.quantize(x, ii, fi, 4)
+    with pytest.raises(RuntimeError, match="either 4 or 8"):
+        quik.asymmetric.quantize(x, ii, fi, 3)
+    with pytest.raises(RuntimeError, match="CUDA"):
+        quik.matmul.int4Matmul(torch.zeros(4, 16, dtype=torch.uint8), torch.zeros(4, 16, dtype=torch.uint8))
+    with pytest.raises(RuntimeError, match="CUDA"):   # device check precedes the bits switch, as in the reference
+        quik.symmetric.quantize(x, x[:, :1].contiguous(), 16)
+
+
+def test_from_float_buffers_on_cpu():
+    """from_float's packing is host/torch work and must match the oracle without a GPU."""
+    import numpy as np
+    import torch
+
+    from oracle import quik_oracle as qo
+    from quik_amd.qlinear import MixedQLinear, SharedQuantizedInput, pack_to_i4
+    rng = np.random.default_rng(0)
+    N, n_in, F = 48, 256, 32
+    fi = rng.permutation(n_in)[:F].astype(np.int64)
+    mask = np.ones(n_in, bool)
+    mask[fi] = False
+    ii = np.arange(n_in)[mask]
+    for bits in (4, 8):
+        lo, hi = (-8, 8) if bits == 4 else (-127, 128)
+        codes = rng.integers(lo, hi, (N, n_in - F))
+        s_w = rng.uniform(0.001, 0.01, (N, 1)).astype(np.float16)
+        W = np.zeros((N, n_in), np.float16)
+        W[:, ii] = (codes * s_w.astype(np.float32)).astype(np.float16)
+        W[:, fi] = (0.02 * rng.standard_normal((N, F))).astype(np.float16)
+        lin = torch.nn.Linear(n_in, N, bias=False)
+        mod = MixedQLinear.from_float(lin, torch.from_numpy(W), torch.from_numpy(s_w), SharedQuantizedInput(1),
+                                      torch.from_numpy(fi), bits=bits)
+        o = qo.from_float(W, s_w, fi, bits)
+        assert np.array_equal(mod.int_weight.numpy(), o["int_weight"])
+        assert np.array_equal(mod.reduced_w.numpy(), o["reduced_w"])
+        assert np.array_equal(mod.fp_weight.numpy(), o["fp_weight"])
+        assert np.array_equal(mod.int_indices.numpy(), o["int_indices"]) and mod.bias is None
+        assert set(mod.state_dict()) == {"weights_scales", "int_weight", "int_indices", "fp_indices", "fp_weight",
+                                         "reduced_w"}
+    assert pack_to_i4(torch.tensor([[-8, 7]])).tolist() == [[0x78]]
+    with pytest.raises(AssertionError, match="duplication"):
+        MixedQLinear.from_float(lin, torch.from_numpy(W), torch.from_numpy(s_w), None, torch.tensor([1, 1]), bits=4)

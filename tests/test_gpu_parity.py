@@ -1,0 +1,551 @@
+"""GPU parity: every op of the C ABI (through the quik Python surface) against the CPU oracle.
+
+Bar: integer codes, packed bytes, metadata and int32 accumulators are bit-exact; fp16/bf16
+outputs of the stand-alone dequantize ops are bit-exact against the oracle's association
+order and within 1 output ulp of a float64 evaluation; the fused forward is within
+1e-2 x output RMS (max abs) of the oracle, the tolerance the task states, and in practice
+within a few output ulps.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import quik_oracle as qo
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _lib():
+    from quik_amd import _lib as L
+    L.load()
+    assert torch.cuda.is_available()
+    yield
+
+
+def _t(a, dtype=None):
+    t = torch.from_numpy(np.ascontiguousarray(a))
+    return t.to(DEV) if dtype is None else t.to(DEV, dtype)
+
+
+def _bf16_t(a32):
+    """float32 numpy array holding bf16-representable values -> bf16 tensor on the GPU."""
+    return torch.from_numpy(np.ascontiguousarray(a32, np.float32)).to(torch.bfloat16).to(DEV)
+
+
+def _bits(t):
+    return t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
+
+
+def _split(rng, n_in, F, shuffle=False):
+    fp_idx = rng.permutation(n_in)[:F].astype(np.int64)
+    mask = np.ones(n_in, bool)
+    mask[fp_idx] = False
+    ii = np.arange(n_in, dtype=np.int64)[mask]
+    if shuffle:
+        ii = rng.permutation(ii)
+    return ii, fp_idx
+
+
+def _acts(rng, M, n_in, fp_idx, kind="x50"):
+    x = rng.standard_normal((M, n_in)).astype(np.float32)
+    if kind == "x50":
+        x[:, fp_idx] *= 50
+    elif kind == "student":
+        x[:, fp_idx] = np.clip(20 * rng.standard_t(3, (M, len(fp_idx))), -6e4, 6e4)
+    elif kind == "uniform":
+        x = rng.random((M, n_in)).astype(np.float32)
+    return x
+
+
+def _edge_rows(x, ii):
+    """Overwrite the first rows with edge cases (needs M >= 8, K >= 16)."""
+    x[0, :] = 1.5                                   # constant row: scale clamps at 1e-6
+    x[1, ii[:8]] = [0, 0.5, 1.5, 2.5, 3.5, 4.5, 15, 7.5]
+    x[2, :] *= 1e-7                                 # fp16 subnormals
+    x[3, ii[3]] = 65504.0
+    x[3, ii[4]] = -65504.0                          # range overflows fp16
+    x[4, ii[5]] = np.inf
+    x[5, ii[6]] = np.nan
+    x[6, :] = 0.0
+    x[7, ii] = np.nan                               # all-NaN row
+    return x
+
+
+# ------------------------------------------------------------------------------ asym quantize
+QCASES = [
+    # M, in, F, kind, shuffle
+    (33, 512, 32, "x50", False),
+    (9, 4096, 128, "student", False),
+    (64, 1024, 0, "x50", False),
+    (17, 100, 10, "x50", True),        # row length not a multiple of 8: scalar load path
+    (40, 384, 32, "uniform", True),    # int_indices in arbitrary order
+    (12, 2050, 2, "x50", False),
+]
+
+
+@pytest.mark.parametrize("case", QCASES)
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("bf16", [False, True])
+def test_asym_quantize_bit_exact(case, bits, bf16):
+    import quik
+    M, n_in, F, kind, shuffle = case
+    rng = np.random.default_rng(hash((M, n_in, F, bits, bf16)) % 2 ** 31)
+    ii, fi = _split(rng, n_in, F, shuffle)
+    x32 = _edge_rows(_acts(rng, M, n_in, fi, kind), ii)
+    if bf16:
+        xs = qo.bf16_round(x32)
+        xt = _bf16_t(xs)
+        dst, meta, fp_x = qo.asym_quantize(xs, ii, fi, bits, qo.BF16)
+        meta_b, fp_b = qo.f32_to_bf16_bits(meta), qo.f32_to_bf16_bits(fp_x)
+    else:
+        with np.errstate(over="ignore"):
+            xs = x32.astype(np.float16)
+        xt = _t(xs)
+        dst, meta, fp_x = qo.asym_quantize(xs, ii, fi, bits, qo.F16)
+        meta_b, fp_b = meta.view(np.uint16), fp_x.view(np.uint16)
+    q, m, f = quik.asymmetric.quantize(xt, _t(ii), _t(fi), bits)
+    assert q.dtype == (torch.uint8 if bits == 4 else torch.int8)
+    assert m.shape == (2 * M,) and f.shape == (M, F) and m.dtype == xt.dtype
+    got_m = _bits(m)
+    # scale bit-exact; zero bit-exact except that -0/+0 and NaN payloads are not distinguished
+    want_f = np.asarray(meta, np.float32)
+    got_f = m.float().cpu().numpy()
+    assert np.array_equal(got_m[0::2], meta_b[0::2])
+    assert np.array_equal(np.nan_to_num(got_f[1::2], nan=12345.0), np.nan_to_num(want_f[1::2], nan=12345.0))
+    assert np.array_equal(q.cpu().numpy(), dst)
+    assert np.array_equal(_bits(f), fp_b)
+
+
+def test_asym_quantize_config1_shape_and_reference_invariants():
+    """BASELINE config 1 shape (512 x 4096, 128 outliers x50) plus the reference's own checks
+    (test/python/test_quant.py:24-39): indexed quantize == find_meta + quantizeOld on the gathered
+    columns, fp_x == x[:, fp_indices]."""
+    import quik
+    g = torch.Generator().manual_seed(0)
+    M, n_in, F = 512, 4096, 128
+    x = torch.randn(M, n_in, generator=g)
+    fi = torch.randperm(n_in, generator=g)[:F]
+    x[:, fi] *= 50
+    x = x.half()
+    ii = torch.arange(n_in)
+    ii = ii[~torch.isin(ii, fi)]
+    xd = x.to(DEV)
+    for bits in (4, 8):
+        q, meta, fp = quik.asymmetric.quantize(xd, ii.to(DEV), fi.to(DEV), bits)
+        int_t = xd[:, ii.to(DEV)].contiguous()
+        meta_base = quik.asymmetric.find_meta(int_t, bits)
+        q_base = quik.asymmetric.quantizeOld(int_t, meta_base, bits)
+        assert torch.equal(meta, meta_base) and torch.equal(q, q_base)
+        assert torch.equal(fp, xd[:, fi.to(DEV)])
+        dst, m, f = qo.asym_quantize(x.numpy(), ii.numpy(), fi.numpy(), bits)
+        assert np.array_equal(q.cpu().numpy(), dst)
+        assert np.array_equal(_bits(meta), m.view(np.uint16))
+
+
+def test_quotient_exhaustive_numerators():
+    """Every non-negative fp16 numerator (finite, inf, NaN) against 300 scales, through
+    quantizeOld with zero = 0: pins storage(d / scale) -> rne -> clamp for the whole domain."""
+    import quik
+    num = np.arange(0, 0x8000, dtype=np.uint16).view(np.float16)       # 0 .. +inf .. NaN
+    rng = np.random.default_rng(11)
+    scales = np.concatenate([
+        np.array([1.0133e-6, 6e-8, 1.0, 0.5, 3.0, 65504.0, 4368.0, 0.1, 1 / 3], np.float32),
+        np.exp(rng.uniform(np.log(1e-6), np.log(6e4), 291)).astype(np.float32)]).astype(np.float16)
+    R = scales.size
+    x = np.broadcast_to(num, (R, num.size)).copy()
+    meta = np.zeros(2 * R, np.float16)
+    meta[0::2] = scales
+    for bits in (8, 4):
+        got = quik.asymmetric.quantizeOld(_t(x), _t(meta), bits).cpu().numpy()
+        want = qo.quantize_old(x, meta, bits)
+        assert np.array_equal(got, want)
+
+
+def test_fast_quotient_path_exhaustive_rows():
+    """The row kernel's reciprocal + correction quotient: rows that contain every fp16 value in
+    [0, hi] so that x - zero runs over all numerators for a fixed scale."""
+    import quik
+    rng = np.random.default_rng(12)
+    rows = []
+    for hi_bits in [0x3C00, 0x4B80, 0x5BF8, 0x7BFF, 0x0400, 0x2E66, 0x5640] + list(rng.integers(0x0400, 0x7BFF, 40)):
+        vals = np.arange(0, int(hi_bits) + 1, dtype=np.uint16)
+        row = np.zeros(0x7C00, np.uint16)
+        row[:vals.size] = vals
+        rows.append(row)
+    x = np.stack(rows).view(np.float16)
+    n_in = x.shape[1]
+    ii = np.arange(n_in, dtype=np.int64)
+    fi = np.zeros(0, np.int64)
+    for bits in (4, 8):
+        q, m, _ = quik.asymmetric.quantize(_t(x), _t(ii), _t(fi), bits)
+        dst, meta, _ = qo.asym_quantize(x, ii, fi, bits)
+        assert np.array_equal(_bits(m), meta.view(np.uint16))
+        assert np.array_equal(q.cpu().numpy(), dst)
+
+
+def test_asym_quantize_argument_errors():
+    import quik
+    x = torch.randn(4, 64, dtype=torch.float16, device=DEV)
+    ii = torch.arange(62, device=DEV)
+    fi = torch.tensor([62, 63], device=DEV)
+    with pytest.raises(RuntimeError, match="either 4 or 8"):
+        quik.asymmetric.quantize(x, ii, fi, 5)
+    with pytest.raises(RuntimeError, match="not equal to total number of columns"):
+        quik.asymmetric.quantize(x, ii[:-2], fi, 4)
+    with pytest.raises(RuntimeError, match="has to be even"):
+        quik.asymmetric.quantize(x, torch.arange(61, device=DEV), torch.tensor([61, 62, 63], device=DEV), 4)
+    with pytest.raises(RuntimeError, match="contiguous"):
+        quik.asymmetric.quantize(x.t().contiguous().t(), ii, fi, 4)
+    with pytest.raises(RuntimeError, match="CUDA"):
+        quik.asymmetric.quantize(x.cpu(), ii, fi, 4)
+    with pytest.raises(RuntimeError, match="float16"):
+        quik.asymmetric.quantize(x.float(), ii, fi, 4)
+    with pytest.raises(TypeError):
+        quik.asymmetric.quantize(x, ii, fi)
+    q, m, f = quik.asymmetric.quantize(x[:0], ii, fi, 4)   # empty batch
+    assert q.shape == (0, 31) and m.shape == (0,) and f.shape == (0, 2)
+
+
+# ------------------------------------------------------------------------------ integer GEMM
+MM_CASES = [
+    # M, N, K
+    (512, 32, 512),      # the reference's test_matmul.py case
+    (1, 128, 3968),
+    (16, 300, 96),
+    (100, 40, 32),
+    (257, 384, 3840),
+    (128, 512, 4864),
+    (300, 260, 7936),
+    (512, 1024, 3968),
+]
+
+
+@pytest.mark.parametrize("M,N,K", MM_CASES)
+def test_int4_matmul_exact(M, N, K):
+    import quik
+    rng = np.random.default_rng(M * 7 + N * 3 + K)
+    a = rng.integers(-8, 8, (M, K)).astype(np.int8)
+    b = rng.integers(-8, 8, (N, K)).astype(np.int8)
+    if M >= 2 and N >= 2:
+        a[0, :] = -8
+        b[0, :] = -8      # largest magnitude accumulators: 64 * K
+        a[1, :] = 7
+        b[1, :] = -8
+    want = qo.int_matmul(a, b)
+    c = quik.matmul.int4Matmul(_t(qo.pack_i4(a)), _t(qo.pack_i4(b)))
+    assert c.dtype == torch.int32 and c.shape == (M, N)
+    assert np.array_equal(c.cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("M,N,K", [(512, 32, 512), (1, 128, 13568), (16, 300, 16), (100, 40, 48),
+                                     (257, 384, 10752), (300, 260, 2048), (2, 2, 28416)])
+def test_int8_matmul_exact(M, N, K):
+    import quik
+    rng = np.random.default_rng(M * 5 + N * 11 + K)
+    a = rng.integers(-128, 128, (M, K)).astype(np.int8)
+    b = rng.integers(-128, 128, (N, K)).astype(np.int8)
+    if M >= 2 and N >= 2:
+        a[0, :] = -128
+        b[0, :] = -128
+        a[1, :] = 127
+        b[1, :] = -128
+    want = qo.int_matmul(a, b)
+    c = quik.matmul.int8Matmul(_t(a), _t(b))
+    assert np.array_equal(c.cpu().numpy(), want)
+
+
+def test_matmul_reference_known_answer():
+    """test/python/test_matmul.py:16-26 as written there: randint(-8, 7), float bmm, round, int32."""
+    import quik
+    from quik_amd.qlinear import pack_to_i4
+    torch.manual_seed(0)
+    B, M, K, N = 1, 512, 512, 32
+    a = torch.randint(-8, 7, (B, M, K), dtype=torch.int8).to(DEV)
+    b = torch.randint(-8, 7, (B, N, K), dtype=torch.int8).to(DEV)
+    c_gt = torch.bmm(a.float(), b.float().transpose(1, 2)).round().to(torch.int32)
+    c = quik.matmul.int4Matmul(pack_to_i4(a[0]), pack_to_i4(b[0]))
+    assert torch.equal(c, c_gt[0])
+
+
+def test_matmul_argument_errors():
+    import quik
+    a = torch.zeros((4, 16), dtype=torch.uint8, device=DEV)
+    with pytest.raises(RuntimeError, match="alignment"):
+        quik.matmul.int4Matmul(a[:, :8].contiguous(), a[:, :8].contiguous())     # K = 16 int4, not % 32
+    with pytest.raises(RuntimeError, match="agree in K"):
+        quik.matmul.int4Matmul(a, torch.zeros((4, 32), dtype=torch.uint8, device=DEV))
+    with pytest.raises(RuntimeError, match="contiguous"):
+        quik.matmul.int4Matmul(torch.zeros((16, 4), dtype=torch.uint8, device=DEV).t(), a)
+    with pytest.raises(RuntimeError, match="CUDA"):
+        quik.matmul.int4Matmul(a.cpu(), a.cpu())
+    with pytest.raises(RuntimeError, match="expected torch.int8"):
+        quik.matmul.int8Matmul(a, a)
+    assert quik.matmul.int4Matmul(a[:0], a).shape == (0, 4)
+
+
+# ------------------------------------------------------------------------------ dequantize
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("M,N", [(24, 40), (33, 100), (256, 1024), (5, 7)])
+def test_asym_dequantize(bits, bf16, M, N):
+    import quik
+    rng = np.random.default_rng(M + N + bits)
+    dt = qo.BF16 if bf16 else qo.F16
+    rnd = (lambda v: qo.bf16_round(v.astype(np.float32))) if bf16 else (lambda v: v.astype(np.float16))
+    tt = _bf16_t if bf16 else _t
+    acc = rng.integers(-500000, 500000, (M, N)).astype(np.int32)
+    acc[0, 0] = 2 ** 31 - 1
+    acc[-1, -1] = -2 ** 31
+    meta = rnd(np.stack([rng.uniform(0.01, 0.3, M), rng.uniform(-3, 0, M)], 1).reshape(-1))
+    scol = rnd(rng.uniform(0.001, 0.01, (N, 1)))
+    wred = rnd(rng.standard_normal((1, N)))
+    y = rnd(rng.standard_normal((M, N)) * 3)
+    out = quik.asymmetric.dequantize(_t(acc), tt(meta), tt(scol), tt(wred), tt(y), bits)
+    want = qo.asym_dequantize(acc, meta, scol, wred, y, bits, dt)
+    want_b = qo.f32_to_bf16_bits(want) if bf16 else want.view(np.uint16)
+    assert out.dtype == (torch.bfloat16 if bf16 else torch.float16)
+    assert np.array_equal(_bits(out), want_b)
+    ref = qo.asym_dequantize_f64(acc, meta, scol, wred, y, bits, dt)
+    ulp = np.maximum(np.abs(ref), 2.0 ** -14) * (2.0 ** -7 if bf16 else 2.0 ** -10)
+    got = out.float().cpu().numpy().astype(np.float64)
+    fin = np.isfinite(got)
+    assert (np.abs(got - ref)[fin] <= ulp[fin]).all()
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("cols", [128, 130, 127])
+def test_sym_quantize_bit_exact(bits, cols):
+    import quik
+    torch.manual_seed(1)
+    src = torch.randn(48, cols, dtype=torch.float16)
+    scale = torch.randn(48, 1, dtype=torch.float16)
+    src[0, :4] = torch.tensor([float("inf"), float("nan"), 65504.0, -65504.0], dtype=torch.float16)
+    got = quik.symmetric.quantize(src.to(DEV), scale.to(DEV), bits).cpu().numpy()
+    want = qo.sym_quantize(src.numpy(), scale.numpy(), bits)
+    assert np.array_equal(got, want)
+    if bits == 8:
+        # the reference's own assertion (test/python/test_cuaprseLt.py:21-23) where it is defined
+        ref = (src / scale).round()
+        ok = (ref.abs() <= 127).numpy()
+        assert np.array_equal(got[ok], ref.to(torch.int8).numpy()[ok])
+
+
+@pytest.mark.parametrize("bits", [8, 16, 32])
+def test_sym_dequantize_bit_exact(bits):
+    """test/python/test_cuaprseLt.py:45-47: c * scale_row * scale_col + y in torch fp16, bit-equal."""
+    import quik
+    torch.manual_seed(2)
+    M, N = 37, 53
+    sr = torch.randn(M, 1, dtype=torch.float16)
+    sc = torch.randn(1, N, dtype=torch.float16)
+    y = torch.randn(M, N, dtype=torch.float16)
+    if bits == 16:
+        c = (torch.randn(M, N) * 100).half()
+        ch = c
+    elif bits == 8:
+        c = torch.randint(-128, 128, (M, N), dtype=torch.int8)
+        ch = c.half()
+    else:
+        c = torch.randint(-70000, 70000, (M, N), dtype=torch.int32)
+        ch = c.half()
+    out = quik.symmetric.dequantize(c.to(DEV), sr.to(DEV), sc.to(DEV), y.to(DEV), bits).cpu()
+    ref = ch * sr * sc + y
+    fin = torch.isfinite(ref)
+    assert torch.equal(out[fin], ref[fin]) and torch.equal(torch.isnan(out), torch.isnan(ref))
+    want = qo.sym_dequantize(c.numpy(), sr.numpy(), sc.numpy(), y.numpy(), bits)
+    assert np.array_equal(out.numpy()[fin.numpy()], want[fin.numpy()])
+
+
+# ------------------------------------------------------------------------------ MixedQLinear
+def _layer(rng, N, n_in, F, bits):
+    ii, fi = _split(rng, n_in, F)
+    lo, hi = (-8, 8) if bits == 4 else (-127, 128)
+    codes = rng.integers(lo, hi, (N, n_in - F))
+    s_w = rng.uniform(0.001, 0.01, (N, 1)).astype(np.float16)
+    W = np.zeros((N, n_in), np.float16)
+    W[:, ii] = (codes * s_w.astype(np.float32)).astype(np.float16)
+    W[:, fi] = (0.02 * rng.standard_normal((N, F))).astype(np.float16)
+    return W, s_w, ii, fi
+
+
+def _module(W, s_w, fi, bits, bias=None, symm=False, fused=True, shared=None):
+    from quik_amd.qlinear import MixedQLinear
+    N, n_in = W.shape
+    lin = torch.nn.Linear(n_in, N, bias=bias is not None)
+    if bias is not None:
+        lin.bias.data = torch.from_numpy(bias)
+    mod = MixedQLinear.from_float(lin, torch.from_numpy(W), torch.from_numpy(s_w), shared,
+                                  torch.from_numpy(fi) if fi.size else None, symm=symm, bits=bits, fused=fused)
+    return mod.to(DEV)
+
+
+FWD_CASES = [
+    # M, N, in, F, bits, bias, kind
+    (32, 64, 512, 32, 4, False, "x50"),
+    (100, 200, 1024, 64, 4, True, "student"),
+    (300, 520, 4096, 128, 4, False, "x50"),
+    (16, 256, 2048, 256, 8, False, "x50"),
+    (260, 300, 1280, 256, 8, True, "x50"),
+    (64, 128, 512, 0, 4, True, "x50"),
+    (1, 384, 1024, 64, 4, False, "x50"),
+]
+
+
+@pytest.mark.parametrize("case", FWD_CASES)
+def test_mixed_qlinear_forward(case):
+    M, N, n_in, F, bits, with_bias, kind = case
+    rng = np.random.default_rng(sum(case[:5]))
+    W, s_w, ii, fi = _layer(rng, N, n_in, F, bits)
+    bias = rng.standard_normal(N).astype(np.float16) if with_bias else None
+    x = _acts(rng, M, n_in, fi, kind).astype(np.float16)
+    omod = qo.from_float(W, s_w, fi, bits)
+    want, inter = qo.mixed_qlinear_forward(x, omod, bits, bias)
+    mod = _module(W, s_w, fi, bits, bias)
+    # from_float buffers are those of the oracle
+    assert np.array_equal(mod.int_weight.cpu().numpy(), omod["int_weight"])
+    assert np.array_equal(mod.int_indices.cpu().numpy(), omod["int_indices"])
+    assert np.array_equal(mod.reduced_w.cpu().numpy(), omod["reduced_w"])
+    out = mod(_t(x))
+    assert out.shape == (1, M, N) and out.dtype == torch.float16
+    got = out[0].float().cpu().numpy().astype(np.float64)
+    w64 = want.astype(np.float64)
+    rms = np.sqrt((w64 ** 2).mean())
+    err = np.abs(got - w64).max()
+    assert err <= 1e-2 * rms, (err, rms)
+    # much tighter in practice: a few output ulps of the largest term
+    assert err <= 4 * np.abs(w64).max() * 2.0 ** -10
+    # unfused op sequence: integer stages bit-exact, output = oracle up to the outlier GEMM's order
+    mod_u = _module(W, s_w, fi, bits, bias, fused=False)
+    out_u = mod_u(_t(x))[0].float().cpu().numpy().astype(np.float64)
+    assert np.abs(out_u - w64).max() <= 4 * np.abs(w64).max() * 2.0 ** -10
+    # the algebraic identity against a float64 linear layer on the dequantised activation
+    xd = qo.dequantized_activation_f64(x, ii, fi, bits)
+    ref = xd @ W.astype(np.float64).T + (0 if bias is None else bias.astype(np.float64))
+    assert np.abs(got - ref).max() <= 1e-2 * np.sqrt((ref ** 2).mean())
+
+
+def test_mixed_qlinear_bf16_and_3d_input():
+    from quik_amd.qlinear import MixedQLinear
+    rng = np.random.default_rng(21)
+    N, n_in, F, bits = 192, 768, 64, 4
+    W, s_w, ii, fi = _layer(rng, N, n_in, F, bits)
+    Wb = torch.from_numpy(W.astype(np.float32)).to(torch.bfloat16)
+    sb = torch.from_numpy(s_w.astype(np.float32)).to(torch.bfloat16)
+    # rebuild W so that codes * scale round-trips in bf16
+    codes = (torch.from_numpy(W[:, ii].astype(np.float32)) / torch.from_numpy(s_w.astype(np.float32))).round()
+    Wb[:, torch.from_numpy(ii)] = (codes * sb.float()).to(torch.bfloat16)
+    lin = torch.nn.Linear(n_in, N, bias=False)
+    mod = MixedQLinear.from_float(lin, Wb, sb, None, torch.from_numpy(fi), bits=bits).to(DEV)
+    x = torch.from_numpy(_acts(rng, 2 * 48, n_in, fi)).to(torch.bfloat16).reshape(2, 48, n_in)
+    out = mod(x.to(DEV))
+    assert out.shape == (2, 48, N) and out.dtype == torch.bfloat16
+    xs = x.reshape(-1, n_in).float().numpy()
+    omod = qo.from_float(Wb.float().numpy(), sb.float().numpy(), fi, bits, dtype=qo.BF16)
+    want, _ = qo.mixed_qlinear_forward(xs, omod, bits, None, dtype=qo.BF16)
+    got = out.reshape(-1, N).float().cpu().numpy()
+    rms = np.sqrt((want.astype(np.float64) ** 2).mean())
+    assert np.abs(got - want).max() <= 1e-2 * rms
+
+
+def test_shared_quantized_input_group():
+    """q/k/v-style group (experiments/llama.py:402-411): the first member quantizes, all reuse."""
+    from quik_amd.qlinear import SharedQuantizedInput
+    rng = np.random.default_rng(22)
+    n_in, F, bits, M = 512, 32, 4, 40
+    shared = SharedQuantizedInput(3)
+    mods, omods = [], []
+    fi = None
+    for N in (64, 96, 128):
+        W, s_w, ii, fi_new = _layer(np.random.default_rng(5), N, n_in, F, bits)   # same split for the group
+        fi = fi_new
+        mods.append(_module(W, s_w, fi, bits, shared=shared))
+        omods.append(qo.from_float(W, s_w, fi, bits))
+    x = _acts(rng, M, n_in, fi).astype(np.float16)
+    xt = _t(x)
+    for i, (m, om) in enumerate(zip(mods, omods)):
+        out = m(xt)[0].float().cpu().numpy()
+        want, _ = qo.mixed_qlinear_forward(x, om, bits)
+        assert np.abs(out - want).max() <= 1e-2 * np.sqrt((want.astype(np.float64) ** 2).mean())
+        assert (shared.qint_x is None) == (i == 2)
+
+
+def test_symmetric_mixed_qlinear():
+    """Symmetric activations (scale = max|x| / 4 as the reference's expression evaluates):
+    codes bit-exact with the oracle; fused fp32 epilogue within tolerance of the fp16-chain op."""
+    rng = np.random.default_rng(23)
+    M, N, n_in, F, bits = 48, 96, 512, 32, 4
+    W, s_w, ii, fi = _layer(rng, N, n_in, F, bits)
+    x = _acts(rng, M, n_in, fi).astype(np.float16)
+    omod = qo.from_float(W, s_w, fi, bits, symm=True)
+    want, inter = qo.mixed_qlinear_forward(x, omod, bits, None, symm=True)
+    mod_u = _module(W, s_w, fi, bits, symm=True, fused=False)
+    out_u = mod_u(_t(x))[0].cpu().numpy()
+    fin = np.isfinite(want)
+    rms = np.sqrt((want[fin].astype(np.float64) ** 2).mean())
+    assert np.abs(out_u[fin].astype(np.float64) - want[fin]).max() <= 1e-2 * rms
+    mod = _module(W, s_w, fi, bits, symm=True, fused=True)
+    out = mod(_t(x))[0].float().cpu().numpy()
+    assert np.abs(out[fin].astype(np.float64) - want[fin]).max() <= 1e-2 * rms
+
+
+# ------------------------------------------------------------------------------ full-size properties
+def test_full_size_properties_llama70b_gate_proj():
+    """Llama-2-70B gate_proj (M=2048, in=8192, K=7936, N=28672): too large for a CPU product, so
+    the integer GEMM is checked through size-independent identities (row and column checksums,
+    exact in float64), the quantize kernel against the full oracle, and the fused output against
+    dequantize applied to the exact accumulators on a tile sample."""
+    import quik
+    g = torch.Generator().manual_seed(0)
+    M, n_in, F, N = 2048, 8192, 256, 28672
+    K = n_in - F
+    x = torch.randn(M, n_in, generator=g)
+    fi = torch.randperm(n_in, generator=g)[:F]
+    x[:, fi] *= 50
+    x = x.half()
+    ii = torch.arange(n_in)
+    ii = ii[~torch.isin(ii, fi)]
+    xd, iid, fid = x.to(DEV), ii.to(DEV), fi.to(DEV)
+    q, meta, fp = quik.asymmetric.quantize(xd, iid, fid, 4)
+    dst, m, f = qo.asym_quantize(x.numpy(), ii.numpy(), fi.numpy(), 4)
+    assert np.array_equal(q.cpu().numpy(), dst)
+    assert np.array_equal(_bits(meta), m.view(np.uint16))
+    assert torch.equal(fp.cpu(), x[:, fi])
+
+    qw = torch.randint(0, 256, (N, K // 2), dtype=torch.uint8, generator=g).to(DEV)
+    c = quik.matmul.int4Matmul(q, qw)
+
+    def unpack(p):  # uint8 [R, K/2] -> float64 [R, K] on the GPU
+        lo = (p & 0xF).to(torch.int16)
+        hi = (p >> 4).to(torch.int16)
+        lo = torch.where(lo >= 8, lo - 16, lo)
+        hi = torch.where(hi >= 8, hi - 16, hi)
+        return torch.stack([lo, hi], dim=2).reshape(p.shape[0], -1).double()
+
+    a64 = unpack(q)
+    colsum_b = torch.zeros(K, dtype=torch.float64, device=DEV)
+    for s in range(0, N, 4096):
+        colsum_b += unpack(qw[s:s + 4096]).sum(0)
+    assert torch.equal(c.double().sum(1), a64 @ colsum_b)            # sum_n C[m, n]
+    rowsum_a = a64.sum(0)
+    for s in range(0, N, 4096):
+        assert torch.equal(c[:, s:s + 4096].double().sum(0), unpack(qw[s:s + 4096]) @ rowsum_a)   # sum_m C[m, n]
+    # exact spot tiles against the oracle
+    for (r0, c0) in [(0, 0), (1000, 14000), (2048 - 64, 28672 - 64)]:
+        want = qo.int4_matmul(dst[r0:r0 + 64], qw[c0:c0 + 64].cpu().numpy())
+        assert np.array_equal(c[r0:r0 + 64, c0:c0 + 64].cpu().numpy(), want)
+
+    s_w = (torch.rand(N, 1, generator=g) * 0.009 + 0.001).half().to(DEV)
+    wred = torch.randn(1, N, generator=g).half().to(DEV)
+    fpw = (0.02 * torch.randn(N, F, generator=g)).half().to(DEV)
+    out = quik.matmul.mixed_linear(q, qw, meta, s_w, wred, fp, fpw, None, 4, torch.float16)
+    for (r0, c0) in [(0, 0), (1000, 14000), (2048 - 64, 28672 - 64)]:
+        y = qo.fp_linear(f[r0:r0 + 64], fpw[c0:c0 + 64].cpu().numpy(), None)
+        want = qo.asym_dequantize(c[r0:r0 + 64, c0:c0 + 64].cpu().numpy(), m[2 * r0:2 * r0 + 128],
+                                  s_w[c0:c0 + 64].cpu().numpy(), wred[:, c0:c0 + 64].cpu().numpy(), y, 4)
+        got = out[r0:r0 + 64, c0:c0 + 64].float().cpu().numpy()
+        w64 = want.astype(np.float64)
+        assert np.abs(got - w64).max() <= 1e-2 * np.sqrt((w64 ** 2).mean())
+        assert np.abs(got - w64).max() <= 4 * np.abs(w64).max() * 2.0 ** -10
