@@ -33,14 +33,17 @@ def act_fake_quant(q_features: torch.Tensor, bits: int) -> torch.Tensor:
 
 
 def sim_mixed_linear(x: torch.Tensor, weight: torch.Tensor, int_idx: torch.Tensor, fp_idx: torch.Tensor,
-                     bits: int, bias: torch.Tensor | None = None) -> torch.Tensor:
+                     bits: int, bias: torch.Tensor | None = None,
+                     weight_f32: torch.Tensor | None = None) -> torch.Tensor:
     """ActQuantWrapper.forward (quant_sim.py:227-256) around F.linear with the fake-quant weight.
 
-    x [M, in] and weight [N, in] are fp16 (storage); compute in fp32; result fp16."""
+    x [M, in] and weight [N, in] are fp16 (storage); compute in fp32; result fp16.  `weight_f32`
+    may carry the weight already widened to fp32 so that a timing loop excludes that copy."""
     xf = x.float()
     mixed = torch.zeros_like(xf)
     mixed[:, int_idx] = act_fake_quant(xf[:, int_idx], bits).to(x.dtype).float()
     if fp_idx.numel():
         mixed[:, fp_idx] = xf[:, fp_idx]
-    out = torch.nn.functional.linear(mixed, weight.float(), None if bias is None else bias.float())
+    w32 = weight.float() if weight_f32 is None else weight_f32
+    out = torch.nn.functional.linear(mixed, w32, None if bias is None else bias.float())
     return out.to(x.dtype)

@@ -444,10 +444,19 @@ def test_mixed_qlinear_bf16_and_3d_input():
     assert out.shape == (2, 48, N) and out.dtype == torch.bfloat16
     xs = x.reshape(-1, n_in).float().numpy()
     omod = qo.from_float(Wb.float().numpy(), sb.float().numpy(), fi, bits, dtype=qo.BF16)
-    want, _ = qo.mixed_qlinear_forward(xs, omod, bits, None, dtype=qo.BF16)
-    got = out.reshape(-1, N).float().cpu().numpy()
-    rms = np.sqrt((want.astype(np.float64) ** 2).mean())
-    assert np.abs(got - want).max() <= 1e-2 * rms
+    want, inter = qo.mixed_qlinear_forward(xs, omod, bits, None, dtype=qo.BF16)
+    got = out.reshape(-1, N).float().cpu().numpy().astype(np.float64)
+    w64 = want.astype(np.float64)
+    # bf16 keeps 8 significant bits: one output ulp (2^-7 relative) already exceeds 1e-2 x RMS for the
+    # larger outputs, and the oracle (like the reference) rounds the outlier product to bf16 before the
+    # final sum.  Bound: one bf16 ulp of the output plus one of that intermediate; then the stated
+    # tolerance against the unrounded float64 result.
+    y64 = np.abs(inter["fp_result"].astype(np.float64))
+    assert (np.abs(got - w64) <= (np.abs(w64) + y64) * 2.0 ** -7).all()
+    xd = qo.dequantized_activation_f64(xs, omod["int_indices"], fi, bits, qo.BF16)
+    ref = xd @ Wb.double().numpy().T
+    rms = np.sqrt((ref ** 2).mean())
+    assert (np.abs(got - ref) <= 1e-2 * rms + np.abs(ref) * 2.0 ** -8).all()
 
 
 def test_shared_quantized_input_group():
