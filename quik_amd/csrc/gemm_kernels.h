@@ -69,6 +69,14 @@ __device__ __forceinline__ void unpack_i4(const v4i w, v4i &f0, v4i &f1) {
   f1 = v4i{(w.z << 4) & kMask, w.z & kMask, (w.w << 4) & kMask, w.w & kMask};
 }
 
+template <int N, int I = 0, class F>
+__device__ __forceinline__ void static_for(F &&f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    static_for<N, I + 1>(f);
+  }
+}
+
 template <int MODE>
 struct FragOps {
   static constexpr int H = MODE == kInt4 ? 2 : 1;  // MFMA k-steps per 32-byte sub-step
@@ -285,21 +293,31 @@ struct DmaPipe {
     w_off = X_REGION + (wn * C::WN + (lane & 31)) * 64 + (((lane >> 5) ^ fl) << 4);
   }
 
-  // stage index is clamped: surplus issues re-load the last stage into a dead slot.  Branch-free
-  // (selects only) so the loads stay in the main loop's basic block and interleave with MFMAs.
-  __device__ __forceinline__ void issue(int stage) const {
+  // Load `idx` (0 .. kPerStage-1) of a stage.  The stage index is clamped: surplus issues re-load the
+  // last stage into a dead slot.  Branch-free (selects only) so the loads stay in the main loop's
+  // basic block, where they are spread between the MFMAs.
+  template <int IDX>
+  __device__ __forceinline__ void issue_one(int stage) const {
     const int st = stage < stages ? stage : stages - 1;
     const uint32_t slot = lds0 + (stage & (NS - 1)) * STAGE;
     const bool second = st >= stages0;
     const int kb = (second ? st - stages0 : st) * 64;
-    const uint8_t *xb = (second ? X[1] : X[0]) + kb, *wb = (second ? W[1] : W[0]) + kb;
-#pragma unroll
-    for (int j = 0; j < X_INSTR; ++j)
-      dma_load16(xb, second ? vx[1][j] : vx[0][j], slot + (wave * X_INSTR + j) * 1024);
-#pragma unroll
-    for (int j = 0; j < W_INSTR; ++j)
-      dma_load16(wb, second ? vw[1][j] : vw[0][j], slot + X_REGION + (wave * W_INSTR + j) * 1024);
+    if constexpr (IDX < X_INSTR) {
+      dma_load16((second ? X[1] : X[0]) + kb, second ? vx[1][IDX] : vx[0][IDX], slot + (wave * X_INSTR + IDX) * 1024);
+    } else {
+      constexpr int J = IDX - X_INSTR;
+      dma_load16((second ? W[1] : W[0]) + kb, second ? vw[1][J] : vw[0][J],
+                 slot + X_REGION + (wave * W_INSTR + J) * 1024);
+    }
   }
+  template <int FIRST, int COUNT>
+  __device__ __forceinline__ void issue_range(int stage) const {
+    if constexpr (COUNT > 0) {
+      issue_one<FIRST>(stage);
+      issue_range<FIRST + 1, COUNT - 1>(stage);
+    }
+  }
+  __device__ __forceinline__ void issue(int stage) const { issue_range<0, kPerStage>(stage); }
 
   __device__ __forceinline__ const v4i *frag_ptr(int stage, int ks, int j) const {
     const int off = j < MI ? (x_off ^ (ks * 32)) + j * 2048 : (w_off ^ (ks * 32)) + (j - MI) * 2048;
@@ -322,7 +340,8 @@ struct DmaPipe {
     using Ops = FragOps<MODE>;
     constexpr int H = Ops::H;
     // U[p]: operand set consumed by a sub-step of parity p (fragment j < MI: X row block j,
-    // fragment MI + j: W column block j).  R (int4 only): raw nibbles one sub-step further ahead.
+    // fragment MI + j: W column block j).  R (int4 only): raw nibbles, read from LDS two sub-steps
+    // ahead of their MFMAs and unpacked one sub-step ahead.
     v4i U[2][NF][H];
     v4i R[NF];
     if constexpr (MODE == kInt4) {
@@ -337,19 +356,31 @@ struct DmaPipe {
       for (int j = 0; j < NF; ++j) U[0][j][0] = *frag_ptr(kt_begin, 0, j);
     }
 
-    // (rs, rk): the sub-step whose fragments are read from LDS now.
-    auto substep = [&](auto parity, int rs, int rk) {
+    // Sub-step of parity P: MFMAs consume U[P]; R (raw, sub-step t+1) is unpacked into U[1-P] and
+    // refilled, fragment by fragment, from (rs, rk) (sub-step t+2; for the other modes the fragments
+    // of sub-step t+1 go straight into U[1-P]).  `half` selects which half of stage `ld_stage`'s
+    // global loads is issued here; in program order one load follows every few fragment reads, which
+    // keeps them spread over the MFMAs instead of bunched, where their issue time would stall the
+    // matrix pipe.
+    auto substep = [&](auto parity, auto half, int rs, int rk, int ld_stage) {
       constexpr int P = decltype(parity)::value;
-      if constexpr (MODE == kInt4) {
-#pragma unroll
-        for (int j = 0; j < NF; ++j) {
+      constexpr int kLoads = (kPerStage + 1) / 2;
+      constexpr int kFirst = decltype(half)::value * kLoads;
+      constexpr int kCount = kFirst + kLoads <= kPerStage ? kLoads : kPerStage - kFirst;
+      constexpr int kEvery = NF / (kCount > 0 ? kCount : 1) > 0 ? NF / (kCount > 0 ? kCount : 1) : 1;
+      auto per_frag = [&](auto jc) {
+        constexpr int j = decltype(jc)::value;
+        if constexpr (MODE == kInt4) {
           Ops::unpack(R[j], U[1 - P][j]);
           R[j] = *frag_ptr(rs, rk, j);
+        } else {
+          U[1 - P][j][0] = *frag_ptr(rs, rk, j);
         }
-      } else {
-#pragma unroll
-        for (int j = 0; j < NF; ++j) U[1 - P][j][0] = *frag_ptr(rs, rk, j);
-      }
+        if constexpr ((j + 1) % kEvery == 0 && (j + 1) / kEvery - 1 < kCount) {
+          if ((C::EXP & 15) != 2) issue_one<kFirst + (j + 1) / kEvery - 1>(ld_stage);
+        }
+      };
+      static_for<NF>(per_frag);
 #pragma unroll
       for (int ni = 0; ni < NI; ++ni)
 #pragma unroll
@@ -367,17 +398,20 @@ struct DmaPipe {
       }
     };
 
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
     for (int kt = kt_begin; kt < kt_end; ++kt) {
-      if ((C::EXP & 15) != 2) issue(kt + 3);
       if constexpr (MODE == kInt4) {
-        substep(std::integral_constant<int, 0>{}, kt + 1, 0);
-        substep(std::integral_constant<int, 1>{}, kt + 1, 1);
+        substep(I0{}, I0{}, kt + 1, 0, kt + 3);
+        substep(I1{}, I1{}, kt + 1, 1, kt + 3);
       } else {
-        substep(std::integral_constant<int, 0>{}, kt, 1);
-        substep(std::integral_constant<int, 1>{}, kt + 1, 0);
+        substep(I0{}, I0{}, kt, 1, kt + 3);
+        substep(I1{}, I1{}, kt + 1, 0, kt + 3);
       }
-      __builtin_amdgcn_s_waitcnt(vmcnt_imm(kPerStage));  // stage kt+2 has landed, stage kt+3 may be in flight
-      __syncthreads();
+      // Stage kt+2 has landed (stage kt+3 may stay in flight), then a bare barrier: the LDS reads
+      // still outstanding target a slot nobody writes before the next barrier, so they need no wait.
+      __builtin_amdgcn_s_waitcnt(vmcnt_imm(kPerStage));
+      __builtin_amdgcn_s_barrier();
     }
   }
 
