@@ -49,15 +49,42 @@ __device__ __forceinline__ float round_storage(float f) {
   return to_f32<BF16>(from_f32<BF16>(f));
 }
 
+// Lane exchange inside a row of 16 lanes through the DPP path of the vector ALU (no LDS traffic).
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, false));
+}
+constexpr int kDppSwap1 = 0xB1;        // quad_perm [1,0,3,2]
+constexpr int kDppSwap2 = 0x4E;        // quad_perm [2,3,0,1]
+constexpr int kDppHalfMirror = 0x141;  // lane i <-> 7 - i inside each group of 8
+constexpr int kDppMirror = 0x140;      // lane i <-> 15 - i inside each row of 16
+
+// Wave-wide reductions; every lane of the wave must be active.  Four DPP steps make each row of 16
+// uniform, the four rows are then combined through scalar registers.
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-  return v;
+  v = fmaxf(v, dpp_move<kDppSwap1>(v));
+  v = fmaxf(v, dpp_move<kDppSwap2>(v));
+  v = fmaxf(v, dpp_move<kDppHalfMirror>(v));
+  v = fmaxf(v, dpp_move<kDppMirror>(v));
+  const int b = __builtin_bit_cast(int, v);
+  const float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 0));
+  const float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 16));
+  const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 32));
+  const float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 48));
+  return fmaxf(fmaxf(r0, r1), fmaxf(r2, r3));
 }
 __device__ __forceinline__ float wave_min(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v = fminf(v, __shfl_xor(v, o, 64));
-  return v;
+  v = fminf(v, dpp_move<kDppSwap1>(v));
+  v = fminf(v, dpp_move<kDppSwap2>(v));
+  v = fminf(v, dpp_move<kDppHalfMirror>(v));
+  v = fminf(v, dpp_move<kDppMirror>(v));
+  const int b = __builtin_bit_cast(int, v);
+  const float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 0));
+  const float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 16));
+  const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 32));
+  const float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 48));
+  return fminf(fminf(r0, r1), fminf(r2, r3));
 }
 
 }  // namespace quik

@@ -8,19 +8,24 @@
 //   v     = rne_int(t), NaN -> 0;  code = clamp(v, 0, 2^bits - 1) - 2^(bits-1)
 // (reference: src/asymmetric/asymmetric.cu:340-435).
 //
-// Data flow of the asymmetric kernel, one 256-thread workgroup per row:
-//   1. the row is streamed once from HBM with 16-byte loads into LDS; min/max are taken on
-//      the fly over the non-outlier columns using one mask bit per column;
-//   2. each lane then gathers two consecutive destination codes per step from LDS through a
-//      compact source-column table, quantises them and stores one packed byte (int4) or two
-//      bytes (int8); consecutive lanes hit consecutive LDS dwords and consecutive output bytes;
-//   3. the outlier columns are gathered from LDS in the order the caller listed them.
-// The quotient uses r = 1/scale (one IEEE division per row) and one Markstein correction
-// step, q = d*r; e = fma(-q, s, d); q' = fma(e, r, q).  q' is within 2^-24(1+eps) of d/s
-// relative, while d/s with 11-bit (8-bit for bf16) significands stays more than 2^-23
-// relative away from every rounding boundary of the storage type, so storage(q') equals the
-// correctly rounded storage(d/s).  Rows whose range overflows the storage type, or whose
-// scale is below 1e-20 (bf16 only), take the plain IEEE division instead.
+// Two kernels implement it.  The streaming kernel (see "Streaming path" below) serves the usual
+// layout, ascending int_indices; the gather kernel serves any other order: it copies the row
+// to LDS with 16-byte loads while taking min/max over the non-outlier columns (one mask bit per
+// column), then each lane gathers two consecutive destination codes per step from LDS through a
+// compact source-column table and stores one packed byte (int4) or two bytes (int8).
+//
+// The quotient.  r = 1/scale is one IEEE division per row.  The gather kernel and the bf16
+// streaming path use q = d*r; e = fma(-q, s, d); q' = fma(e, r, q): q' is within
+// 2^-24(1+eps) of d/s relative, while d/s with 11-bit (8-bit for bf16) significands stays more
+// than 2^-23 relative away from every rounding boundary of the storage type, so storage(q')
+// equals the correctly rounded storage(d/s).  The fp16 streaming path uses fp16(d*r) without
+// the correction step: that value can differ from storage(d/s) in the last place (about 1.5e-6
+// of all (d, s) pairs) but never across a k + 1/2 boundary, so rne_int gives the same level for
+// every fp16 d >= 0 and every fp16 scale >= 1e-6 with both 4 and 8 bits; the tests enumerate
+// that whole domain.  Rows whose range overflows the storage type, or whose scale is below
+// 1e-20 (bf16 only), take the plain IEEE division instead.
+#include <type_traits>
+
 #include "common.h"
 
 namespace quik {
@@ -30,13 +35,31 @@ constexpr int kThreads = 256;
 
 // ---------------------------------------------------------------------------------------
 // column map layout: [src_col: num_int idx][fp_col: num_fp idx][mask: ceil(cols/32) u32]
+//                    [grp: ceil(cols/8) u32][dirty: min(num_fp, ceil(cols/8)) u32][flags: 4 u32]
 // idx is uint16_t when cols <= 65536, else uint32_t.  Section offsets are 16-byte aligned.
+// A "group" is 8 consecutive source columns (one 16-byte load).  A group without outliers is
+// clean, one with outliers is dirty; dirty groups are numbered in ascending order (slots).
+//   grp[g]   clean: (destination column of the group's first element) << 8
+//            dirty: (slot << 8) | mask byte (bit e set = column 8g+e is an outlier)
+//   dirty[s] (destination column of the group's first non-outlier element) << 8 | mask byte
+//   flags[0] bit 0: int_indices ascending, the two lists partition the columns and the shape
+//            fits the streaming kernel;  flags[1] = number of dirty groups.
+// grp and dirty exist only when cols <= kStreamMaxCols.
 struct ColmapLayout {
   bool idx16;
-  int64_t off_fp, off_mask, bytes;
+  int64_t off_fp, off_mask, off_grp, off_dirty, off_flags, bytes;
 };
 
 __host__ __device__ inline int64_t align16(int64_t v) { return (v + 15) & ~int64_t(15); }
+
+// Streaming (source-order) quantisation needs ascending int_indices, whole 16-byte chunks and at
+// most kStreamMaxCols columns (16 chunks per thread held in registers).
+constexpr int64_t kStreamMaxCols = 32768;
+
+__host__ __device__ inline int64_t max_dirty_groups(int64_t cols, int64_t num_fp) {
+  const int64_t groups = (cols + 7) / 8;
+  return num_fp < groups ? num_fp : groups;
+}
 
 __host__ __device__ inline ColmapLayout colmap_layout(int64_t cols, int64_t num_int, int64_t num_fp) {
   ColmapLayout l;
@@ -44,21 +67,38 @@ __host__ __device__ inline ColmapLayout colmap_layout(int64_t cols, int64_t num_
   const int64_t isz = l.idx16 ? 2 : 4;
   l.off_fp = align16(num_int * isz);
   l.off_mask = l.off_fp + align16(num_fp * isz);
-  l.bytes = l.off_mask + align16(((cols + 31) / 32) * 4);
+  l.off_grp = l.off_mask + align16(((cols + 31) / 32) * 4);
+  const bool stream = cols <= kStreamMaxCols;
+  l.off_dirty = l.off_grp + align16(stream ? ((cols + 7) / 8) * 4 : 0);
+  l.off_flags = l.off_dirty + align16(stream ? max_dirty_groups(cols, num_fp) * 4 : 0);
+  l.bytes = l.off_flags + 16;
   return l;
+}
+
+// number of non-zero bytes among the low `nbytes` bytes of w
+__device__ __forceinline__ uint32_t nonzero_bytes(uint32_t w, int nbytes) {
+  uint32_t n = 0;
+  for (int b = 0; b < nbytes; ++b) n += ((w >> (8 * b)) & 0xFFu) != 0u;
+  return n;
 }
 
 template <typename IdxT>
 __global__ __launch_bounds__(1024) void colmap_build_kernel(const int64_t *__restrict__ int_idx, int64_t num_int,
                                                             const int64_t *__restrict__ fp_idx, int64_t num_fp,
                                                             int64_t cols, IdxT *__restrict__ src_col,
-                                                            IdxT *__restrict__ fp_col, uint32_t *__restrict__ mask) {
+                                                            IdxT *__restrict__ fp_col, uint32_t *__restrict__ mask,
+                                                            uint32_t *__restrict__ grp, uint32_t *__restrict__ dirty,
+                                                            uint32_t *__restrict__ flags) {
   // single workgroup: the mask is cleared before any bit is set
+  __shared__ int ascending;
+  if (threadIdx.x == 0) ascending = 1;
   const int64_t words = (cols + 31) / 32;
   for (int64_t i = threadIdx.x; i < words; i += blockDim.x) mask[i] = 0u;
   __syncthreads();
   for (int64_t j = threadIdx.x; j < num_int; j += blockDim.x) {
     int64_t c = int_idx[j];
+    if (j + 1 < num_int && !(c < int_idx[j + 1])) ascending = 0;
+    if (c < 0 || c >= cols) ascending = 0;
     c = c < 0 ? 0 : (c >= cols ? cols - 1 : c);
     src_col[j] = static_cast<IdxT>(c);
   }
@@ -67,6 +107,42 @@ __global__ __launch_bounds__(1024) void colmap_build_kernel(const int64_t *__res
     c = c < 0 ? 0 : (c >= cols ? cols - 1 : c);
     fp_col[j] = static_cast<IdxT>(c);
     atomicOr(&mask[c >> 5], 1u << (c & 31));
+  }
+  __syncthreads();
+  const bool stream_shape = cols <= kStreamMaxCols && cols % 8 == 0;
+  // duplicates between the two index lists would make the popcount prefix wrong: require a partition
+  uint32_t total = 0, total_dirty = 0;
+  if (threadIdx.x == 0) {
+    for (int64_t w = 0; w < words; ++w) {
+      total += __popc(mask[w]);
+      total_dirty += nonzero_bytes(mask[w], 4);
+    }
+    flags[0] = (ascending && stream_shape && total == num_fp) ? 1u : 0u;
+    flags[1] = total_dirty;
+    flags[2] = flags[3] = 0u;
+  }
+  if (cols <= kStreamMaxCols) {
+    const int64_t groups = (cols + 7) / 8;
+    const int64_t cap = max_dirty_groups(cols, num_fp);
+    for (int64_t g = threadIdx.x; g < groups; g += blockDim.x) {
+      uint32_t before = 0, slot = 0;
+      for (int64_t w = 0; w < (g >> 2); ++w) {
+        before += __popc(mask[w]);
+        slot += nonzero_bytes(mask[w], 4);
+      }
+      const uint32_t word = mask[g >> 2];
+      const int sh = static_cast<int>(g & 3) * 8;
+      before += __popc(word & ((1u << sh) - 1u));
+      slot += nonzero_bytes(word, static_cast<int>(g & 3));
+      const uint32_t mb = (word >> sh) & 0xFFu;
+      const uint32_t dest = static_cast<uint32_t>(g * 8) - before;
+      if (mb == 0u) {
+        grp[g] = dest << 8;
+      } else {
+        grp[g] = (slot << 8) | mb;
+        if (slot < cap) dirty[slot] = (dest << 8) | mb;
+      }
+    }
   }
 }
 
@@ -107,6 +183,27 @@ struct RowQuant {
     slow = !(range <= max_finite) || !(scale >= 1e-20f);
   }
 
+  // same with the path chosen at compile time (callers branch once per row on `slow`)
+  template <bool SLOW>
+  __device__ __forceinline__ float quotient_t(uint16_t xbits) const {
+    float d;
+    if constexpr (BF16) {
+      d = round_storage<true>(to_f32<true>(xbits) - zero);
+    } else {
+      const _Float16 dh = __builtin_bit_cast(_Float16, xbits) - static_cast<_Float16>(zero);
+      d = static_cast<float>(dh);
+    }
+    float q;
+    if constexpr (SLOW) {
+      q = d / scale;
+    } else {
+      q = d * rcp;
+      const float e = __builtin_fmaf(-q, scale, d);
+      q = __builtin_fmaf(e, rcp, q);
+    }
+    return round_storage<BF16>(q);
+  }
+
   // storage(storage(x - zero) / scale) as fp32
   __device__ __forceinline__ float quotient(uint16_t xbits) const {
     float d;
@@ -135,12 +232,11 @@ struct RowQuant {
 };
 
 template <typename IdxT, int BITS, bool BF16>
-__global__ __launch_bounds__(kThreads) void asym_quantize_kernel(
+__device__ __forceinline__ void gather_rows(
     const uint16_t *__restrict__ x, int64_t rows, int64_t cols, const IdxT *__restrict__ src_col,
     const IdxT *__restrict__ fp_col, const uint32_t *__restrict__ mask, int64_t num_int, int64_t num_fp,
-    uint8_t *__restrict__ dst, uint16_t *__restrict__ meta, uint16_t *__restrict__ fp_x, int vec_ok) {
-  extern __shared__ __align__(16) uint16_t row_s[];
-  __shared__ float red[8];
+    uint8_t *__restrict__ dst, uint16_t *__restrict__ meta, uint16_t *__restrict__ fp_x, int vec_ok,
+    uint16_t *row_s, float *red) {
   const int tid = threadIdx.x;
   constexpr float kMaxQ = static_cast<float>((1 << BITS) - 1);
   constexpr uint32_t kFlip = BITS == 4 ? 0x88u : 0x8080u;
@@ -212,6 +308,299 @@ __global__ __launch_bounds__(kThreads) void asym_quantize_kernel(
     uint16_t *frow = fp_x + row * num_fp;
     for (int64_t f = tid; f < num_fp; f += kThreads) frow[f] = row_s[fp_col[f]];
     __syncthreads();  // the next row overwrites row_s
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// Streaming path (ascending int_indices, the layout MixedQLinear.from_float produces).
+//
+// Works in source order, so nothing is gathered.  Every lane keeps NV 16-byte groups of the row
+// in registers (the next row's groups are already in flight while the current row is processed).
+// All lanes run the same branch-free code on their groups as if they were clean: packed fp16
+// min/max (a dirty group's contribution is replaced by the neutral element with one select),
+// then 8 codes per group, written as 8 bytes to the group's destination position in an LDS byte
+// buffer (only that write is predicated).  Dirty groups are also copied raw to LDS, indexed by
+// their slot, and handled by lanes 0..ndirty-1, one group each, with per-element masking: that
+// keeps the expensive masked code off the all-lanes path, where a divergent branch would make
+// every wave pay for both sides.  A last pass reads 16 code bytes per lane, packs them to
+// nibbles (int4) and writes 8 or 16 contiguous bytes per lane; outliers are read from the row
+// early in the iteration and stored at its end.
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+typedef float f2 __attribute__((ext_vector_type(2)));
+
+struct __attribute__((packed, aligned(1))) Bytes8 {
+  uint32_t a, b;
+};
+
+// Codes of the two halves of word w in bytes 0 and 2 of the result (other bytes: don't care).
+// The code is (level - 2^(BITS-1)) mod 256; for BITS == 4 only its low nibble is meaningful.
+template <int BITS, bool BF16, bool SLOW>
+__device__ __forceinline__ uint32_t code_pair(uint32_t w, const RowQuant<BF16> &rq) {
+  constexpr float kMaxQ = static_cast<float>((1 << BITS) - 1);
+  constexpr uint32_t kBias = 1u << (BITS - 1);
+  if constexpr (BF16) {
+    const uint32_t a = RowQuant<true>::to_level(rq.template quotient_t<SLOW>(static_cast<uint16_t>(w & 0xFFFFu)), kMaxQ);
+    const uint32_t b = RowQuant<true>::to_level(rq.template quotient_t<SLOW>(static_cast<uint16_t>(w >> 16)), kMaxQ);
+    return (a + kBias) | ((b + kBias) << 16);
+  } else {
+    const h2 x = __builtin_bit_cast(h2, w);
+    const _Float16 zh = static_cast<_Float16>(rq.zero);
+    const h2 d = x - h2{zh, zh};  // storage(x - zero), both halves
+    h2 t;                         // storage(d / scale), or a value that rounds to the same level
+    if constexpr (SLOW) {
+      const f2 q = f2{static_cast<float>(d.x) / rq.scale, static_cast<float>(d.y) / rq.scale};
+      t = __builtin_convertvector(q, h2);
+    } else {
+      // fp16(f32(d) * rcp) for both halves: the mixed-precision FMA reads an fp16 half and an fp32
+      // register and writes an fp16 half, so the quotient costs one instruction per element
+      uint32_t tb;
+      asm("v_fma_mixlo_f16 %0, %1, %2, 0 op_sel_hi:[1,0,0]\n\t"
+          "v_fma_mixhi_f16 %0, %1, %2, 0 op_sel:[1,0,0] op_sel_hi:[1,0,0]"
+          : "=&v"(tb)
+          : "v"(__builtin_bit_cast(uint32_t, d)), "v"(rq.rcp));
+      t = __builtin_bit_cast(h2, tb);
+    }
+    // clamp to [0, maxq] (NaN -> 0), then + 1024 + 2^(BITS-1): in [1024, 2048) one fp16 ulp is 1, so the
+    // sum is round-to-nearest-even(t) + 2^(BITS-1) and that integer sits in the low mantissa bits
+    const _Float16 mq = static_cast<_Float16>(kMaxQ);
+    t = __builtin_elementwise_min(__builtin_elementwise_max(t, h2{0, 0}), h2{mq, mq});
+    constexpr _Float16 magic = static_cast<_Float16>(1024 + (1 << (BITS - 1)));
+    t = t + h2{magic, magic};
+    return __builtin_bit_cast(uint32_t, t);
+  }
+}
+
+// 8 codes of one group as 8 bytes
+template <int BITS, bool BF16, bool SLOW>
+__device__ __forceinline__ uint2 group_codes(const uint4 &v, const RowQuant<BF16> &rq) {
+  const uint32_t p0 = code_pair<BITS, BF16, SLOW>(v.x, rq), p1 = code_pair<BITS, BF16, SLOW>(v.y, rq);
+  const uint32_t p2 = code_pair<BITS, BF16, SLOW>(v.z, rq), p3 = code_pair<BITS, BF16, SLOW>(v.w, rq);
+  uint2 c;
+  c.x = __builtin_amdgcn_perm(p1, p0, 0x06040200u);  // bytes 0, 2 of p0 then bytes 0, 2 of p1
+  c.y = __builtin_amdgcn_perm(p3, p2, 0x06040200u);
+  if constexpr (BITS == 4) {
+    c.x &= 0x0F0F0F0Fu;
+    c.y &= 0x0F0F0F0Fu;
+  }
+  return c;
+}
+
+template <int BITS, bool BF16, int NV>
+__device__ __forceinline__ void stream_rows(const uint16_t *__restrict__ x, int64_t rows, int64_t cols,
+                                            const uint32_t *__restrict__ grp, const uint32_t *__restrict__ dirty,
+                                            int ndirty, const uint16_t *__restrict__ fp_col, int64_t num_int,
+                                            int64_t num_fp, uint8_t *__restrict__ dst, uint16_t *__restrict__ meta,
+                                            uint16_t *__restrict__ fp_x, uint8_t *codes_s, uint4 *dirty_s,
+                                            float *red, int vec_out) {
+  const int tid = threadIdx.x;
+  const int nvec = static_cast<int>(cols >> 3);
+  const float inf = __builtin_inff();
+  uint32_t g[NV];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) g[i] = tid + i * kThreads < nvec ? grp[tid + i * kThreads] : 0xFFFFFFFFu;
+  const uint32_t my_dirty = tid < ndirty ? dirty[tid] : 0u;
+  const uint32_t my_fp_col = tid < num_fp ? fp_col[tid] : 0u;
+
+  auto load_row = [&](int64_t row, uint4 (&v)[NV]) {
+    const uint4 *xv = reinterpret_cast<const uint4 *>(x + row * cols);
+#pragma unroll
+    for (int i = 0; i < NV; ++i)
+      if (tid + i * kThreads < nvec) v[i] = xv[tid + i * kThreads];
+  };
+
+  // per-element masked min/max of one dirty group
+  auto dirty_minmax = [&](const uint4 &v, uint32_t mb, float &mn, float &mx) {
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float f = to_f32<BF16>(static_cast<uint16_t>(w[e >> 1] >> (16 * (e & 1))));
+      const bool out = (mb >> e) & 1u;
+      mn = fminf(mn, out ? inf : f);
+      mx = fmaxf(mx, out ? -inf : f);
+    }
+  };
+  // codes of one dirty group, outliers squeezed out
+  auto dirty_codes = [&](const uint4 &v, uint32_t info, const RowQuant<BF16> &rq, auto slow_c) {
+    constexpr bool SLOW = decltype(slow_c)::value;
+    const uint32_t mb = info & 0xFFu;
+    const uint2 c = group_codes<BITS, BF16, SLOW>(v, rq);
+    uint8_t *out = codes_s + (info >> 8);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      if (!((mb >> e) & 1u))
+        out[e - __popc(mb & ((1u << e) - 1u))] = static_cast<uint8_t>((e < 4 ? c.x : c.y) >> (8 * (e & 3)));
+    }
+  };
+
+  // one row; `cur` holds its groups, `parity` alternates so that two sets of reduction slots are used
+  auto process = [&](int64_t row, const uint4 (&cur)[NV], int parity) {
+    const uint16_t *xr = x + row * cols;
+    const uint16_t my_fp = tid < num_fp ? xr[my_fp_col] : uint16_t(0);
+
+    // ---- all lanes: min / max as if every group were clean; dirty groups go to LDS
+    float mn = inf, mx = -inf;
+    if constexpr (!BF16) {
+      const h2 pinf = h2{static_cast<_Float16>(inf), static_cast<_Float16>(inf)};
+      h2 pmn = pinf, pmx = -pinf;
+#pragma unroll
+      for (int i = 0; i < NV; ++i) {
+        const h2 a = __builtin_bit_cast(h2, cur[i].x), b = __builtin_bit_cast(h2, cur[i].y);
+        const h2 c = __builtin_bit_cast(h2, cur[i].z), d = __builtin_bit_cast(h2, cur[i].w);
+        const h2 lo = __builtin_elementwise_min(__builtin_elementwise_min(a, b), __builtin_elementwise_min(c, d));
+        const h2 hi = __builtin_elementwise_max(__builtin_elementwise_max(a, b), __builtin_elementwise_max(c, d));
+        const bool clean = (g[i] & 0xFFu) == 0u;
+        pmn = __builtin_elementwise_min(pmn, clean ? lo : pinf);
+        pmx = __builtin_elementwise_max(pmx, clean ? hi : -pinf);
+      }
+      mn = fminf(static_cast<float>(pmn.x), static_cast<float>(pmn.y));
+      mx = fmaxf(static_cast<float>(pmx.x), static_cast<float>(pmx.y));
+    } else {
+#pragma unroll
+      for (int i = 0; i < NV; ++i) {
+        const uint32_t w[4] = {cur[i].x, cur[i].y, cur[i].z, cur[i].w};
+        float lo = inf, hi = -inf;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          const float f0 = __uint_as_float(w[k] << 16), f1 = __uint_as_float(w[k] & 0xFFFF0000u);
+          lo = fminf(lo, fminf(f0, f1));
+          hi = fmaxf(hi, fmaxf(f0, f1));
+        }
+        const bool clean = (g[i] & 0xFFu) == 0u;
+        mn = fminf(mn, clean ? lo : inf);
+        mx = fmaxf(mx, clean ? hi : -inf);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      if ((g[i] & 0xFFu) != 0u && tid + i * kThreads < nvec) dirty_s[g[i] >> 8] = cur[i];
+    }
+    __syncthreads();  // dirty_s complete; also: the previous row's pack pass has finished reading codes_s
+
+    // ---- lanes 0 .. ndirty-1: one dirty group each
+    uint4 dv = make_uint4(0, 0, 0, 0);
+    if (tid < ndirty) {
+      dv = dirty_s[tid];
+      dirty_minmax(dv, my_dirty & 0xFFu, mn, mx);
+    }
+    for (int j = tid + kThreads; j < ndirty; j += kThreads) dirty_minmax(dirty_s[j], dirty[j] & 0xFFu, mn, mx);
+
+    mn = wave_min(mn);
+    mx = wave_max(mx);
+    float *r = red + parity * 8;  // two sets: the next row's writes cannot overtake this row's reads
+    if ((tid & 63) == 0) {
+      r[tid >> 6] = mn;
+      r[4 + (tid >> 6)] = mx;
+    }
+    __syncthreads();
+    mn = fminf(fminf(r[0], r[1]), fminf(r[2], r[3]));
+    mx = fmaxf(fmaxf(r[4], r[5]), fmaxf(r[6], r[7]));
+
+    RowQuant<BF16> rq;
+    rq.init(mn, mx, BITS);
+    if (tid == 0) {
+      meta[2 * row] = rq.scale_bits;
+      meta[2 * row + 1] = rq.zero_bits;
+    }
+
+    // ---- quantise in source order, 8 code bytes per clean group to their destination position
+    auto quantise = [&](auto slow_c) {
+      constexpr bool SLOW = decltype(slow_c)::value;
+#pragma unroll
+      for (int i = 0; i < NV; ++i) {
+        const uint2 c = group_codes<BITS, BF16, SLOW>(cur[i], rq);
+        if ((g[i] & 0xFFu) == 0u) *reinterpret_cast<Bytes8 *>(codes_s + (g[i] >> 8)) = Bytes8{c.x, c.y};
+      }
+      if (tid < ndirty) dirty_codes(dv, my_dirty, rq, slow_c);
+      for (int j = tid + kThreads; j < ndirty; j += kThreads) dirty_codes(dirty_s[j], dirty[j], rq, slow_c);
+    };
+    if (__builtin_amdgcn_readfirstlane(rq.slow ? 1 : 0)) {
+      quantise(std::true_type{});
+    } else {
+      quantise(std::false_type{});
+    }
+    __syncthreads();
+
+    // ---- pack pass: 16 code bytes per lane -> 8 bytes (int4) or 16 bytes (int8)
+    const int units = static_cast<int>((num_int + 15) >> 4);
+    for (int u = tid; u < units; u += kThreads) {
+      const uint4 c = *reinterpret_cast<const uint4 *>(codes_s + u * 16);
+      const int valid = static_cast<int>(num_int) - u * 16;  // codes of this unit that exist (16 except at the tail)
+      if constexpr (BITS == 4) {
+        // byte pairs (c0, c1) -> c0 | c1 << 4: t = w | w >> 4 leaves them in bytes 0 and 2
+        const uint32_t t0 = c.x | (c.x >> 4), t1 = c.y | (c.y >> 4), t2 = c.z | (c.z >> 4), t3 = c.w | (c.w >> 4);
+        const uint2 packed = make_uint2(__builtin_amdgcn_perm(t1, t0, 0x06040200u),
+                                        __builtin_amdgcn_perm(t3, t2, 0x06040200u));
+        uint8_t *drow = dst + row * (num_int >> 1) + u * 8;
+        if (valid >= 16 && vec_out) {
+          *reinterpret_cast<uint2 *>(drow) = packed;
+        } else {
+          for (int b = 0; b < (valid < 16 ? valid : 16) / 2; ++b)
+            drow[b] = static_cast<uint8_t>((b < 4 ? packed.x : packed.y) >> (8 * (b & 3)));
+        }
+      } else {
+        uint8_t *drow = dst + row * num_int + u * 16;
+        if (valid >= 16 && vec_out) {
+          *reinterpret_cast<uint4 *>(drow) = c;
+        } else {
+          for (int b = 0; b < (valid < 16 ? valid : 16); ++b) {
+            const uint32_t w = b < 4 ? c.x : (b < 8 ? c.y : (b < 12 ? c.z : c.w));
+            drow[b] = static_cast<uint8_t>(w >> (8 * (b & 3)));
+          }
+        }
+      }
+    }
+    // ---- outliers, in the caller's order
+    if (tid < num_fp) fp_x[row * num_fp + tid] = my_fp;
+    for (int64_t f = tid + kThreads; f < num_fp; f += kThreads) fp_x[row * num_fp + f] = xr[fp_col[f]];
+  };
+
+  // two register sets alternate: while one row is processed the next one is in flight
+  uint4 buf_a[NV], buf_b[NV];
+  const int64_t stride = gridDim.x;
+  int64_t row = blockIdx.x;
+  if (row < rows) load_row(row, buf_a);
+  while (row < rows) {
+    if (row + stride < rows) load_row(row + stride, buf_b);
+    process(row, buf_a, 0);
+    row += stride;
+    if (row >= rows) break;
+    if (row + stride < rows) load_row(row + stride, buf_a);
+    process(row, buf_b, 1);
+    row += stride;
+  }
+}
+
+template <typename IdxT, int BITS, bool BF16>
+__global__ __launch_bounds__(kThreads) void asym_quantize_kernel(
+    const uint16_t *__restrict__ x, int64_t rows, int64_t cols, const IdxT *__restrict__ src_col,
+    const IdxT *__restrict__ fp_col, const uint32_t *__restrict__ mask, int64_t num_int, int64_t num_fp,
+    uint8_t *__restrict__ dst, uint16_t *__restrict__ meta, uint16_t *__restrict__ fp_x, int vec_ok) {
+  extern __shared__ __align__(16) uint16_t row_s[];
+  __shared__ float red[8];
+  gather_rows<IdxT, BITS, BF16>(x, rows, cols, src_col, fp_col, mask, num_int, num_fp, dst, meta, fp_x, vec_ok, row_s,
+                                red);
+}
+
+// Shapes that may stream: the column map's flag (known only on the device) picks the path.
+// Dynamic LDS: max(row bytes for the gather path, code bytes + 16 bytes per possible dirty group).
+template <typename IdxT, int BITS, bool BF16, int NV>
+__global__ __launch_bounds__(kThreads) void asym_quantize_stream_kernel(
+    const uint16_t *__restrict__ x, int64_t rows, int64_t cols, const IdxT *__restrict__ src_col,
+    const IdxT *__restrict__ fp_col, const uint32_t *__restrict__ mask, const uint32_t *__restrict__ grp,
+    const uint32_t *__restrict__ dirty, const uint32_t *__restrict__ flags, int64_t num_int, int64_t num_fp,
+    uint8_t *__restrict__ dst, uint16_t *__restrict__ meta, uint16_t *__restrict__ fp_x, int vec_out) {
+  static_assert(sizeof(IdxT) == 2, "streaming needs cols <= 32768");
+  extern __shared__ __align__(16) uint16_t row_s[];
+  __shared__ float red[16];
+  if (flags[0] & 1u) {
+    uint8_t *codes_s = reinterpret_cast<uint8_t *>(row_s);
+    uint4 *dirty_s = reinterpret_cast<uint4 *>(codes_s + align16(num_int));
+    stream_rows<BITS, BF16, NV>(x, rows, cols, grp, dirty, static_cast<int>(flags[1]),
+                                reinterpret_cast<const uint16_t *>(fp_col), num_int, num_fp, dst, meta, fp_x,
+                                codes_s, dirty_s, red, vec_out);
+  } else {
+    gather_rows<IdxT, BITS, BF16>(x, rows, cols, src_col, fp_col, mask, num_int, num_fp, dst, meta, fp_x, 1, row_s,
+                                  red);
   }
 }
 
@@ -348,12 +737,47 @@ int grid_for(int64_t work_items, int64_t per_block) {
 
 constexpr int64_t kMaxLdsRowBytes = 128 * 1024;  // of the 160 KB per CU
 
+template <typename IdxT, int BITS, bool BF16, int NV>
+int launch_stream(const void *x, int64_t rows, int64_t cols, const uint8_t *cm, const ColmapLayout &l, int64_t num_int,
+                  int64_t num_fp, void *dst, void *meta, void *fp_x, hipStream_t st) {
+  auto kern = asym_quantize_stream_kernel<IdxT, BITS, BF16, NV>;
+  const int64_t lds_stream = align16(num_int) + 16 * max_dirty_groups(cols, num_fp);
+  const int64_t lds = lds_stream > align16(cols * 2) ? lds_stream : align16(cols * 2);
+  if (lds > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+    if (e != hipSuccess) {
+      set_last_hip_error(e);
+      return QUIK_ERR_LAUNCH;
+    }
+  }
+  // a few rows per workgroup so that the next row's loads overlap the current row's arithmetic
+  const int64_t per_cu = lds <= 20 * 1024 ? 4 : (lds <= 40 * 1024 ? 3 : 2);
+  const int grid = static_cast<int>(rows < 256 * per_cu ? rows : 256 * per_cu);
+  const int vec_out = num_int % 16 == 0 && reinterpret_cast<uintptr_t>(dst) % 16 == 0;
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), static_cast<size_t>(lds), st,
+                     static_cast<const uint16_t *>(x), rows, cols, reinterpret_cast<const IdxT *>(cm),
+                     reinterpret_cast<const IdxT *>(cm + l.off_fp), reinterpret_cast<const uint32_t *>(cm + l.off_mask),
+                     reinterpret_cast<const uint32_t *>(cm + l.off_grp),
+                     reinterpret_cast<const uint32_t *>(cm + l.off_dirty),
+                     reinterpret_cast<const uint32_t *>(cm + l.off_flags), num_int, num_fp,
+                     static_cast<uint8_t *>(dst), static_cast<uint16_t *>(meta), static_cast<uint16_t *>(fp_x), vec_out);
+  return check_launch();
+}
+
 template <typename IdxT, int BITS, bool BF16>
 int launch_asym(const void *x, int64_t rows, int64_t cols, const uint8_t *cm, const ColmapLayout &l, int64_t num_int,
                 int64_t num_fp, void *dst, void *meta, void *fp_x, hipStream_t st) {
   const IdxT *src_col = reinterpret_cast<const IdxT *>(cm);
   const IdxT *fp_col = reinterpret_cast<const IdxT *>(cm + l.off_fp);
   const uint32_t *mask = reinterpret_cast<const uint32_t *>(cm + l.off_mask);
+  if constexpr (sizeof(IdxT) == 2) if (cols <= kStreamMaxCols && cols % 8 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0) {
+    const int64_t per_thread = (cols / 8 + kThreads - 1) / kThreads;
+    if (per_thread <= 2) return launch_stream<IdxT, BITS, BF16, 2>(x, rows, cols, cm, l, num_int, num_fp, dst, meta, fp_x, st);
+    if (per_thread <= 4) return launch_stream<IdxT, BITS, BF16, 4>(x, rows, cols, cm, l, num_int, num_fp, dst, meta, fp_x, st);
+    if (per_thread <= 8) return launch_stream<IdxT, BITS, BF16, 8>(x, rows, cols, cm, l, num_int, num_fp, dst, meta, fp_x, st);
+    return launch_stream<IdxT, BITS, BF16, 16>(x, rows, cols, cm, l, num_int, num_fp, dst, meta, fp_x, st);
+  }
   const int grid = static_cast<int>(rows < 65535 * 8 ? rows : 65535 * 8);
   const int64_t lds = align16(cols * 2);
   if (lds <= kMaxLdsRowBytes) {
@@ -400,11 +824,13 @@ extern "C" int quik_colmap_build(const int64_t *int_indices, int64_t num_int, co
   if (l.idx16) {
     hipLaunchKernelGGL(colmap_build_kernel<uint16_t>, dim3(1), dim3(1024), 0, as_stream(stream), int_indices,
                        num_int, fp_indices, num_fp, cols, reinterpret_cast<uint16_t *>(cm),
-                       reinterpret_cast<uint16_t *>(cm + l.off_fp), mask);
+                       reinterpret_cast<uint16_t *>(cm + l.off_fp), mask, reinterpret_cast<uint32_t *>(cm + l.off_grp),
+                       reinterpret_cast<uint32_t *>(cm + l.off_dirty), reinterpret_cast<uint32_t *>(cm + l.off_flags));
   } else {
     hipLaunchKernelGGL(colmap_build_kernel<uint32_t>, dim3(1), dim3(1024), 0, as_stream(stream), int_indices,
                        num_int, fp_indices, num_fp, cols, reinterpret_cast<uint32_t *>(cm),
-                       reinterpret_cast<uint32_t *>(cm + l.off_fp), mask);
+                       reinterpret_cast<uint32_t *>(cm + l.off_fp), mask, reinterpret_cast<uint32_t *>(cm + l.off_grp),
+                       reinterpret_cast<uint32_t *>(cm + l.off_dirty), reinterpret_cast<uint32_t *>(cm + l.off_flags));
   }
   return check_launch();
 }

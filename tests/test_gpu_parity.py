@@ -83,6 +83,9 @@ QCASES = [
     (17, 100, 10, "x50", True),        # row length not a multiple of 8: scalar load path
     (40, 384, 32, "uniform", True),    # int_indices in arbitrary order
     (12, 2050, 2, "x50", False),
+    (20, 520, 6, "x50", False),        # K = 514: not a multiple of 16, scalar tail of the packed output
+    (300, 8192, 256, "x50", False),    # several rows per workgroup (register prefetch of the next row)
+    (70, 28672, 256, "student", False),
 ]
 
 
@@ -184,6 +187,36 @@ def test_fast_quotient_path_exhaustive_rows():
         dst, meta, _ = qo.asym_quantize(x, ii, fi, bits)
         assert np.array_equal(_bits(m), meta.view(np.uint16))
         assert np.array_equal(q.cpu().numpy(), dst)
+
+
+def test_streaming_quotient_full_domain_on_device():
+    """Every fp16 scale the row kernel can produce against every numerator: one row per row maximum
+    hi in [2^-14, 65504) holding all fp16 values 0 .. hi, zero = 0, so d = x and the scale is
+    fp16(hi / maxq).  Expected codes come from IEEE float64 division on the device (the quotient of
+    two fp16 numbers rounds to fp16 the same way from float64 as from the exact value); the 47-row
+    test above ties the same arithmetic to the oracle."""
+    import quik
+    n_in = 0x7C00
+    ii = torch.arange(n_in, device=DEV)
+    fi = torch.zeros(0, dtype=torch.int64, device=DEV)
+    cols = torch.arange(n_in, device=DEV, dtype=torch.int32)
+    his = torch.arange(0x0400, 0x7BFF, device=DEV, dtype=torch.int32)
+    for bits in (4, 8):
+        maxq = float(2 ** bits - 1)
+        for lo in range(0, his.numel(), 4096):
+            hi = his[lo:lo + 4096]
+            xb = torch.where(cols[None, :] <= hi[:, None], cols[None, :], torch.zeros_like(cols[None, :]))
+            x = xb.to(torch.int16).view(torch.float16)
+            q, m, _ = quik.asymmetric.quantize(x, ii, fi, bits)
+            scale = (hi.to(torch.int16).view(torch.float16).float() / maxq).clamp_min(1e-6).half()
+            assert torch.equal(m[0::2], scale) and not m[1::2].any()
+            t = (x.double() / scale.double()[:, None]).half()
+            lvl = t.float().clamp(0, maxq).round().to(torch.int32) - 2 ** (bits - 1)
+            if bits == 4:
+                want = ((lvl[:, 0::2] & 0xF) | ((lvl[:, 1::2] & 0xF) << 4)).to(torch.uint8)
+            else:
+                want = lvl.to(torch.int8)
+            assert torch.equal(q, want), (bits, lo)
 
 
 def test_asym_quantize_argument_errors():
