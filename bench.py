@@ -101,6 +101,9 @@ def main():
     ap.add_argument("--workload", default="llama2-70b.gate_proj", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--unfused", action="store_true", help="run the reference's three-op sequence instead")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="run only plain device-to-device copies of a 256 MiB buffer (known traffic: 256 MiB read, "
+                         "256 MiB written per launch) to scale the FETCH_SIZE / WRITE_SIZE counters")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU only; run with --gpus 1 (no multi-GPU path exists)",
@@ -114,6 +117,16 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+
+    if args.copy_calibration:
+        src = torch.randn(128 * 1024 * 1024, device=dev).half()       # 256 MiB
+        dst = torch.empty_like(src)
+        for _ in range(max(args.steps, 1)):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_calibration": True, "bytes_read_per_launch": src.numel() * 2,
+                          "bytes_written_per_launch": src.numel() * 2, "launches": max(args.steps, 1)}))
+        return
 
     name = args.workload
     M, n_in, N, F, bits = WORKLOADS[name]

@@ -35,19 +35,21 @@ constexpr int kThreads = 256;
 
 // ---------------------------------------------------------------------------------------
 // column map layout: [src_col: num_int idx][fp_col: num_fp idx][mask: ceil(cols/32) u32]
-//                    [grp: ceil(cols/8) u32][dirty: min(num_fp, ceil(cols/8)) u32][flags: 4 u32]
+//                    [grp: ceil(cols/8) u32][dirty: min(num_fp, ceil(cols/8)) u32][fp_slot: num_fp u16]
+//                    [flags: 4 u32]
 // idx is uint16_t when cols <= 65536, else uint32_t.  Section offsets are 16-byte aligned.
 // A "group" is 8 consecutive source columns (one 16-byte load).  A group without outliers is
 // clean, one with outliers is dirty; dirty groups are numbered in ascending order (slots).
 //   grp[g]   clean: (destination column of the group's first element) << 8
 //            dirty: (slot << 8) | mask byte (bit e set = column 8g+e is an outlier)
 //   dirty[s] (destination column of the group's first non-outlier element) << 8 | mask byte
+//   fp_slot[f] = 8 * slot + e: where outlier f sits when the dirty groups are laid out by slot
 //   flags[0] bit 0: int_indices ascending, the two lists partition the columns and the shape
 //            fits the streaming kernel;  flags[1] = number of dirty groups.
-// grp and dirty exist only when cols <= kStreamMaxCols.
+// grp, dirty and fp_slot exist only when cols <= kStreamMaxCols.
 struct ColmapLayout {
   bool idx16;
-  int64_t off_fp, off_mask, off_grp, off_dirty, off_flags, bytes;
+  int64_t off_fp, off_mask, off_grp, off_dirty, off_slot, off_flags, bytes;
 };
 
 __host__ __device__ inline int64_t align16(int64_t v) { return (v + 15) & ~int64_t(15); }
@@ -70,7 +72,8 @@ __host__ __device__ inline ColmapLayout colmap_layout(int64_t cols, int64_t num_
   l.off_grp = l.off_mask + align16(((cols + 31) / 32) * 4);
   const bool stream = cols <= kStreamMaxCols;
   l.off_dirty = l.off_grp + align16(stream ? ((cols + 7) / 8) * 4 : 0);
-  l.off_flags = l.off_dirty + align16(stream ? max_dirty_groups(cols, num_fp) * 4 : 0);
+  l.off_slot = l.off_dirty + align16(stream ? max_dirty_groups(cols, num_fp) * 4 : 0);
+  l.off_flags = l.off_slot + align16(stream ? num_fp * 2 : 0);
   l.bytes = l.off_flags + 16;
   return l;
 }
@@ -88,6 +91,7 @@ __global__ __launch_bounds__(1024) void colmap_build_kernel(const int64_t *__res
                                                             int64_t cols, IdxT *__restrict__ src_col,
                                                             IdxT *__restrict__ fp_col, uint32_t *__restrict__ mask,
                                                             uint32_t *__restrict__ grp, uint32_t *__restrict__ dirty,
+                                                            uint16_t *__restrict__ fp_slot,
                                                             uint32_t *__restrict__ flags) {
   // single workgroup: the mask is cleared before any bit is set
   __shared__ int ascending;
@@ -143,23 +147,37 @@ __global__ __launch_bounds__(1024) void colmap_build_kernel(const int64_t *__res
         if (slot < cap) dirty[slot] = (dest << 8) | mb;
       }
     }
+    __syncthreads();
+    for (int64_t j = threadIdx.x; j < num_fp; j += blockDim.x) {
+      const int64_t c = static_cast<int64_t>(fp_col[j]);
+      const uint32_t slot = grp[c >> 3] >> 8;
+      fp_slot[j] = static_cast<uint16_t>(slot < cap ? slot * 8 + (c & 7) : 0);
+    }
   }
 }
 
 // ---------------------------------------------------------------------------------------
 // block-wide (min, max) reduction; every thread returns the result
+template <int TPR = kThreads>
 __device__ __forceinline__ void block_minmax(float &mn, float &mx, float *red) {
   mn = wave_min(mn);
   mx = wave_max(mx);
-  const int wave = threadIdx.x >> 6;
-  __syncthreads();  // protects `red` from the previous use
-  if ((threadIdx.x & 63) == 0) {
-    red[wave] = mn;
-    red[4 + wave] = mx;
+  __syncthreads();  // protects `red` from the previous use (and orders the callers' LDS row writes)
+  if constexpr (TPR > 64) {
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) {
+      red[wave] = mn;
+      red[4 + wave] = mx;
+    }
+    __syncthreads();
+    mn = red[0];
+    mx = red[4];
+#pragma unroll
+    for (int w = 1; w < TPR / 64; ++w) {
+      mn = fminf(mn, red[w]);
+      mx = fmaxf(mx, red[4 + w]);
+    }
   }
-  __syncthreads();
-  mn = fminf(fminf(red[0], red[1]), fminf(red[2], red[3]));
-  mx = fmaxf(fmaxf(red[4], red[5]), fmaxf(red[6], red[7]));
 }
 
 template <bool BF16>
@@ -231,7 +249,7 @@ struct RowQuant {
   }
 };
 
-template <typename IdxT, int BITS, bool BF16>
+template <typename IdxT, int BITS, bool BF16, int TPR = kThreads>
 __device__ __forceinline__ void gather_rows(
     const uint16_t *__restrict__ x, int64_t rows, int64_t cols, const IdxT *__restrict__ src_col,
     const IdxT *__restrict__ fp_col, const uint32_t *__restrict__ mask, int64_t num_int, int64_t num_fp,
@@ -248,7 +266,7 @@ __device__ __forceinline__ void gather_rows(
       const uint4 *xv = reinterpret_cast<const uint4 *>(xr);
       uint4 *sv = reinterpret_cast<uint4 *>(row_s);
       const int64_t nvec = cols >> 3;
-      for (int64_t c8 = tid; c8 < nvec; c8 += kThreads) {
+      for (int64_t c8 = tid; c8 < nvec; c8 += TPR) {
         const uint4 v = xv[c8];
         sv[c8] = v;
         uint32_t mb = (mask[c8 >> 2] >> ((c8 & 3) * 8)) & 0xFFu;
@@ -268,7 +286,7 @@ __device__ __forceinline__ void gather_rows(
         }
       }
     } else {
-      for (int64_t c = tid; c < cols; c += kThreads) {
+      for (int64_t c = tid; c < cols; c += TPR) {
         const uint16_t v = xr[c];
         row_s[c] = v;
         if (!((mask[c >> 5] >> (c & 31)) & 1u)) {
@@ -278,7 +296,7 @@ __device__ __forceinline__ void gather_rows(
         }
       }
     }
-    block_minmax(mn, mx, red);  // also orders the LDS row writes before the gathers below
+    block_minmax<TPR>(mn, mx, red);  // also orders the LDS row writes before the gathers below
 
     RowQuant<BF16> rq;
     rq.init(mn, mx, BITS);
@@ -290,7 +308,7 @@ __device__ __forceinline__ void gather_rows(
     const int64_t pairs = num_int >> 1;
     if constexpr (BITS == 4) {
       uint8_t *drow = dst + row * pairs;
-      for (int64_t p = tid; p < pairs; p += kThreads) {
+      for (int64_t p = tid; p < pairs; p += TPR) {
         const IdxT c0 = src_col[2 * p], c1 = src_col[2 * p + 1];
         const uint32_t v0 = RowQuant<BF16>::to_level(rq.quotient(row_s[c0]), kMaxQ);
         const uint32_t v1 = RowQuant<BF16>::to_level(rq.quotient(row_s[c1]), kMaxQ);
@@ -298,7 +316,7 @@ __device__ __forceinline__ void gather_rows(
       }
     } else {
       uint16_t *drow = reinterpret_cast<uint16_t *>(dst + row * num_int);
-      for (int64_t p = tid; p < pairs; p += kThreads) {
+      for (int64_t p = tid; p < pairs; p += TPR) {
         const IdxT c0 = src_col[2 * p], c1 = src_col[2 * p + 1];
         const uint32_t v0 = RowQuant<BF16>::to_level(rq.quotient(row_s[c0]), kMaxQ);
         const uint32_t v1 = RowQuant<BF16>::to_level(rq.quotient(row_s[c1]), kMaxQ);
@@ -306,7 +324,7 @@ __device__ __forceinline__ void gather_rows(
       }
     }
     uint16_t *frow = fp_x + row * num_fp;
-    for (int64_t f = tid; f < num_fp; f += kThreads) frow[f] = row_s[fp_col[f]];
+    for (int64_t f = tid; f < num_fp; f += TPR) frow[f] = row_s[fp_col[f]];
     __syncthreads();  // the next row overwrites row_s
   }
 }
@@ -315,7 +333,7 @@ __device__ __forceinline__ void gather_rows(
 // Streaming path (ascending int_indices, the layout MixedQLinear.from_float produces).
 //
 // Works in source order, so nothing is gathered.  Every lane keeps NV 16-byte groups of the row
-// in registers (the next row's groups are already in flight while the current row is processed).
+// in registers.
 // All lanes run the same branch-free code on their groups as if they were clean: packed fp16
 // min/max (a dirty group's contribution is replaced by the neutral element with one select),
 // then 8 codes per group, written as 8 bytes to the group's destination position in an LDS byte
@@ -385,10 +403,12 @@ __device__ __forceinline__ uint2 group_codes(const uint4 &v, const RowQuant<BF16
   return c;
 }
 
-template <int BITS, bool BF16, int NV>
+// One row is handled by the TPR threads of one workgroup (a multiple of 64, at most 256; the
+// launches use 256), which walks over rows blockIdx.x, blockIdx.x + gridDim.x, ...
+template <int BITS, bool BF16, int NV, int TPR>
 __device__ __forceinline__ void stream_rows(const uint16_t *__restrict__ x, int64_t rows, int64_t cols,
                                             const uint32_t *__restrict__ grp, const uint32_t *__restrict__ dirty,
-                                            int ndirty, const uint16_t *__restrict__ fp_col, int64_t num_int,
+                                            int ndirty, const uint16_t *__restrict__ fp_slot, int64_t num_int,
                                             int64_t num_fp, uint8_t *__restrict__ dst, uint16_t *__restrict__ meta,
                                             uint16_t *__restrict__ fp_x, uint8_t *codes_s, uint4 *dirty_s,
                                             float *red, int vec_out) {
@@ -397,26 +417,45 @@ __device__ __forceinline__ void stream_rows(const uint16_t *__restrict__ x, int6
   const float inf = __builtin_inff();
   uint32_t g[NV];
 #pragma unroll
-  for (int i = 0; i < NV; ++i) g[i] = tid + i * kThreads < nvec ? grp[tid + i * kThreads] : 0xFFFFFFFFu;
-  const uint32_t my_dirty = tid < ndirty ? dirty[tid] : 0u;
-  const uint32_t my_fp_col = tid < num_fp ? fp_col[tid] : 0u;
+  for (int i = 0; i < NV; ++i) g[i] = tid + i * TPR < nvec ? grp[tid + i * TPR] : 0xFFFFFFFFu;
+  // row-invariant tables of this lane's first ND dirty groups and outliers, kept in registers so
+  // that the per-row loops below wait on no global load
+  constexpr int ND = 256 / TPR;
+  uint32_t my_dirty[ND], my_slot[ND];
+#pragma unroll
+  for (int k = 0; k < ND; ++k) {
+    my_dirty[k] = tid + k * TPR < ndirty ? dirty[tid + k * TPR] : 0u;
+    my_slot[k] = tid + k * TPR < num_fp ? fp_slot[tid + k * TPR] : 0u;
+  }
 
   auto load_row = [&](int64_t row, uint4 (&v)[NV]) {
     const uint4 *xv = reinterpret_cast<const uint4 *>(x + row * cols);
 #pragma unroll
     for (int i = 0; i < NV; ++i)
-      if (tid + i * kThreads < nvec) v[i] = xv[tid + i * kThreads];
+      if (tid + i * TPR < nvec) v[i] = xv[tid + i * TPR];
   };
 
-  // per-element masked min/max of one dirty group
-  auto dirty_minmax = [&](const uint4 &v, uint32_t mb, float &mn, float &mx) {
+  // min/max of one dirty group.  fp16: the outlier halves are overwritten with 0xFFFF, a quiet NaN,
+  // which the packed min/max skip; bf16: per-element selects on fp32
+  auto dirty_minmax = [&](const uint4 &v, uint32_t mb, h2 &pmn, h2 &pmx, float &mn, float &mx) {
     const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    if constexpr (!BF16) {
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const float f = to_f32<BF16>(static_cast<uint16_t>(w[e >> 1] >> (16 * (e & 1))));
-      const bool out = (mb >> e) & 1u;
-      mn = fminf(mn, out ? inf : f);
-      mx = fmaxf(mx, out ? -inf : f);
+      for (int k = 0; k < 4; ++k) {
+        const uint32_t lo = static_cast<uint32_t>(__builtin_amdgcn_sbfe(static_cast<int>(mb), 2 * k, 1));
+        const uint32_t hi = static_cast<uint32_t>(__builtin_amdgcn_sbfe(static_cast<int>(mb), 2 * k + 1, 1));
+        const h2 m = __builtin_bit_cast(h2, w[k] | __builtin_amdgcn_perm(hi, lo, 0x07060100u));
+        pmn = __builtin_elementwise_min(pmn, m);
+        pmx = __builtin_elementwise_max(pmx, m);
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float f = to_f32<true>(static_cast<uint16_t>(w[e >> 1] >> (16 * (e & 1))));
+        const bool out = (mb >> e) & 1u;
+        mn = fminf(mn, out ? inf : f);
+        mx = fmaxf(mx, out ? -inf : f);
+      }
     }
   };
   // codes of one dirty group, outliers squeezed out
@@ -434,14 +473,11 @@ __device__ __forceinline__ void stream_rows(const uint16_t *__restrict__ x, int6
 
   // one row; `cur` holds its groups, `parity` alternates so that two sets of reduction slots are used
   auto process = [&](int64_t row, const uint4 (&cur)[NV], int parity) {
-    const uint16_t *xr = x + row * cols;
-    const uint16_t my_fp = tid < num_fp ? xr[my_fp_col] : uint16_t(0);
-
-    // ---- all lanes: min / max as if every group were clean; dirty groups go to LDS
+    // ---- all lanes: min / max as if every group were clean
     float mn = inf, mx = -inf;
+    const h2 pinf = h2{static_cast<_Float16>(inf), static_cast<_Float16>(inf)};
+    h2 pmn = pinf, pmx = -pinf;
     if constexpr (!BF16) {
-      const h2 pinf = h2{static_cast<_Float16>(inf), static_cast<_Float16>(inf)};
-      h2 pmn = pinf, pmx = -pinf;
 #pragma unroll
       for (int i = 0; i < NV; ++i) {
         const h2 a = __builtin_bit_cast(h2, cur[i].x), b = __builtin_bit_cast(h2, cur[i].y);
@@ -452,8 +488,6 @@ __device__ __forceinline__ void stream_rows(const uint16_t *__restrict__ x, int6
         pmn = __builtin_elementwise_min(pmn, clean ? lo : pinf);
         pmx = __builtin_elementwise_max(pmx, clean ? hi : -pinf);
       }
-      mn = fminf(static_cast<float>(pmn.x), static_cast<float>(pmn.y));
-      mx = fmaxf(static_cast<float>(pmx.x), static_cast<float>(pmx.y));
     } else {
 #pragma unroll
       for (int i = 0; i < NV; ++i) {
@@ -470,30 +504,50 @@ __device__ __forceinline__ void stream_rows(const uint16_t *__restrict__ x, int6
         mx = fmaxf(mx, clean ? hi : -inf);
       }
     }
+    // ---- dirty groups go to LDS, indexed by slot
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
-      if ((g[i] & 0xFFu) != 0u && tid + i * kThreads < nvec) dirty_s[g[i] >> 8] = cur[i];
+      if ((g[i] & 0xFFu) != 0u && tid + i * TPR < nvec) dirty_s[g[i] >> 8] = cur[i];
     }
     __syncthreads();  // dirty_s complete; also: the previous row's pack pass has finished reading codes_s
-
-    // ---- lanes 0 .. ndirty-1: one dirty group each
-    uint4 dv = make_uint4(0, 0, 0, 0);
-    if (tid < ndirty) {
-      dv = dirty_s[tid];
-      dirty_minmax(dv, my_dirty & 0xFFu, mn, mx);
+    // ---- outliers, in the caller's order (before the next barrier: the next row overwrites dirty_s)
+    const uint16_t *dirty16 = reinterpret_cast<const uint16_t *>(dirty_s);
+#pragma unroll
+    for (int k = 0; k < ND; ++k)
+      if (tid + k * TPR < num_fp) fp_x[row * num_fp + tid + k * TPR] = dirty16[my_slot[k]];
+    for (int64_t f = tid + ND * TPR; f < num_fp; f += TPR) fp_x[row * num_fp + f] = dirty16[fp_slot[f]];
+    // ---- lanes 0 .. ndirty-1: one dirty group each (more when there are more than TPR of them)
+    uint4 dv[ND];
+#pragma unroll
+    for (int k = 0; k < ND; ++k) {
+      dv[k] = make_uint4(0, 0, 0, 0);
+      if (tid + k * TPR < ndirty) {
+        dv[k] = dirty_s[tid + k * TPR];
+        dirty_minmax(dv[k], my_dirty[k] & 0xFFu, pmn, pmx, mn, mx);
+      }
     }
-    for (int j = tid + kThreads; j < ndirty; j += kThreads) dirty_minmax(dirty_s[j], dirty[j] & 0xFFu, mn, mx);
-
+    for (int j = tid + ND * TPR; j < ndirty; j += TPR) dirty_minmax(dirty_s[j], dirty[j] & 0xFFu, pmn, pmx, mn, mx);
+    if constexpr (!BF16) {
+      mn = fminf(static_cast<float>(pmn.x), static_cast<float>(pmn.y));
+      mx = fmaxf(static_cast<float>(pmx.x), static_cast<float>(pmx.y));
+    }
     mn = wave_min(mn);
     mx = wave_max(mx);
-    float *r = red + parity * 8;  // two sets: the next row's writes cannot overtake this row's reads
-    if ((tid & 63) == 0) {
-      r[tid >> 6] = mn;
-      r[4 + (tid >> 6)] = mx;
+    if constexpr (TPR > 64) {
+      float *r = red + parity * 8;  // two sets: the next row's writes cannot overtake this row's reads
+      if ((tid & 63) == 0) {
+        r[tid >> 6] = mn;
+        r[4 + (tid >> 6)] = mx;
+      }
+      __syncthreads();
+      mn = r[0];
+      mx = r[4];
+#pragma unroll
+      for (int w = 1; w < TPR / 64; ++w) {
+        mn = fminf(mn, r[w]);
+        mx = fmaxf(mx, r[4 + w]);
+      }
     }
-    __syncthreads();
-    mn = fminf(fminf(r[0], r[1]), fminf(r[2], r[3]));
-    mx = fmaxf(fmaxf(r[4], r[5]), fmaxf(r[6], r[7]));
 
     RowQuant<BF16> rq;
     rq.init(mn, mx, BITS);
@@ -501,7 +555,6 @@ __device__ __forceinline__ void stream_rows(const uint16_t *__restrict__ x, int6
       meta[2 * row] = rq.scale_bits;
       meta[2 * row + 1] = rq.zero_bits;
     }
-
     // ---- quantise in source order, 8 code bytes per clean group to their destination position
     auto quantise = [&](auto slow_c) {
       constexpr bool SLOW = decltype(slow_c)::value;
@@ -510,8 +563,10 @@ __device__ __forceinline__ void stream_rows(const uint16_t *__restrict__ x, int6
         const uint2 c = group_codes<BITS, BF16, SLOW>(cur[i], rq);
         if ((g[i] & 0xFFu) == 0u) *reinterpret_cast<Bytes8 *>(codes_s + (g[i] >> 8)) = Bytes8{c.x, c.y};
       }
-      if (tid < ndirty) dirty_codes(dv, my_dirty, rq, slow_c);
-      for (int j = tid + kThreads; j < ndirty; j += kThreads) dirty_codes(dirty_s[j], dirty[j], rq, slow_c);
+#pragma unroll
+      for (int k = 0; k < ND; ++k)
+        if (tid + k * TPR < ndirty) dirty_codes(dv[k], my_dirty[k], rq, slow_c);
+      for (int j = tid + ND * TPR; j < ndirty; j += TPR) dirty_codes(dirty_s[j], dirty[j], rq, slow_c);
     };
     if (__builtin_amdgcn_readfirstlane(rq.slow ? 1 : 0)) {
       quantise(std::true_type{});
@@ -522,7 +577,7 @@ __device__ __forceinline__ void stream_rows(const uint16_t *__restrict__ x, int6
 
     // ---- pack pass: 16 code bytes per lane -> 8 bytes (int4) or 16 bytes (int8)
     const int units = static_cast<int>((num_int + 15) >> 4);
-    for (int u = tid; u < units; u += kThreads) {
+    for (int u = tid; u < units; u += TPR) {
       const uint4 c = *reinterpret_cast<const uint4 *>(codes_s + u * 16);
       const int valid = static_cast<int>(num_int) - u * 16;  // codes of this unit that exist (16 except at the tail)
       if constexpr (BITS == 4) {
@@ -549,24 +604,16 @@ __device__ __forceinline__ void stream_rows(const uint16_t *__restrict__ x, int6
         }
       }
     }
-    // ---- outliers, in the caller's order
-    if (tid < num_fp) fp_x[row * num_fp + tid] = my_fp;
-    for (int64_t f = tid + kThreads; f < num_fp; f += kThreads) fp_x[row * num_fp + f] = xr[fp_col[f]];
   };
 
-  // two register sets alternate: while one row is processed the next one is in flight
-  uint4 buf_a[NV], buf_b[NV];
-  const int64_t stride = gridDim.x;
-  int64_t row = blockIdx.x;
-  if (row < rows) load_row(row, buf_a);
-  while (row < rows) {
-    if (row + stride < rows) load_row(row + stride, buf_b);
-    process(row, buf_a, 0);
-    row += stride;
-    if (row >= rows) break;
-    if (row + stride < rows) load_row(row + stride, buf_a);
-    process(row, buf_b, 1);
-    row += stride;
+  // No software prefetch: the launch makes one workgroup per row (up to the grid limit), several of
+  // them are resident per CU, and their phases drift apart, so loads, arithmetic and stores of
+  // different rows overlap.
+  int parity = 0;
+  for (int64_t row = blockIdx.x; row < rows; row += gridDim.x, parity ^= 1) {
+    uint4 cur[NV];
+    load_row(row, cur);
+    process(row, cur, parity);
   }
 }
 
@@ -583,24 +630,24 @@ __global__ __launch_bounds__(kThreads) void asym_quantize_kernel(
 
 // Shapes that may stream: the column map's flag (known only on the device) picks the path.
 // Dynamic LDS: max(row bytes for the gather path, code bytes + 16 bytes per possible dirty group).
-template <typename IdxT, int BITS, bool BF16, int NV>
-__global__ __launch_bounds__(kThreads) void asym_quantize_stream_kernel(
+template <typename IdxT, int BITS, bool BF16, int NV, int TPR>
+__global__ __launch_bounds__(TPR) void asym_quantize_stream_kernel(
     const uint16_t *__restrict__ x, int64_t rows, int64_t cols, const IdxT *__restrict__ src_col,
     const IdxT *__restrict__ fp_col, const uint32_t *__restrict__ mask, const uint32_t *__restrict__ grp,
-    const uint32_t *__restrict__ dirty, const uint32_t *__restrict__ flags, int64_t num_int, int64_t num_fp,
-    uint8_t *__restrict__ dst, uint16_t *__restrict__ meta, uint16_t *__restrict__ fp_x, int vec_out) {
+    const uint32_t *__restrict__ dirty, const uint16_t *__restrict__ fp_slot, const uint32_t *__restrict__ flags,
+    int64_t num_int, int64_t num_fp, uint8_t *__restrict__ dst, uint16_t *__restrict__ meta,
+    uint16_t *__restrict__ fp_x, int vec_out) {
   static_assert(sizeof(IdxT) == 2, "streaming needs cols <= 32768");
   extern __shared__ __align__(16) uint16_t row_s[];
   __shared__ float red[16];
   if (flags[0] & 1u) {
     uint8_t *codes_s = reinterpret_cast<uint8_t *>(row_s);
     uint4 *dirty_s = reinterpret_cast<uint4 *>(codes_s + align16(num_int));
-    stream_rows<BITS, BF16, NV>(x, rows, cols, grp, dirty, static_cast<int>(flags[1]),
-                                reinterpret_cast<const uint16_t *>(fp_col), num_int, num_fp, dst, meta, fp_x,
-                                codes_s, dirty_s, red, vec_out);
+    stream_rows<BITS, BF16, NV, TPR>(x, rows, cols, grp, dirty, static_cast<int>(flags[1]), fp_slot, num_int, num_fp,
+                                     dst, meta, fp_x, codes_s, dirty_s, red, vec_out);
   } else {
-    gather_rows<IdxT, BITS, BF16>(x, rows, cols, src_col, fp_col, mask, num_int, num_fp, dst, meta, fp_x, 1, row_s,
-                                  red);
+    gather_rows<IdxT, BITS, BF16, TPR>(x, rows, cols, src_col, fp_col, mask, num_int, num_fp, dst, meta, fp_x, 1,
+                                       row_s, red);
   }
 }
 
@@ -737,10 +784,10 @@ int grid_for(int64_t work_items, int64_t per_block) {
 
 constexpr int64_t kMaxLdsRowBytes = 128 * 1024;  // of the 160 KB per CU
 
-template <typename IdxT, int BITS, bool BF16, int NV>
+template <typename IdxT, int BITS, bool BF16, int NV, int TPR>
 int launch_stream(const void *x, int64_t rows, int64_t cols, const uint8_t *cm, const ColmapLayout &l, int64_t num_int,
                   int64_t num_fp, void *dst, void *meta, void *fp_x, hipStream_t st) {
-  auto kern = asym_quantize_stream_kernel<IdxT, BITS, BF16, NV>;
+  auto kern = asym_quantize_stream_kernel<IdxT, BITS, BF16, NV, TPR>;
   const int64_t lds_stream = align16(num_int) + 16 * max_dirty_groups(cols, num_fp);
   const int64_t lds = lds_stream > align16(cols * 2) ? lds_stream : align16(cols * 2);
   if (lds > 48 * 1024) {
@@ -751,15 +798,14 @@ int launch_stream(const void *x, int64_t rows, int64_t cols, const uint8_t *cm, 
       return QUIK_ERR_LAUNCH;
     }
   }
-  // a few rows per workgroup so that the next row's loads overlap the current row's arithmetic
-  const int64_t per_cu = lds <= 20 * 1024 ? 4 : (lds <= 40 * 1024 ? 3 : 2);
-  const int grid = static_cast<int>(rows < 256 * per_cu ? rows : 256 * per_cu);
+  const int grid = static_cast<int>(rows < (int64_t(1) << 30) ? rows : (int64_t(1) << 30));
   const int vec_out = num_int % 16 == 0 && reinterpret_cast<uintptr_t>(dst) % 16 == 0;
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), static_cast<size_t>(lds), st,
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(TPR), static_cast<size_t>(lds), st,
                      static_cast<const uint16_t *>(x), rows, cols, reinterpret_cast<const IdxT *>(cm),
                      reinterpret_cast<const IdxT *>(cm + l.off_fp), reinterpret_cast<const uint32_t *>(cm + l.off_mask),
                      reinterpret_cast<const uint32_t *>(cm + l.off_grp),
                      reinterpret_cast<const uint32_t *>(cm + l.off_dirty),
+                     reinterpret_cast<const uint16_t *>(cm + l.off_slot),
                      reinterpret_cast<const uint32_t *>(cm + l.off_flags), num_int, num_fp,
                      static_cast<uint8_t *>(dst), static_cast<uint16_t *>(meta), static_cast<uint16_t *>(fp_x), vec_out);
   return check_launch();
@@ -772,11 +818,16 @@ int launch_asym(const void *x, int64_t rows, int64_t cols, const uint8_t *cm, co
   const IdxT *fp_col = reinterpret_cast<const IdxT *>(cm + l.off_fp);
   const uint32_t *mask = reinterpret_cast<const uint32_t *>(cm + l.off_mask);
   if constexpr (sizeof(IdxT) == 2) if (cols <= kStreamMaxCols && cols % 8 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0) {
-    const int64_t per_thread = (cols / 8 + kThreads - 1) / kThreads;
-    if (per_thread <= 2) return launch_stream<IdxT, BITS, BF16, 2>(x, rows, cols, cm, l, num_int, num_fp, dst, meta, fp_x, st);
-    if (per_thread <= 4) return launch_stream<IdxT, BITS, BF16, 4>(x, rows, cols, cm, l, num_int, num_fp, dst, meta, fp_x, st);
-    if (per_thread <= 8) return launch_stream<IdxT, BITS, BF16, 8>(x, rows, cols, cm, l, num_int, num_fp, dst, meta, fp_x, st);
-    return launch_stream<IdxT, BITS, BF16, 16>(x, rows, cols, cm, l, num_int, num_fp, dst, meta, fp_x, st);
+    // Four waves per row, one row per workgroup: more, shorter waves hide the load and LDS latencies
+    // better than fewer waves with less per-row fixed work (measured with 64, 128 and 256 threads).
+    const int64_t groups = cols / 8;
+#define QUIK_STREAM(NV) \
+  return launch_stream<IdxT, BITS, BF16, NV, kThreads>(x, rows, cols, cm, l, num_int, num_fp, dst, meta, fp_x, st)
+    if (groups <= 512) QUIK_STREAM(2);
+    if (groups <= 1024) QUIK_STREAM(4);
+    if (groups <= 2048) QUIK_STREAM(8);
+    QUIK_STREAM(16);
+#undef QUIK_STREAM
   }
   const int grid = static_cast<int>(rows < 65535 * 8 ? rows : 65535 * 8);
   const int64_t lds = align16(cols * 2);
@@ -825,12 +876,14 @@ extern "C" int quik_colmap_build(const int64_t *int_indices, int64_t num_int, co
     hipLaunchKernelGGL(colmap_build_kernel<uint16_t>, dim3(1), dim3(1024), 0, as_stream(stream), int_indices,
                        num_int, fp_indices, num_fp, cols, reinterpret_cast<uint16_t *>(cm),
                        reinterpret_cast<uint16_t *>(cm + l.off_fp), mask, reinterpret_cast<uint32_t *>(cm + l.off_grp),
-                       reinterpret_cast<uint32_t *>(cm + l.off_dirty), reinterpret_cast<uint32_t *>(cm + l.off_flags));
+                       reinterpret_cast<uint32_t *>(cm + l.off_dirty), reinterpret_cast<uint16_t *>(cm + l.off_slot),
+                       reinterpret_cast<uint32_t *>(cm + l.off_flags));
   } else {
     hipLaunchKernelGGL(colmap_build_kernel<uint32_t>, dim3(1), dim3(1024), 0, as_stream(stream), int_indices,
                        num_int, fp_indices, num_fp, cols, reinterpret_cast<uint32_t *>(cm),
                        reinterpret_cast<uint32_t *>(cm + l.off_fp), mask, reinterpret_cast<uint32_t *>(cm + l.off_grp),
-                       reinterpret_cast<uint32_t *>(cm + l.off_dirty), reinterpret_cast<uint32_t *>(cm + l.off_flags));
+                       reinterpret_cast<uint32_t *>(cm + l.off_dirty), reinterpret_cast<uint16_t *>(cm + l.off_slot),
+                       reinterpret_cast<uint32_t *>(cm + l.off_flags));
   }
   return check_launch();
 }

@@ -86,6 +86,10 @@ QCASES = [
     (20, 520, 6, "x50", False),        # K = 514: not a multiple of 16, scalar tail of the packed output
     (300, 8192, 256, "x50", False),    # several rows per workgroup (register prefetch of the next row)
     (70, 28672, 256, "student", False),
+    (530, 8192, 256, "x50", False),    # 512 rows or more: one wave per row, 16 groups per lane
+    (600, 2056, 300, "student", False),  # ... 8 groups per lane, more dirty groups than lanes
+    (515, 520, 6, "x50", False),       # ... 4 groups per lane, scalar tail of the packed output
+    (40, 12288, 64, "x50", False),     # four waves per row, 8 groups per lane
 ]
 
 
