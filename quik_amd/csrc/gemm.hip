@@ -1,5 +1,7 @@
 // Host side of the GEMM entry points: argument checks, tile planning, launches.
 // The kernels live in gemm_kernels.h.
+#include <cstdint>
+
 #include "gemm_kernels.h"
 
 namespace quik {
@@ -36,12 +38,6 @@ int grid_of(int64_t M, int64_t N, int &tiles_m, int &tiles_n) {
   return static_cast<int>(((int64_t(tiles_m) * tiles_n + 7) / 8) * 8);
 }
 
-struct I32Args {
-  const uint8_t *X, *W;
-  int32_t *C;
-  int M, N, ldc, kbytes;
-};
-
 template <class C, int MODE>
 int launch_i32(const I32Args &a, hipStream_t st) {
   if (a.N <= 0) return QUIK_OK;
@@ -49,8 +45,32 @@ int launch_i32(const I32Args &a, hipStream_t st) {
   const int grid = grid_of<C>(a.M, a.N, tiles_m, tiles_n);
   auto kern = gemm_i32_kernel<C, MODE>;
   if (int rc = prepare(kern, C::SMEM)) return rc;
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(C::kThreads), C::SMEM, st, a.X, a.W, a.C, a.M, a.N, a.ldc, a.kbytes,
-                     tiles_m, tiles_n);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(C::kThreads), C::SMEM, st, a, tiles_m, tiles_n);
+  return check_launch();
+}
+
+// Workgroup id layout of a two-shape launch: half of the narrow tiles (at most half a round) lead.
+template <class CW, class CT>
+SplitGrid split_grid(int64_t M, int64_t n_wide, int64_t n_tail, int &tail_blocks) {
+  SplitGrid g;
+  g.wide_blocks = grid_of<CW>(M, n_wide, g.tiles_m, g.tiles_n_wide);
+  tail_blocks = grid_of<CT>(M, n_tail, g.tiles_m, g.tiles_n_tail);
+  int lead = (tail_blocks / 2) & ~7;
+  if (lead > kCUs / 2) lead = kCUs / 2;
+  g.lead = lead;
+  return g;
+}
+
+template <class CW, class CT, int MODE>
+int launch_i32_split(const I32Args &wide, const I32Args &tail, hipStream_t st) {
+  if (wide.N <= 0) return launch_i32<CT, MODE>(tail, st);
+  if (tail.N <= 0) return launch_i32<CW, MODE>(wide, st);
+  int tail_blocks;
+  const SplitGrid grid = split_grid<CW, CT>(wide.M, wide.N, tail.N, tail_blocks);
+  auto kern = gemm_i32_split_kernel<CW, CT, MODE>;
+  constexpr int smem = CW::SMEM > CT::SMEM ? CW::SMEM : CT::SMEM;
+  if (int rc = prepare(kern, smem)) return rc;
+  hipLaunchKernelGGL(kern, dim3(grid.wide_blocks + tail_blocks), dim3(CW::kThreads), smem, st, wide, tail, grid);
   return check_launch();
 }
 
@@ -66,13 +86,73 @@ int launch_fused(const FusedArgs &p, hipStream_t st) {
   return check_launch();
 }
 
-// How a problem is cut into launches.  Columns [0, n_wide) go to 256x256 tiles, [n_wide, N) to
-// 256x128 tiles: with one workgroup per CU the run time is (rounds of 256 tiles) x (tile cost),
-// and a narrower tail keeps the last round from running half empty.
+template <class CW, class CT, int MODE, bool BF16>
+int launch_fused_split(const FusedArgs &wide, const FusedArgs &tail, hipStream_t st) {
+  if (wide.N <= 0) return launch_fused<CT, MODE, BF16>(tail, st);
+  if (tail.N <= 0) return launch_fused<CW, MODE, BF16>(wide, st);
+  int tail_blocks;
+  const SplitGrid grid = split_grid<CW, CT>(wide.M, wide.N, tail.N, tail_blocks);
+  auto kern = gemm_fused_split_kernel<CW, CT, MODE, BF16>;
+  constexpr int smem = fused_smem<CW>() > fused_smem<CT>() ? fused_smem<CW>() : fused_smem<CT>();
+  if (int rc = prepare(kern, smem)) return rc;
+  hipLaunchKernelGGL(kern, dim3(grid.wide_blocks + tail_blocks), dim3(CW::kThreads), smem, st, wide, tail, grid);
+  return check_launch();
+}
+
+// How a problem is cut into tiles.  Columns [0, n_wide) go to 256x256 tiles, [n_wide, N) to
+// 256x128 tiles, all in one launch with the wide tiles first.  One workgroup fits per CU and the
+// hardware hands the next workgroup to whichever CU frees up, so the run time is the makespan of
+// that list schedule; the narrow tiles even out its end.
 struct Plan {
   enum Kind { kSmall, kMid, kMidPlain, kLargePlain, kSplit } kind;
   int64_t n_wide;
 };
+
+// relative tile costs in percent of a 256x256 tile (measured)
+constexpr int kCostWide = 100, kCostHalf = 55, kCostMid = 28;
+
+// Makespan of `wide` tiles followed by `half` tiles on kCUs CUs under greedy list scheduling.
+int64_t makespan(int64_t wide, int64_t half) {
+  // after the wide tiles: `rem` CUs carry one tile more than the others
+  const int64_t full = wide / kCUs, rem = wide % kCUs;
+  int64_t lo_level = full * kCostWide, lo_count = kCUs - rem;  // less loaded CUs
+  int64_t hi_level = lo_level + kCostWide, hi_count = rem;
+  // the half tiles go to the least loaded CUs, a whole level at a time
+  while (half > 0) {
+    if (hi_count == 0 || lo_level + kCostHalf <= hi_level) {
+      if (half >= lo_count && lo_level + kCostHalf < hi_level && hi_count > 0) {
+        lo_level += kCostHalf;
+        half -= lo_count;
+      } else if (hi_count == 0) {
+        const int64_t rounds = half / lo_count, left = half % lo_count;
+        return lo_level + rounds * kCostHalf + (left ? kCostHalf : 0);
+      } else if (half >= lo_count) {  // lo reaches hi's level exactly
+        lo_level += kCostHalf;
+        half -= lo_count;
+        if (lo_level == hi_level) {
+          lo_count += hi_count;
+          hi_count = 0;
+        }
+      } else {
+        const int64_t top = lo_level + kCostHalf;
+        return top > hi_level ? top : hi_level;
+      }
+    } else {
+      // adding a half tile to the lower level overtakes the higher one: swap roles afterwards
+      if (half >= lo_count) {
+        half -= lo_count;
+        const int64_t new_hi = lo_level + kCostHalf, new_hi_count = lo_count;
+        lo_level = hi_level;
+        lo_count = hi_count;
+        hi_level = new_hi;
+        hi_count = new_hi_count;
+      } else {
+        return lo_level + kCostHalf;
+      }
+    }
+  }
+  return hi_count > 0 ? hi_level : lo_level;
+}
 
 Plan make_plan(int64_t M, int64_t N, bool dma_ok) {
   if (M <= 32) return {Plan::kSmall, 0};
@@ -82,14 +162,10 @@ Plan make_plan(int64_t M, int64_t N, bool dma_ok) {
     if (M <= 128 || tiles_m * ((N + 255) / 256) < kCUs / 2) return {Plan::kMidPlain, 0};
     return {Plan::kLargePlain, 0};
   }
-  // relative tile costs (256x256 tile = 1)
-  const double cost_half = 0.55, cost_mid = 0.28;
-  const double mid = double(rounds(((M + 127) / 128) * ((N + 127) / 128))) * cost_mid;
-  double best = 1e30;
-  int64_t best_n = 0;
+  const int64_t mid = rounds(((M + 127) / 128) * ((N + 127) / 128)) * kCostMid;
+  int64_t best = INT64_MAX, best_n = 0;
   for (int64_t n_wide = 0; n_wide <= N; n_wide += 256) {
-    const double c = double(rounds(tiles_m * (n_wide / 256))) +
-                     double(rounds(tiles_m * ((N - n_wide + 127) / 128))) * cost_half;
+    const int64_t c = makespan(tiles_m * (n_wide / 256), tiles_m * ((N - n_wide + 127) / 128));
     if (c <= best) {
       best = c;
       best_n = n_wide;
@@ -127,8 +203,7 @@ int run_i32(const uint8_t *X, const uint8_t *W, int32_t *C, int64_t M, int64_t N
   tail.N = static_cast<int>(N - plan.n_wide);
   tail.W = W + plan.n_wide * kbytes;
   tail.C = C + plan.n_wide;
-  if (int rc = launch_i32<CfgL, MODE>(wide, st)) return rc;
-  return launch_i32<CfgH, MODE>(tail, st);
+  return launch_i32_split<CfgL, CfgH, MODE>(wide, tail, st);
 }
 
 template <int MODE, bool BF16>
@@ -151,8 +226,7 @@ int run_fused(const FusedArgs &p, hipStream_t st) {
   tail.bias = p.bias ? p.bias + nw : nullptr;
   tail.fp_w = p.fp_w ? p.fp_w + nw * p.F : nullptr;
   tail.out = p.out + nw;
-  if (int rc = launch_fused<CfgL, MODE, BF16>(wide, st)) return rc;
-  return launch_fused<CfgH, MODE, BF16>(tail, st);
+  return launch_fused_split<CfgL, CfgH, MODE, BF16>(wide, tail, st);
 }
 
 }  // namespace

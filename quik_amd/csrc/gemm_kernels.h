@@ -38,13 +38,11 @@ typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 
 enum Mode { kInt4 = 0, kInt8 = 1, kF16 = 2, kBF16 = 3 };
 
-// EXP is a measurement hook (0 in every shipped instantiation).
-template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int PIPE_ = 0, int EXP_ = 0>
+template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int PIPE_ = 0>
 struct Cfg {
   static constexpr int BM = BM_, BN = BN_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
   static constexpr int BKB = 64;        // K bytes per row and stage
   static constexpr int PIPE = PIPE_;    // 0: plain double buffer, 2: direct-to-LDS 4-stage ring
-  static constexpr int EXP = EXP_;
   static constexpr int WAVES = WAVES_M * WAVES_N;
   static constexpr int kThreads = WAVES * 64;
   static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
@@ -377,7 +375,7 @@ struct DmaPipe {
           U[1 - P][j][0] = *frag_ptr(rs, rk, j);
         }
         if constexpr ((j + 1) % kEvery == 0 && (j + 1) / kEvery - 1 < kCount) {
-          if ((C::EXP & 15) != 2) issue_one<kFirst + (j + 1) / kEvery - 1>(ld_stage);
+          issue_one<kFirst + (j + 1) / kEvery - 1>(ld_stage);
         }
       };
       static_for<NF>(per_frag);
@@ -447,10 +445,11 @@ __device__ __forceinline__ void run_mainloop(const uint8_t *__restrict__ X, int6
 // Workgroup id -> tile.  Hardware deals consecutive workgroup ids round-robin to the 8 XCDs;
 // ids congruent mod 8 therefore share an L2.  Give each XCD a contiguous run of tiles, with M
 // fastest, so concurrently resident tiles of an XCD share W rows and cover all of X.
-__device__ __forceinline__ bool tile_of_block(int tiles_m, int tiles_n, int &tm, int &tn) {
+// `bid` is the workgroup's index inside its launch region; regions start at multiples of 8.
+__device__ __forceinline__ bool tile_of_block(int bid, int tiles_m, int tiles_n, int &tm, int &tn) {
   const int total = tiles_m * tiles_n;
   const int per_xcd = (total + 7) / 8;
-  const int logical = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+  const int logical = (bid % 8) * per_xcd + bid / 8;
   if (logical >= total) return false;
   tm = logical % tiles_m;
   tn = logical / tiles_m;
@@ -513,14 +512,18 @@ struct BlockStore {
 };
 
 // C [M, ldc] int32; this launch covers N columns starting at C's column 0 (host offsets pointers).
+struct I32Args {
+  const uint8_t *X, *W;
+  int32_t *C;
+  int M, N, ldc, kbytes;
+};
+
 template <class C, int MODE>
-__global__ __launch_bounds__(C::kThreads) void gemm_i32_kernel(const uint8_t *__restrict__ X,
-                                                               const uint8_t *__restrict__ W, int32_t *__restrict__ Cm,
-                                                               int M, int N, int ldc, int kbytes, int tiles_m,
-                                                               int tiles_n) {
-  extern __shared__ __align__(16) uint8_t smem[];
-  int tm, tn;
-  if (!tile_of_block(tiles_m, tiles_n, tm, tn)) return;
+__device__ __forceinline__ void i32_tile(const I32Args &a, int tm, int tn, uint8_t *smem) {
+  const uint8_t *__restrict__ X = a.X;
+  const uint8_t *__restrict__ W = a.W;
+  int32_t *__restrict__ Cm = a.C;
+  const int M = a.M, N = a.N, ldc = a.ldc, kbytes = a.kbytes;
   const int m0 = tm * C::BM, n0 = tn * C::BN;
   v16i acc[C::MI][C::NI];
 #pragma unroll
@@ -529,16 +532,8 @@ __global__ __launch_bounds__(C::kThreads) void gemm_i32_kernel(const uint8_t *__
     for (int ni = 0; ni < C::NI; ++ni)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0;
-  long long t_clk = 0, t_wall = 0;
-  if constexpr ((C::EXP & 16) != 0) {
-    t_clk = clock64();
-    t_wall = wall_clock64();
-  }
-  const int lm0 = (C::EXP & 15) == 1 ? 0 : m0, ln0 = (C::EXP & 15) == 1 ? 0 : n0;
-  run_mainloop<C, MODE>(X + int64_t(lm0) * kbytes, kbytes, M - lm0, W + int64_t(ln0) * kbytes, kbytes, N - ln0, kbytes,
+  run_mainloop<C, MODE>(X + int64_t(m0) * kbytes, kbytes, M - m0, W + int64_t(n0) * kbytes, kbytes, N - n0, kbytes,
                         smem, acc);
-  long long t_loop = 0;
-  if constexpr ((C::EXP & 16) != 0) t_loop = clock64();
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = wave / C::WAVES_N, wn = wave % C::WAVES_N;
   constexpr int kShift = MODE == kInt4 ? 8 : 0;
@@ -558,17 +553,47 @@ __global__ __launch_bounds__(C::kThreads) void gemm_i32_kernel(const uint8_t *__
                               acc[mi][ni][4 * g + 2] >> kShift, acc[mi][ni][4 * g + 3] >> kShift};
         Store::put(stage, lane, ni, g, v);
       }
-    if ((C::EXP & 128) == 0 && mb < M && nw < N)
+    if (mb < M && nw < N)
       Store::flush(stage, lane, Cm + int64_t(mb) * ldc + nw, ldc, M - mb, N - nw, vec);
   }
-  if constexpr ((C::EXP & 16) != 0) {
-    if (threadIdx.x == 0 && tm == 0 && tn == 0) {
-      reinterpret_cast<long long *>(Cm)[0] = clock64() - t_clk;
-      reinterpret_cast<long long *>(Cm)[1] = wall_clock64() - t_wall;
-      reinterpret_cast<long long *>(Cm)[2] = t_loop - t_clk;
-    }
+}
+
+template <class C, int MODE>
+__global__ __launch_bounds__(C::kThreads) void gemm_i32_kernel(I32Args a, int tiles_m, int tiles_n) {
+  extern __shared__ __align__(16) uint8_t smem[];
+  int tm, tn;
+  if (!tile_of_block(blockIdx.x, tiles_m, tiles_n, tm, tn)) return;
+  i32_tile<C, MODE>(a, tm, tn, smem);
+}
+
+// One launch, two tile shapes.  Workgroup ids [lead, lead + wide_blocks) take CW tiles of `wide`,
+// the ids before and after take CT tiles of `tail`.  Hardware starts workgroups in id order as CUs
+// free up, so the narrow tiles at the end even out the schedule; the `lead` narrow tiles at the
+// front put part of the CUs half a tile ahead of the others, so that the tiles' store bursts do
+// not all hit memory at the same moment.  lead and wide_blocks are multiples of 8.
+struct SplitGrid {
+  int tiles_m, tiles_n_wide, tiles_n_tail, lead, wide_blocks;
+  // returns 0: no tile, 1: wide tile, 2: tail tile
+  __device__ __forceinline__ int locate(int bid, int &tm, int &tn) const {
+    if (bid >= lead && bid < lead + wide_blocks) return tile_of_block(bid - lead, tiles_m, tiles_n_wide, tm, tn) ? 1 : 0;
+    const int local = bid < lead ? bid : bid - wide_blocks;
+    return tile_of_block(local, tiles_m, tiles_n_tail, tm, tn) ? 2 : 0;
+  }
+};
+
+template <class CW, class CT, int MODE>
+__global__ __launch_bounds__(CW::kThreads) void gemm_i32_split_kernel(I32Args wide, I32Args tail, SplitGrid grid) {
+  static_assert(CW::kThreads == CT::kThreads, "one block size");
+  extern __shared__ __align__(16) uint8_t smem[];
+  int tm, tn;
+  const int kind = grid.locate(blockIdx.x, tm, tn);
+  if (kind == 1) {
+    i32_tile<CW, MODE>(wide, tm, tn, smem);
+  } else if (kind == 2) {
+    i32_tile<CT, MODE>(tail, tm, tn, smem);
   }
 }
+
 
 struct FusedArgs {
   const uint8_t *qx, *qw;
@@ -577,7 +602,6 @@ struct FusedArgs {
   int M, N, ldo, kbytes, F;  // N: columns of this launch; ldo: row stride of out in elements
   int meta_stride;           // 2: (scale, zero) pairs; 1: scales only (symmetric)
   float shift;
-  long long *dbg = nullptr;  // measurement hook (EXP & 16): per-phase cycle stamps of tile 0
 };
 
 // Explicit moves between the accumulation registers (where the MFMA results live) and the vector
@@ -631,10 +655,7 @@ constexpr int fused_smem() {
 }
 
 template <class C, int MODE, bool BF16>
-__global__ __launch_bounds__(C::kThreads) void gemm_fused_kernel(FusedArgs p, int tiles_m, int tiles_n) {
-  extern __shared__ __align__(16) uint8_t smem[];
-  int tm, tn;
-  if (!tile_of_block(tiles_m, tiles_n, tm, tn)) return;
+__device__ __forceinline__ void fused_tile(const FusedArgs &p, int tm, int tn, uint8_t *smem) {
   const int m0 = tm * C::BM, n0 = tn * C::BN;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = wave / C::WAVES_N, wn = wave % C::WAVES_N;
@@ -653,8 +674,6 @@ __global__ __launch_bounds__(C::kThreads) void gemm_fused_kernel(FusedArgs p, in
     const uint8_t *qx = p.qx + int64_t(m0) * p.kbytes, *qw = p.qw + int64_t(n0) * p.kbytes;
     const uint8_t *fx = reinterpret_cast<const uint8_t *>(p.fp_x) + int64_t(m0) * p.F * 2;
     const uint8_t *fw = reinterpret_cast<const uint8_t *>(p.fp_w) + int64_t(n0) * p.F * 2;
-    long long t0 = 0, t1 = 0, t2 = 0, t3 = 0;
-    if constexpr ((C::EXP & 16) != 0) t0 = clock64();
     DmaPipe<C> pipe;
     if constexpr (C::PIPE == 2) {
       pipe.init(smem, qx, p.kbytes, qw, p.kbytes, p.kbytes, fx, int64_t(p.F) * 2, fw, int64_t(p.F) * 2, p.F * 2,
@@ -664,7 +683,6 @@ __global__ __launch_bounds__(C::kThreads) void gemm_fused_kernel(FusedArgs p, in
     } else {
       mainloop_plain<C, MODE>(qx, p.kbytes, p.M - m0, qw, p.kbytes, p.N - n0, p.kbytes, smem, acc);
     }
-    if constexpr ((C::EXP & 16) != 0) t1 = clock64();
     // acc -> f32(acc) * (s_row * s_col), in place.  The int4 accumulators carry a factor 256;
     // it is removed by scaling s_row with 2^-8 instead of shifting: both are exact, so
     // f32(256 a) * ((s_row 2^-8) s_col) rounds to the same float as f32(a) * (s_row s_col).
@@ -691,19 +709,9 @@ __global__ __launch_bounds__(C::kThreads) void gemm_fused_kernel(FusedArgs p, in
         }
       }
     }
-    if constexpr ((C::EXP & 16) != 0) t2 = clock64();
     if constexpr (C::PIPE == 2) {
       pipe.template run<BF16 ? kBF16 : kF16>(pipe.stages0, pipe.stages, accf);
       pipe.drain();
-    }
-    if constexpr ((C::EXP & 16) != 0) {
-      t3 = clock64();
-      if (threadIdx.x == 0 && tm == 0 && tn == 0) {
-        p.dbg[0] = t1 - t0;
-        p.dbg[1] = t2 - t1;
-        p.dbg[2] = t3 - t2;
-        p.dbg[3] = t3;
-      }
     }
   }
   if constexpr (C::PIPE != 2) {
@@ -740,8 +748,28 @@ __global__ __launch_bounds__(C::kThreads) void gemm_fused_kernel(FusedArgs p, in
     if (mb < p.M && nw < p.N) Store::flush(stage, lane, p.out + int64_t(mb) * p.ldo + nw, p.ldo, p.M - mb, p.N - nw, vec);
     __builtin_amdgcn_sched_barrier(0);
   }
-  if constexpr ((C::EXP & 16) != 0) {
-    if (threadIdx.x == 0 && tm == 0 && tn == 0) p.dbg[3] = clock64() - p.dbg[3];
+}
+
+template <class C, int MODE, bool BF16>
+__global__ __launch_bounds__(C::kThreads) void gemm_fused_kernel(FusedArgs p, int tiles_m, int tiles_n) {
+  extern __shared__ __align__(16) uint8_t smem[];
+  int tm, tn;
+  if (!tile_of_block(blockIdx.x, tiles_m, tiles_n, tm, tn)) return;
+  fused_tile<C, MODE, BF16>(p, tm, tn, smem);
+}
+
+// One launch, two tile shapes (see gemm_i32_split_kernel).
+template <class CW, class CT, int MODE, bool BF16>
+__global__ __launch_bounds__(CW::kThreads) void gemm_fused_split_kernel(FusedArgs wide, FusedArgs tail,
+                                                                        SplitGrid grid) {
+  static_assert(CW::kThreads == CT::kThreads, "one block size");
+  extern __shared__ __align__(16) uint8_t smem[];
+  int tm, tn;
+  const int kind = grid.locate(blockIdx.x, tm, tn);
+  if (kind == 1) {
+    fused_tile<CW, MODE, BF16>(wide, tm, tn, smem);
+  } else if (kind == 2) {
+    fused_tile<CT, MODE, BF16>(tail, tm, tn, smem);
   }
 }
 
