@@ -36,6 +36,12 @@ WORKLOADS = {
     "llama2-7b.q_proj": (2048, 4096, 4096, 256, 4),
     "llama2-7b.down_proj.int8": (2048, 11008, 4096, 256, 8),
     "config1": (512, 4096, 4096, 128, 4),
+    "llama2-13b.gate_proj": (2048, 5120, 13824, 256, 4),
+    "llama2-13b.gate_proj.t128": (128, 5120, 13824, 256, 4),
+    "llama2-13b.gate_proj.t16": (16, 5120, 13824, 256, 4),
+    "llama2-13b.gate_proj.t1": (1, 5120, 13824, 256, 4),
+    "llama2-13b.down_proj.int8.t16": (16, 13824, 5120, 256, 8),
+    "llama2-70b.gate_proj.t64": (64, 8192, 28672, 256, 4),
 }
 
 PEAK_INT8_TOPS = 5000.0   # MI355X dense int8 MFMA, published

@@ -2,6 +2,7 @@
 // The kernels live in gemm_kernels.h.
 #include <cstdint>
 
+#include "gemm_decode.h"
 #include "gemm_kernels.h"
 
 namespace quik {
@@ -14,7 +15,6 @@ using CfgH = Cfg<256, 128, 2, 2, 2>;   // half-width tile that evens out the las
 using CfgM = Cfg<128, 128, 2, 2, 2>;   // mid-size problems, two workgroups per CU
 using CfgLp = Cfg<256, 256, 2, 2, 0>;  // plain fallbacks
 using CfgMp = Cfg<128, 128, 2, 2, 0>;
-using CfgS = Cfg<32, 128, 1, 4, 0>;    // decode: M <= 32
 
 constexpr int kCUs = 256;
 
@@ -97,6 +97,32 @@ int launch_fused_split(const FusedArgs &wide, const FusedArgs &tail, hipStream_t
   if (int rc = prepare(kern, smem)) return rc;
   hipLaunchKernelGGL(kern, dim3(grid.wide_blocks + tail_blocks), dim3(CW::kThreads), smem, st, wide, tail, grid);
   return check_launch();
+}
+
+// M <= 32: the weight-streaming kernel of gemm_decode.h.  8 waves per 32-column slab when there are few
+// slabs (so that enough loads are in flight chip-wide) and K gives every wave at least two 128-byte
+// chunks per row; otherwise 4 waves, which lets two workgroups share a CU.
+int decode_waves(int64_t N, int64_t kbytes) {
+  const int64_t slabs = (N + 31) / 32, chunks = (kbytes + kDecodeChunk - 1) / kDecodeChunk;
+  return (chunks >= 16 && slabs <= kCUs) ? 8 : 4;
+}
+
+template <int MODE, bool BF16, bool FUSED, int WAVES>
+int launch_decode_w(const FusedArgs &p, int32_t *C, int ldc, hipStream_t st) {
+  auto kern = gemm_decode_kernel<MODE, BF16, FUSED, WAVES>;
+  constexpr int smem = decode_smem<WAVES, FUSED>();
+  if (int rc = prepare(kern, smem)) return rc;
+  // persistent workgroups: as many as are resident at once (8 waves per CU at this register count)
+  const int64_t slabs = (p.N + 31) / 32, resident = int64_t(kCUs) * (8 / WAVES);
+  hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(slabs < resident ? slabs : resident)), dim3(WAVES * 64), smem, st,
+                     p, C, ldc);
+  return check_launch();
+}
+
+template <int MODE, bool BF16, bool FUSED>
+int launch_decode(const FusedArgs &p, int32_t *C, int ldc, hipStream_t st) {
+  if (decode_waves(p.N, p.kbytes) == 8) return launch_decode_w<MODE, BF16, FUSED, 8>(p, C, ldc, st);
+  return launch_decode_w<MODE, BF16, FUSED, 4>(p, C, ldc, st);
 }
 
 // How a problem is cut into tiles.  Columns [0, n_wide) go to 256x256 tiles, [n_wide, N) to
@@ -192,7 +218,15 @@ int run_i32(const uint8_t *X, const uint8_t *W, int32_t *C, int64_t M, int64_t N
   I32Args a{X, W, C, static_cast<int>(M), static_cast<int>(N), static_cast<int>(N), static_cast<int>(kbytes)};
   const Plan plan = make_plan(M, N, kbytes % 64 == 0);
   switch (plan.kind) {
-    case Plan::kSmall: return launch_i32<CfgS, MODE>(a, st);
+    case Plan::kSmall: {
+      FusedArgs p{};
+      p.qx = X;
+      p.qw = W;
+      p.M = a.M;
+      p.N = a.N;
+      p.kbytes = a.kbytes;
+      return launch_decode<MODE, false, false>(p, C, a.ldc, st);
+    }
     case Plan::kMid: return launch_i32<CfgM, MODE>(a, st);
     case Plan::kMidPlain: return launch_i32<CfgMp, MODE>(a, st);
     case Plan::kLargePlain: return launch_i32<CfgLp, MODE>(a, st);
@@ -210,7 +244,7 @@ template <int MODE, bool BF16>
 int run_fused(const FusedArgs &p, hipStream_t st) {
   const Plan plan = make_plan(p.M, p.N, p.kbytes % 64 == 0 && (p.F * 2) % 64 == 0);
   switch (plan.kind) {
-    case Plan::kSmall: return launch_fused<CfgS, MODE, BF16>(p, st);
+    case Plan::kSmall: return launch_decode<MODE, BF16, true>(p, nullptr, 0, st);
     case Plan::kMid: return launch_fused<CfgM, MODE, BF16>(p, st);
     case Plan::kMidPlain: return launch_fused<CfgMp, MODE, BF16>(p, st);
     case Plan::kLargePlain: return launch_fused<CfgLp, MODE, BF16>(p, st);

@@ -1,0 +1,217 @@
+// Skinny GEMM for at most 32 token rows (decode): the weights are read exactly once, straight from
+// global memory into MFMA operand registers, and the problem is bound by that stream.
+//
+// A slab is 32 output columns (one MFMA row block) times all token rows.  A workgroup of WAVES
+// wavefronts walks over slabs blockIdx.x, blockIdx.x + gridDim.x, ...; inside a slab K is cut into
+// 128-byte chunks per row and wave w takes chunks w, w + WAVES, ...  Every wave runs one
+// continuous stream of (slab, chunk) items with NB register sets in rotation, so NB - 1 chunks
+// are always in flight ahead of the one being multiplied, across slab boundaries too: the memory
+// latency is paid once per wave, not once per slab.
+// Lane l loads 16 bytes of weight row l % 32 at K half l / 32 of each 32-byte step and the
+// matching 16 bytes of token row l % 32: exactly the operand layout of v_mfma_i32_32x32x32_i8, so
+// there is no LDS stage and no shuffle (int4: the same in-register nibble split as the large
+// tiles).  The fp16/bf16 outlier columns are split over the waves the same way; those loads and
+// the epilogue's per-row / per-column scalars are requested when a slab starts.  At the end of a
+// slab the waves' partial accumulators (int32, exact in any order; fp32 outlier sums, added in
+// wave order) meet in LDS, and every wave finalises 16 / WAVES of the 16 values a lane owns with
+// the same epilogue formula as the large tiles.
+#pragma once
+#include "gemm_kernels.h"
+
+namespace quik {
+
+constexpr int kDecodeChunk = 128;  // K bytes per row and wave turn
+constexpr int kDecodeSteps = kDecodeChunk / 32;
+
+template <int WAVES, bool FUSED>
+constexpr int decode_smem() {
+  return WAVES * 4096 * (FUSED ? 2 : 1);
+}
+
+// FUSED: p.out receives the MixedQLinear output.  !FUSED: Cm receives the int32 product.
+template <int MODE, bool BF16, bool FUSED, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void gemm_decode_kernel(FusedArgs args, int32_t *__restrict__ Cm, int ldc) {
+  static_assert(WAVES == 4 || WAVES == 8, "16 values per lane are split over the waves");
+  // plain locals: the lambdas below capture by reference, and a captured argument struct ends up in scratch
+  struct {
+    const uint8_t *qx, *qw;
+    const uint16_t *meta, *s_col, *w_red, *fp_x, *fp_w, *bias;
+    uint16_t *out;
+    int M, N, ldo, kbytes, F, meta_stride;
+    float shift;
+  } p;
+  p.qx = args.qx, p.qw = args.qw, p.meta = args.meta, p.s_col = args.s_col, p.w_red = args.w_red;
+  p.fp_x = args.fp_x, p.fp_w = args.fp_w, p.bias = args.bias, p.out = args.out;
+  p.M = args.M, p.N = args.N, p.ldo = args.ldo, p.kbytes = args.kbytes, p.F = args.F;
+  p.meta_stride = args.meta_stride, p.shift = args.shift;
+  extern __shared__ __align__(16) uint8_t smem[];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 31, h = lane >> 5;
+  const int mrow = r < p.M ? r : p.M - 1;  // rows past the edge are computed on valid memory, never stored
+  const int kbytes = p.kbytes;
+  const int nchunks = (kbytes + kDecodeChunk - 1) / kDecodeChunk;
+  const int slabs = (p.N + 31) / 32;
+  const int stride = gridDim.x;
+  const uint8_t *xp = p.qx + int64_t(mrow) * kbytes + h * 16;
+  constexpr int VPW = 16 / WAVES;                             // values per lane this wave finalises
+  constexpr int kFpEarly = FUSED ? 2 : 0;                     // outlier pieces requested at slab start
+  using FpOps = FragOps<BF16 ? kBF16 : kF16>;
+
+  struct Buf {
+    v4i w[kDecodeSteps], x[kDecodeSteps];
+  };
+  // ---- loader: item (ld_slab, ld_c) -> b, then advance to this wave's next item
+  int ld_slab = blockIdx.x, ld_c = wave;
+  auto issue = [&](Buf &b) __attribute__((always_inline)) {
+    const bool live = ld_slab < slabs && ld_c < nchunks;
+    const int n = ld_slab * 32 + r;
+    const uint8_t *wp = p.qw + int64_t(n < p.N ? n : p.N - 1) * kbytes + h * 16;
+    const int base = ld_c * kDecodeChunk;
+#pragma unroll
+    for (int s = 0; s < kDecodeSteps; ++s) {
+      const int off = base + s * 32;
+      if (live && off + h * 16 < kbytes) {
+        b.w[s] = *reinterpret_cast<const v4i *>(wp + off);
+        b.x[s] = *reinterpret_cast<const v4i *>(xp + off);
+      } else {
+        b.w[s] = v4i{0, 0, 0, 0};
+        b.x[s] = v4i{0, 0, 0, 0};
+      }
+    }
+    ld_c += WAVES;
+    if (ld_c >= nchunks) {  // every wave has at least one (possibly empty) item per slab
+      ld_c = wave;
+      ld_slab += stride;
+    }
+  };
+
+  // ---- per-slab state requested when the slab starts: outlier pieces and epilogue scalars
+  const int fbytes = FUSED ? p.F * 2 : 0;
+  v4i fwe[kFpEarly > 0 ? kFpEarly : 1], fxe[kFpEarly > 0 ? kFpEarly : 1];
+  float srow = 0.0f, zs = 0.0f, e_sc[VPW], e_wr[VPW], e_bs[VPW];
+  const uint8_t *fx = nullptr;
+  if constexpr (FUSED) {
+    fx = reinterpret_cast<const uint8_t *>(p.fp_x) + int64_t(mrow) * fbytes + h * 16;
+    srow = to_f32<BF16>(p.meta[int64_t(mrow) * p.meta_stride]);
+    zs = p.w_red ? to_f32<BF16>(p.meta[2 * int64_t(mrow) + 1]) + p.shift * srow : 0.0f;
+    if constexpr (MODE == kInt4) srow *= 0.00390625f;  // the int4 accumulators carry a factor 256
+  }
+  auto fp_row = [&](int slab) __attribute__((always_inline)) {
+    const int n = slab * 32 + r;
+    return reinterpret_cast<const uint8_t *>(p.fp_w) + int64_t(n < p.N ? n : p.N - 1) * fbytes + h * 16;
+  };
+  auto slab_begin = [&](int slab) __attribute__((always_inline)) {
+    if constexpr (FUSED) {
+      if (slab >= slabs) return;
+      const uint8_t *fw = fp_row(slab);
+#pragma unroll
+      for (int i = 0; i < kFpEarly; ++i) {
+        const int off = (wave + i * WAVES) * 32;
+        fwe[i] = v4i{0, 0, 0, 0};
+        fxe[i] = v4i{0, 0, 0, 0};
+        if (off + h * 16 < fbytes) {
+          fwe[i] = *reinterpret_cast<const v4i *>(fw + off);
+          fxe[i] = *reinterpret_cast<const v4i *>(fx + off);
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < VPW; ++j) {
+        const int v = wave * VPW + j;
+        const int n = slab * 32 + 8 * (v >> 2) + 4 * h + (v & 3);  // accumulator register v of this lane: see acc_col()
+        const int nn = n < p.N ? n : p.N - 1;
+        e_sc[j] = to_f32<BF16>(p.s_col[nn]);
+        e_wr[j] = p.w_red ? to_f32<BF16>(p.w_red[nn]) : 0.0f;
+        e_bs[j] = p.bias ? to_f32<BF16>(p.bias[nn]) : 0.0f;
+      }
+    }
+  };
+
+  v16i acc;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) acc[v] = 0;
+  auto multiply = [&](const Buf &b) __attribute__((always_inline)) {
+#pragma unroll
+    for (int s = 0; s < kDecodeSteps; ++s) {
+      v4i wu[FragOps<MODE>::H], xu[FragOps<MODE>::H];
+      FragOps<MODE>::unpack(b.w[s], wu);
+      FragOps<MODE>::unpack(b.x[s], xu);
+#pragma unroll
+      for (int k = 0; k < FragOps<MODE>::H; ++k) FragOps<MODE>::mma(xu[k], wu[k], acc);
+    }
+  };
+
+  int32_t *red_i = reinterpret_cast<int32_t *>(smem);
+  float *red_f = reinterpret_cast<float *>(smem + WAVES * 4096);
+  // ---- end of a slab: outlier product, cross-wave reduction, epilogue, stores
+  auto slab_end = [&](int slab) __attribute__((always_inline)) {
+    v16f accf;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) accf[v] = 0.0f;
+    if constexpr (FUSED) {
+#pragma unroll
+      for (int i = 0; i < kFpEarly; ++i) FpOps::mma(fxe[i], fwe[i], accf);
+      const uint8_t *fw = fp_row(slab);
+      for (int off = (wave + kFpEarly * WAVES) * 32; off < fbytes; off += WAVES * 32) {
+        v4i wv = v4i{0, 0, 0, 0}, xv = v4i{0, 0, 0, 0};
+        if (off + h * 16 < fbytes) {
+          wv = *reinterpret_cast<const v4i *>(fw + off);
+          xv = *reinterpret_cast<const v4i *>(fx + off);
+        }
+        FpOps::mma(xv, wv, accf);
+      }
+    }
+    // partial sums -> LDS, layout [wave][value][lane]: consecutive lanes, consecutive words
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      red_i[(wave * 16 + v) * 64 + lane] = acc[v];
+      if constexpr (FUSED) red_f[(wave * 16 + v) * 64 + lane] = accf[v];
+      acc[v] = 0;
+    }
+    __syncthreads();
+    // wave w finalises values [w * VPW, (w + 1) * VPW) of every lane
+#pragma unroll
+    for (int j = 0; j < VPW; ++j) {
+      const int v = wave * VPW + j;
+      int32_t ti = 0;
+      float tf = 0.0f;
+#pragma unroll
+      for (int q = 0; q < WAVES; ++q) {
+        ti += red_i[(q * 16 + v) * 64 + lane];
+        if constexpr (FUSED) tf += red_f[(q * 16 + v) * 64 + lane];
+      }
+      const int n = slab * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
+      if (r >= p.M || n >= p.N) continue;
+      if constexpr (FUSED) {
+        const float val = (static_cast<float>(ti) * (srow * e_sc[j]) + tf) + (zs * e_wr[j] + e_bs[j]);
+        p.out[int64_t(r) * p.ldo + n] = from_f32<BF16>(val);
+      } else {
+        Cm[int64_t(r) * ldc + n] = MODE == kInt4 ? (ti >> 8) : ti;
+      }
+    }
+    __syncthreads();  // the next slab's partial sums reuse the area
+  };
+
+  // ---- the stream
+  constexpr int NB = 3;
+  Buf buf[NB];
+  int slab = blockIdx.x, c = wave;  // the item being multiplied
+  slab_begin(slab);
+  static_for<NB - 1>([&](auto I) __attribute__((always_inline)) { issue(buf[I.value]); });
+  while (slab < slabs) {  // uniform over the workgroup: all waves see the same slab sequence
+    static_for<NB>([&](auto I) __attribute__((always_inline)) {
+      if (slab >= slabs) return;
+      constexpr int i = I.value;
+      issue(buf[(i + NB - 1) % NB]);
+      multiply(buf[i]);
+      c += WAVES;
+      if (c >= nchunks) {
+        slab_end(slab);
+        c = wave;
+        slab += stride;
+        slab_begin(slab);
+      }
+    });
+  }
+}
+
+}  // namespace quik

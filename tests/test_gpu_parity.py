@@ -257,6 +257,10 @@ MM_CASES = [
     (128, 512, 4864),
     (300, 260, 7936),
     (512, 1024, 3968),
+    # at most 32 token rows: the weight-streaming kernel (slabs of 32 columns, 128-byte K chunks per wave)
+    (5, 40, 32),         # one chunk, fewer chunks than waves, ragged last slab
+    (32, 8200, 4864),    # more slabs than resident workgroups: several slabs per workgroup
+    (17, 96, 4096 + 32), # 8 waves per slab (long K, few slabs), K tail of half a 32-byte step for int4
 ]
 
 
@@ -278,7 +282,8 @@ def test_int4_matmul_exact(M, N, K):
 
 
 @pytest.mark.parametrize("M,N,K", [(512, 32, 512), (1, 128, 13568), (16, 300, 16), (100, 40, 48),
-                                     (257, 384, 10752), (300, 260, 2048), (2, 2, 28416)])
+                                     (257, 384, 10752), (300, 260, 2048), (2, 2, 28416),
+                                     (3, 31, 16 * 11), (32, 8200, 2048), (17, 96, 4096 + 16)])
 def test_int8_matmul_exact(M, N, K):
     import quik
     rng = np.random.default_rng(M * 5 + N * 11 + K)
@@ -428,6 +433,10 @@ FWD_CASES = [
     (260, 300, 1280, 256, 8, True, "x50"),
     (64, 128, 512, 0, 4, True, "x50"),
     (1, 384, 1024, 64, 4, False, "x50"),
+    (5, 40, 72, 8, 4, True, "x50"),          # decode kernel: one K chunk, half an outlier piece, ragged slab
+    (7, 100, 200, 8, 8, True, "student"),
+    (32, 8200, 1056, 32, 4, False, "x50"),   # decode kernel: several slabs per workgroup
+    (20, 64, 8192 + 520, 520, 8, True, "x50"),  # decode kernel: 8 waves per slab, more outlier pieces than prefetched
 ]
 
 
