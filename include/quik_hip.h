@@ -93,6 +93,31 @@ int quik_sym_dequantize(const void *x, int x_bits, const void *scale_row,
                         const void *scale_col, const void *y, int64_t rows, int64_t cols,
                         void *out, void *stream);
 
+/* quik.asymmetric.int4FusedDequantize / int8FusedDequantize(A, B, scale_row, scale_col, shift_value,
+ *                                                          zero_row, w_reduced, y) -> out fp16 [M, N]
+ * replaces int4FusedDequantizeCUDA / int8FusedDequantizeCUDA, src/asymmetric/fused_dequantize.cu:9-119.
+ *   A [M, K/2] uint8 or [M, K] int8; B [N, K/2] or [N, K]; scale_row, zero_row [M] fp16;
+ *   scale_col, w_reduced [N] fp16; y [M, N] fp16.
+ *   out = ((h(acc) * scale_col) * scale_row + (zero_row + h(shift) * scale_row) * w_reduced) + y
+ * in fp16 arithmetic, one rounding per operation, exactly as the reference's epilogue
+ * (include/asymmetric/epilogue/thread/linear_combination_dequant.h:155-162).
+ * Two launches: the exact int32 product goes to acc_workspace ([M, N] int32, caller-provided),
+ * the epilogue reads it back. */
+int quik_asym_fused_dequantize(const void *A, const void *B, const void *scale_row,
+                               const void *scale_col, float shift_value, const void *zero_row,
+                               const void *w_reduced, const void *y, int64_t M, int64_t N,
+                               int64_t K, int bits, int32_t *acc_workspace, void *out,
+                               void *stream);
+
+/* quik.symmetric.int4FusedDequantize / int8FusedDequantize(A, B, scale_row, scale_col, y) -> out
+ * replaces int4FusedDequantizeCUDA / int8FusedDequantizeCUDA, src/symmetric/fused_dequantize.cu:9-107.
+ *   out = ((h(acc) * scale_row) * scale_col) + y in fp16 arithmetic
+ * (include/symmetric/epilogue/thread/linear_combination_dequant.h:149-150).  Workspace as above. */
+int quik_sym_fused_dequantize(const void *A, const void *B, const void *scale_row,
+                              const void *scale_col, const void *y, int64_t M, int64_t N,
+                              int64_t K, int bits, int32_t *acc_workspace, void *out,
+                              void *stream);
+
 /* quik.matmul.int4Matmul(A, B) -> C int32 [M, N]
  * replaces int4MatmulCUDA, src/matmul/matmul.cu:17-55.
  *   A [M, K/2], B [N, K/2] uint8 nibble-packed, K = number of int4 elements per row.

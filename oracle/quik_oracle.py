@@ -269,6 +269,28 @@ def asym_dequantize_f64(acc, meta, scale_col, w_reduced, y, bits, dtype=F16):
     return np.asarray(acc, np.float64) * (s * c) + (z + shift_value * s) * w + _as_f32(y, dtype).astype(np.float64)
 
 
+def asym_fused_dequantize(acc, scale_row, scale_col, shift_value, zero_row, w_reduced, y):
+    """Epilogue of quik.asymmetric.int{4,8}FusedDequantize, fp16 arithmetic, one rounding per op:
+
+        ((h(acc) * scale_col) * scale_row + (zero_row + h(shift) * scale_row) * w_reduced) + y
+
+    include/asymmetric/epilogue/thread/linear_combination_dequant.h:155-162 (c10::Half operators:
+    fp32 op, result rounded to half; `row_vec` is bound to scale_col and `col_vec` to scale_row,
+    src/asymmetric/fused_dequantize.cu:46-57); the same expression is the reference's own
+    known-answer formula, test/python/test_fused.py:56-62."""
+    h = np.float16
+    with np.errstate(over="ignore", invalid="ignore"):
+        a = np.asarray(acc, np.int32).astype(np.float64).astype(h)       # exact int -> one rounding to half
+        sr = np.asarray(scale_row, h).reshape(-1, 1)
+        sc = np.asarray(scale_col, h).reshape(1, -1)
+        z = np.asarray(zero_row, h).reshape(-1, 1)
+        w = np.asarray(w_reduced, h).reshape(1, -1)
+        sh = h(np.float32(shift_value))
+        t = ((a * sc).astype(h) * sr).astype(h)
+        u = ((z + (sh * sr).astype(h)).astype(h) * w).astype(h)
+        return ((t + u).astype(h) + np.asarray(y, h)).astype(h)
+
+
 # --------------------------------------------------------------------------- #
 # symmetric variants (src/symmetric/symmetric.cu)
 # --------------------------------------------------------------------------- #

@@ -26,6 +26,9 @@ SIGNATURES = {
     "quik_asym_dequantize": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _int, _vp, _vp]),
     "quik_sym_quantize": (_int, [_vp, _vp, _i64, _i64, _int, _vp, _vp]),
     "quik_sym_dequantize": (_int, [_vp, _int, _vp, _vp, _vp, _i64, _i64, _vp, _vp]),
+    "quik_asym_fused_dequantize": (_int, [_vp, _vp, _vp, _vp, ctypes.c_float, _vp, _vp, _vp, _i64, _i64, _i64, _int,
+                                          _vp, _vp, _vp]),
+    "quik_sym_fused_dequantize": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp, _vp, _vp]),
     "quik_int4_matmul": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "quik_int8_matmul": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "quik_mixed_linear_fwd": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _i64, _int,

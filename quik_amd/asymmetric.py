@@ -11,7 +11,7 @@ import torch
 
 from . import _lib as L
 
-__all__ = ["quantize", "dequantize", "find_meta", "quantizeOld", "build_colmap", "quantize_mapped"]
+__all__ = ["int4FusedDequantize", "int8FusedDequantize", "quantize", "dequantize", "find_meta", "quantizeOld", "build_colmap", "quantize_mapped"]
 
 
 def _check_bits(bits):
@@ -142,3 +142,43 @@ def quantizeOld(src: torch.Tensor, meta: torch.Tensor, bits: int) -> torch.Tenso
         L.check(lib.quik_asym_quantize_old(L.ptr(src), L.ptr(meta), rows, cols, bits, L.ptr(dst), L.stream()),
                 "quantize")
     return dst
+
+
+def _fused_operands(op, A, B, bits):
+    want = torch.uint8 if bits == 4 else torch.int8
+    if A.dtype != want or B.dtype != want:
+        raise RuntimeError(f"{op}: expected {want} operands but got {A.dtype} and {B.dtype}")
+    if A.dim() != 2 or B.dim() != 2 or A.size(1) != B.size(1):
+        raise RuntimeError(f"{op}: A [M, K] and B [N, K] must agree in K, got {tuple(A.shape)} and {tuple(B.shape)}")
+    return A.size(0), B.size(0), A.size(1) * (2 if bits == 4 else 1)
+
+
+def _fused_dequantize(op, bits, A, B, scale_row, scale_col, shift_value, zero_row, w_reduced, y):
+    L.check_cuda_contiguous(op, A=A, B=B, scale_row=scale_row, scale_col=scale_col, zero_row=zero_row,
+                            w_reduced=w_reduced, y=y)
+    M, N, K = _fused_operands(op, A, B, bits)
+    for name, t, n in (("scale_row", scale_row, M), ("zero_row", zero_row, M), ("scale_col", scale_col, N),
+                       ("w_reduced", w_reduced, N), ("y", y, M * N)):
+        L.dtype_id(t, op, allow_bf16=False)
+        if t.numel() != n:
+            raise RuntimeError(f"{op}: expected {name} to have {n} elements but got {t.numel()}")
+    lib = L.load()
+    with torch.cuda.device(A.device):
+        acc = torch.empty((M, N), dtype=torch.int32, device=A.device)
+        out = torch.empty((M, N), dtype=torch.float16, device=A.device)
+        L.check(lib.quik_asym_fused_dequantize(L.ptr(A), L.ptr(B), L.ptr(scale_row), L.ptr(scale_col),
+                                               float(shift_value), L.ptr(zero_row), L.ptr(w_reduced), L.ptr(y), M, N,
+                                               K, bits, L.ptr(acc), L.ptr(out), L.stream()), op)
+    return out
+
+
+def int4FusedDequantize(A, B, scale_row, scale_col, shift_value, zero_row, w_reduced, y):
+    """out = int4(A) @ int4(B)^T * scale_col * scale_row + (zero_row + shift_value * scale_row) * w_reduced + y,
+    evaluated left to right in fp16 like the reference's epilogue (src/asymmetric/asymmetric.cpp:46-65).
+    A [M, K/2], B [N, K/2] uint8; scale_row, zero_row [M, 1]; scale_col, w_reduced [1, N]; y [M, N]; all fp16."""
+    return _fused_dequantize("int4FusedDequantize", 4, A, B, scale_row, scale_col, shift_value, zero_row, w_reduced, y)
+
+
+def int8FusedDequantize(A, B, scale_row, scale_col, shift_value, zero_row, w_reduced, y):
+    """int8 operands [M, K] / [N, K]; otherwise as int4FusedDequantize (src/asymmetric/asymmetric.cpp:67-88)."""
+    return _fused_dequantize("int8FusedDequantize", 8, A, B, scale_row, scale_col, shift_value, zero_row, w_reduced, y)

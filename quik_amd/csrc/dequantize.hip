@@ -97,6 +97,29 @@ __global__ __launch_bounds__(kThreads) void sym_dequant_kernel(const T *__restri
   }
 }
 
+// Epilogue of the reference's asymmetric fused GEMM, fp16 arithmetic with one rounding per operation
+// (reference: include/asymmetric/epilogue/thread/linear_combination_dequant.h:155-162):
+//   ((h(acc) * scale_col) * scale_row + (zero_row + h(shift) * scale_row) * w_reduced) + y
+__global__ __launch_bounds__(kThreads) void asym_fused_chain_kernel(
+    const int32_t *__restrict__ acc, const uint16_t *__restrict__ srow, const uint16_t *__restrict__ scol,
+    _Float16 shift, const uint16_t *__restrict__ zrow, const uint16_t *__restrict__ wred,
+    const uint16_t *__restrict__ y, int64_t rows, int64_t cols, uint16_t *__restrict__ out) {
+  const int64_t total = rows * cols;
+  for (int64_t i = blockIdx.x * int64_t(kThreads) + threadIdx.x; i < total; i += int64_t(gridDim.x) * kThreads) {
+    const int64_t r = i / cols, c = i - r * cols;
+    const _Float16 sr = __builtin_bit_cast(_Float16, srow[r]);
+    _Float16 t = sym_to_half<int32_t>(acc[i]);
+    t = t * __builtin_bit_cast(_Float16, scol[c]);
+    t = t * sr;
+    _Float16 u = shift * sr;
+    u = __builtin_bit_cast(_Float16, zrow[r]) + u;
+    u = u * __builtin_bit_cast(_Float16, wred[c]);
+    t = t + u;
+    t = t + __builtin_bit_cast(_Float16, y[i]);
+    out[i] = __builtin_bit_cast(uint16_t, t);
+  }
+}
+
 int grid_for(int64_t items) {
   int64_t g = (items + kThreads - 1) / kThreads;
   if (g < 1) g = 1;
@@ -166,4 +189,43 @@ extern "C" int quik_sym_dequantize(const void *x, int x_bits, const void *scale_
     hipLaunchKernelGGL(sym_dequant_kernel<int32_t>, dim3(grid), dim3(kThreads), 0, st,
                        static_cast<const int32_t *>(x), sr, sc, yy, rows, cols, o);
   return check_launch();
+}
+
+// The reference's fused GEMM + dequantize ops as two launches: the exact int32 product into the
+// caller's workspace, then the fp16-arithmetic epilogue of the reference on top of it.
+static int int_matmul(const void *A, const void *B, int32_t *acc, int64_t M, int64_t N, int64_t K, int bits,
+                      void *stream) {
+  if (bits == 4)
+    return quik_int4_matmul(static_cast<const uint8_t *>(A), static_cast<const uint8_t *>(B), acc, M, N, K, stream);
+  if (bits == 8)
+    return quik_int8_matmul(static_cast<const int8_t *>(A), static_cast<const int8_t *>(B), acc, M, N, K, stream);
+  return QUIK_ERR_BITS;
+}
+
+extern "C" int quik_asym_fused_dequantize(const void *A, const void *B, const void *scale_row, const void *scale_col,
+                                          float shift_value, const void *zero_row, const void *w_reduced,
+                                          const void *y, int64_t M, int64_t N, int64_t K, int bits,
+                                          int32_t *acc_workspace, void *out, void *stream) {
+  if (bits != 4 && bits != 8) return QUIK_ERR_BITS;
+  if (M < 0 || N < 0 || K <= 0) return QUIK_ERR_SHAPE;
+  if (M == 0 || N == 0) return QUIK_OK;
+  if (!scale_row || !scale_col || !zero_row || !w_reduced || !y || !acc_workspace || !out) return QUIK_ERR_NULL;
+  if (int rc = int_matmul(A, B, acc_workspace, M, N, K, bits, stream)) return rc;
+  hipLaunchKernelGGL(asym_fused_chain_kernel, dim3(grid_for(M * N)), dim3(kThreads), 0, as_stream(stream),
+                     acc_workspace, static_cast<const uint16_t *>(scale_row), static_cast<const uint16_t *>(scale_col),
+                     static_cast<_Float16>(shift_value), static_cast<const uint16_t *>(zero_row),
+                     static_cast<const uint16_t *>(w_reduced), static_cast<const uint16_t *>(y), M, N,
+                     static_cast<uint16_t *>(out));
+  return check_launch();
+}
+
+extern "C" int quik_sym_fused_dequantize(const void *A, const void *B, const void *scale_row, const void *scale_col,
+                                         const void *y, int64_t M, int64_t N, int64_t K, int bits,
+                                         int32_t *acc_workspace, void *out, void *stream) {
+  if (bits != 4 && bits != 8) return QUIK_ERR_BITS;
+  if (M < 0 || N < 0 || K <= 0) return QUIK_ERR_SHAPE;
+  if (M == 0 || N == 0) return QUIK_OK;
+  if (!scale_row || !scale_col || !y || !acc_workspace || !out) return QUIK_ERR_NULL;
+  if (int rc = int_matmul(A, B, acc_workspace, M, N, K, bits, stream)) return rc;
+  return quik_sym_dequantize(acc_workspace, 32, scale_row, scale_col, y, M, N, out, stream);
 }

@@ -11,7 +11,7 @@ import torch
 
 from . import _lib as L
 
-__all__ = ["quantize", "dequantize"]
+__all__ = ["quantize", "dequantize", "int4FusedDequantize", "int8FusedDequantize"]
 
 
 def quantize(src: torch.Tensor, scale: torch.Tensor, bits: int = 4) -> torch.Tensor:
@@ -63,3 +63,35 @@ def dequantize(x: torch.Tensor, scale_row: torch.Tensor, scale_col: torch.Tensor
         L.check(lib.quik_sym_dequantize(L.ptr(x), bits, L.ptr(scale_row), L.ptr(scale_col), L.ptr(y), rows, cols,
                                         L.ptr(out), L.stream()), "dequantize")
     return out
+
+
+def _fused_dequantize(op, bits, A, B, scale_row, scale_col, y):
+    L.check_cuda_contiguous(op, A=A, B=B, scale_row=scale_row, scale_col=scale_col, y=y)
+    want = torch.uint8 if bits == 4 else torch.int8
+    if A.dtype != want or B.dtype != want:
+        raise RuntimeError(f"{op}: expected {want} operands but got {A.dtype} and {B.dtype}")
+    if A.dim() != 2 or B.dim() != 2 or A.size(1) != B.size(1):
+        raise RuntimeError(f"{op}: A [M, K] and B [N, K] must agree in K, got {tuple(A.shape)} and {tuple(B.shape)}")
+    M, N, K = A.size(0), B.size(0), A.size(1) * (2 if bits == 4 else 1)
+    for name, t, n in (("scale_row", scale_row, M), ("scale_col", scale_col, N), ("y", y, M * N)):
+        L.dtype_id(t, op, allow_bf16=False)
+        if t.numel() != n:
+            raise RuntimeError(f"{op}: expected {name} to have {n} elements but got {t.numel()}")
+    lib = L.load()
+    with torch.cuda.device(A.device):
+        acc = torch.empty((M, N), dtype=torch.int32, device=A.device)
+        out = torch.empty((M, N), dtype=torch.float16, device=A.device)
+        L.check(lib.quik_sym_fused_dequantize(L.ptr(A), L.ptr(B), L.ptr(scale_row), L.ptr(scale_col), L.ptr(y), M, N, K,
+                                              bits, L.ptr(acc), L.ptr(out), L.stream()), op)
+    return out
+
+
+def int4FusedDequantize(A, B, scale_row, scale_col, y):
+    """out = int4(A) @ int4(B)^T * scale_row * scale_col + y, left to right in fp16
+    (src/symmetric/symmetric.cpp:44-57).  A [M, K/2], B [N, K/2] uint8; scale_row [M, 1], scale_col [1, N], y [M, N] fp16."""
+    return _fused_dequantize("int4FusedDequantize", 4, A, B, scale_row, scale_col, y)
+
+
+def int8FusedDequantize(A, B, scale_row, scale_col, y):
+    """int8 operands [M, K] / [N, K]; otherwise as int4FusedDequantize (src/symmetric/symmetric.cpp:59-72)."""
+    return _fused_dequantize("int8FusedDequantize", 8, A, B, scale_row, scale_col, y)

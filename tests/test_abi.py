@@ -75,6 +75,11 @@ def test_python_surface_matches_reference_names():
     assert sig(symmetric.quantize) == ["src", "scale", "bits"]
     assert sig(symmetric.dequantize) == ["x", "scale_row", "scale_col", "y", "bits"]
     assert sig(matmul.int4Matmul) == ["A", "B"] and sig(matmul.int8Matmul) == ["A", "B"]
+    # fused GEMM + dequantize ops (src/asymmetric/asymmetric.cpp:182-211, src/symmetric/symmetric.cpp:120-136)
+    for f in (asymmetric.int4FusedDequantize, asymmetric.int8FusedDequantize):
+        assert sig(f) == ["A", "B", "scale_row", "scale_col", "shift_value", "zero_row", "w_reduced", "y"]
+    for f in (symmetric.int4FusedDequantize, symmetric.int8FusedDequantize):
+        assert sig(f) == ["A", "B", "scale_row", "scale_col", "y"]
     from quik_amd import qlinear
     assert sig(qlinear.MixedQLinear.from_float)[:7] == ["module", "weight_matrix", "weights_scales", "shared_input",
                                                          "fp_indices", "symm", "bits"]

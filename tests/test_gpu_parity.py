@@ -696,3 +696,66 @@ def test_decoder_block_linears_chained(tokens):
     assert shared_mlp.qint_x is None
     out = h2 + run("down", (torch.nn.functional.silu(g) * u).half())
     assert torch.isfinite(out).all()
+
+
+# ------------------------------------------------------------------------------ fused GEMM + dequantize ops
+def _fused_operands(bits, M, N, K, spread, seed):
+    torch.manual_seed(seed)
+    a_ref = torch.randint(-spread, spread, (M, K), dtype=torch.int8)
+    b_ref = torch.randint(-spread, spread, (N, K), dtype=torch.int8)
+    if bits == 4:
+        a, b = _t(qo.pack_i4(a_ref.numpy())), _t(qo.pack_i4(b_ref.numpy()))
+    else:
+        a, b = a_ref.to(DEV), b_ref.to(DEV)
+    return a_ref.to(DEV), b_ref.to(DEV), a, b
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_fused_dequantize_reference_known_answers(bits):
+    """The reference's own known-answer tests for the fused ops, same shapes, distributions and
+    formulas (test/python/test_fused.py:16-67 int4, :130-177 int8), evaluated by torch on the device."""
+    import quik
+    M, N, K = 1024, 5120, 2048
+    a_ref, b_ref, a, b = _fused_operands(bits, M, N, K, 3, 1)
+    scale_row = torch.rand(M, 1, dtype=torch.float16).to(DEV)
+    scale_col = torch.rand(1, N, dtype=torch.float16).to(DEV)
+    y = torch.rand(M, N).to(torch.float16).to(DEV)
+    c_int = torch.matmul(a_ref.float(), b_ref.float().transpose(1, 0)).round().to(torch.int32)
+    sym = quik.symmetric.int4FusedDequantize if bits == 4 else quik.symmetric.int8FusedDequantize
+    c = sym(a, b, scale_row, scale_col, y)
+    assert torch.equal(c, c_int * scale_row * scale_col + y)
+
+    shift_value = 0.6394267984578837          # random.random() under seed 42
+    zero_row = torch.rand(M, 1, dtype=torch.float16).to(DEV)
+    w_reduce = torch.rand(1, N, dtype=torch.float16).to(DEV)
+    c_ref = c_int * scale_col * scale_row + \
+        (zero_row + torch.tensor([shift_value], dtype=torch.float16).item() * scale_row) * w_reduce + y
+    asym = quik.asymmetric.int4FusedDequantize if bits == 4 else quik.asymmetric.int8FusedDequantize
+    c = asym(a, b, scale_row, scale_col, shift_value, zero_row, w_reduce, y)
+    assert torch.equal(c, c_ref)
+
+
+@pytest.mark.parametrize("bits,spread", [(4, 8), (8, 128)])
+def test_fused_dequantize_vs_oracle_full_operand_range(bits, spread):
+    """Full-range operands: accumulators far beyond 2048, so the int32 -> fp16 conversion rounds and,
+    for int8, overflows to inf; bit-exact against the oracle (NaN positions equal, payloads ignored)."""
+    import quik
+    M, N, K = 70, 200, 1024
+    a_ref, b_ref, a, b = _fused_operands(bits, M, N, K, spread, 5)
+    rng = np.random.default_rng(7)
+    scale_row = rng.uniform(0, 1, (M, 1)).astype(np.float16)
+    scale_col = rng.uniform(0, 1, (1, N)).astype(np.float16)
+    zero_row = rng.standard_normal((M, 1)).astype(np.float16)
+    w_reduce = rng.standard_normal((1, N)).astype(np.float16)
+    y = rng.standard_normal((M, N)).astype(np.float16)
+    acc = qo.int_matmul(a_ref.cpu().numpy(), b_ref.cpu().numpy())
+    sym = quik.symmetric.int4FusedDequantize if bits == 4 else quik.symmetric.int8FusedDequantize
+    asym = quik.asymmetric.int4FusedDequantize if bits == 4 else quik.asymmetric.int8FusedDequantize
+    got = sym(a, b, _t(scale_row), _t(scale_col), _t(y)).cpu().numpy()
+    want = qo.sym_dequantize(acc, scale_row, scale_col, y, 32)
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    assert np.array_equal(got[~np.isnan(want)].view(np.uint16), want[~np.isnan(want)].view(np.uint16))
+    got = asym(a, b, _t(scale_row), _t(scale_col), 8.0, _t(zero_row), _t(w_reduce), _t(y)).cpu().numpy()
+    want = qo.asym_fused_dequantize(acc, scale_row, scale_col, 8.0, zero_row, w_reduce, y)
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    assert np.array_equal(got[~np.isnan(want)].view(np.uint16), want[~np.isnan(want)].view(np.uint16))

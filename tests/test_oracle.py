@@ -376,3 +376,35 @@ def test_sim_path_agrees_to_quantisation_noise():
     scale = 3.0 / 15
     assert torch.allclose(q, torch.tensor([[-1.0, 0.0, 0.4, 2.0]]), atol=scale / 2 + 1e-6)
     assert q[0, 1] == 0 and abs(q[0, 0] + 1.0) < 1e-6
+
+
+# ---------------------------------------------------------------------------- fused dequantize ops
+@pytest.mark.parametrize("spread", [3, 8, 128])
+def test_fused_dequantize_epilogues_vs_reference_known_answer_formula(spread):
+    """The reference pins its fused GEMM + dequantize ops by evaluating the formula with torch tensor
+    arithmetic (test/python/test_fused.py:33-37 symmetric, :56-62 asymmetric): int32 times fp16 tensors
+    promote to fp16 and every operation rounds to fp16.  The same expressions, evaluated here by torch
+    on the CPU, must equal the oracle bit for bit; `spread` widens the operands beyond the reference's
+    randint(-3, 3) so that the int32 -> fp16 conversion rounds (|acc| > 2048) and overflows."""
+    g = torch.Generator().manual_seed(spread)
+    M, N, K = 48, 80, 256
+    a = torch.randint(-spread, spread, (M, K), generator=g, dtype=torch.int32)
+    b = torch.randint(-spread, spread, (N, K), generator=g, dtype=torch.int32)
+    c_ref = a @ b.t()
+    scale_row = torch.rand(M, 1, generator=g).half()
+    scale_col = torch.rand(1, N, generator=g).half()
+    zero_row = torch.rand(M, 1, generator=g).half()
+    w_reduce = torch.rand(1, N, generator=g).half()
+    y = torch.rand(M, N, generator=g).half()
+    shift_value = 0.7371
+    want_sym = c_ref * scale_row * scale_col + y
+    want_asym = c_ref * scale_col * scale_row + \
+        (zero_row + torch.tensor([shift_value], dtype=torch.float16).item() * scale_row) * w_reduce + y
+    assert want_sym.dtype == torch.float16 and want_asym.dtype == torch.float16
+    got_sym = qo.sym_dequantize(c_ref.numpy(), scale_row.numpy(), scale_col.numpy(), y.numpy(), 32)
+    got_asym = qo.asym_fused_dequantize(c_ref.numpy(), scale_row.numpy(), scale_col.numpy(), shift_value,
+                                        zero_row.numpy(), w_reduce.numpy(), y.numpy())
+    assert np.array_equal(got_sym.view(np.uint16), want_sym.numpy().view(np.uint16))
+    assert np.array_equal(got_asym.view(np.uint16), want_asym.numpy().view(np.uint16))
+    if spread == 128:
+        assert np.isinf(got_asym).any()       # the overflow case is really exercised
