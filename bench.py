@@ -31,6 +31,7 @@ WORKLOADS = {
     "llama2-70b.gate_proj": (2048, 8192, 28672, 256, 4),
     "llama2-70b.q_proj": (2048, 8192, 8192, 256, 4),
     "llama2-70b.k_proj": (2048, 8192, 1024, 256, 4),
+    "llama2-70b.qkv_fused": (2048, 8192, 10240, 256, 4),       # q + k + v as one GEMM (FusedMixedQLinearGroup)
     "llama2-70b.down_proj.int8": (2048, 28672, 8192, 256, 8),
     "llama2-7b.gate_proj": (2048, 4096, 11008, 256, 4),
     "llama2-7b.q_proj": (2048, 4096, 4096, 256, 4),

@@ -22,7 +22,8 @@ from torch import Tensor
 
 from . import asymmetric, matmul, symmetric
 
-__all__ = ["MixedQLinear", "SharedQuantizedInput", "Linear4bit", "Linear8bit", "pack_to_i4", "two_compl"]
+__all__ = ["MixedQLinear", "SharedQuantizedInput", "FusedMixedQLinearGroup", "Linear4bit", "Linear8bit", "pack_to_i4",
+           "two_compl"]
 
 
 def two_compl(x: Tensor, bits: int) -> Tensor:
@@ -201,6 +202,49 @@ class MixedQLinear(torch.nn.Module):
         if mod.fp_features_num > 0:
             mod.fp_weight.copy_(weight_matrix[:, fp_indices.to(dev)].to(weight_matrix.dtype))
         return mod
+
+
+class FusedMixedQLinearGroup(torch.nn.Module):
+    """One quantize and ONE GEMM for layers that read the same input (q/k/v, gate/up).
+
+    The reference shares only the quantized activation between such layers
+    (SharedQuantizedInput, qlinear.py:21-37; experiments/llama.py:402-411) and still runs one
+    GEMM per layer.  Here their packed weights are concatenated along the output dimension, so
+    narrow members (Llama-2-70B k/v: 1024 columns) ride in the tiles of the wide one.  The
+    per-column arithmetic is that of the member layers, so the outputs are bit-identical to theirs.
+    forward(x) returns one tensor per member, views of a single [.., sum(out_features)] result."""
+
+    def __init__(self, layers):
+        super().__init__()
+        layers = list(layers)
+        first = layers[0]
+        for m in layers[1:]:
+            same = (m.in_features == first.in_features and m.bits == first.bits and m.symmetric == first.symmetric
+                    and m.dtype == first.dtype and m.fp_features_num == first.fp_features_num
+                    and torch.equal(m.fp_indices.cpu(), first.fp_indices.cpu())
+                    and (m.bias is None) == (first.bias is None))
+            if not same:
+                raise ValueError("FusedMixedQLinearGroup: members must agree in input size, outlier columns, "
+                                 "bits, symmetry, dtype and presence of a bias")
+        self.split_sizes = [m.out_features for m in layers]
+        total = sum(self.split_sizes)
+        fused = MixedQLinear(first.in_features, total, None, fp_features_num=first.fp_features_num,
+                             symm=first.symmetric, bits=first.bits, dtype=first.dtype, fused=True)
+        dev = first.int_weight.device
+        fused = fused.to(dev)
+        fused.int_weight = torch.cat([m.int_weight for m in layers], dim=0).contiguous()
+        fused.weights_scales = torch.cat([m.weights_scales for m in layers], dim=0).contiguous()
+        fused.int_indices = first.int_indices.clone()
+        fused.fp_indices = first.fp_indices.clone()
+        if first.fp_features_num > 0:
+            fused.fp_weight = torch.cat([m.fp_weight for m in layers], dim=0).contiguous()
+        if not first.symmetric:
+            fused.reduced_w = torch.cat([m.reduced_w for m in layers], dim=1).contiguous()
+        fused.bias = None if first.bias is None else torch.cat([m.bias for m in layers], dim=0).contiguous()
+        self.fused = fused
+
+    def forward(self, x):
+        return self.fused(x).split(self.split_sizes, dim=-1)
 
 
 class Linear8bit(torch.nn.Module):

@@ -527,6 +527,33 @@ def test_shared_quantized_input_group():
         assert (shared.qint_x is None) == (i == 2)
 
 
+@pytest.mark.parametrize("tokens,bits", [(300, 4), (8, 4), (40, 8)])
+def test_fused_group_equals_member_layers(tokens, bits):
+    """q/k/v-style group as ONE GEMM over concatenated output columns: bit-identical to the members run
+    one by one (same per-column arithmetic), for the large-tile, mid-tile and decode kernels."""
+    from quik_amd.qlinear import FusedMixedQLinearGroup
+    rng = np.random.default_rng(40 + tokens)
+    n_in, F = 1024, 64
+    mods = []
+    fi = None
+    for i, N in enumerate((512, 128, 160)):
+        W, s_w, ii, fi = _layer(np.random.default_rng(9), N, n_in, F, bits)        # same column split
+        W2, s_w2, _, _ = _layer(np.random.default_rng(100 + i), N, n_in, F, bits)  # different weights
+        codes = np.random.default_rng(200 + i).integers(-8 if bits == 4 else -127, 8 if bits == 4 else 128,
+                                                        (N, n_in - F))
+        Wm = np.zeros((N, n_in), np.float16)
+        Wm[:, ii] = (codes * s_w2.astype(np.float32)).astype(np.float16)
+        Wm[:, fi] = (0.02 * np.random.default_rng(300 + i).standard_normal((N, F))).astype(np.float16)
+        bias = np.random.default_rng(400 + i).standard_normal(N).astype(np.float16)
+        mods.append(_module(Wm, s_w2, fi, bits, bias))
+    x = _t(_acts(rng, tokens, n_in, fi).astype(np.float16))
+    group = FusedMixedQLinearGroup(mods)
+    outs = group(x)
+    assert len(outs) == 3
+    for m, o in zip(mods, outs):
+        assert torch.equal(o, m(x))
+
+
 def test_symmetric_mixed_qlinear():
     """Symmetric activations (scale = max|x| / 4 as the reference's expression evaluates):
     codes bit-exact with the oracle; fused fp32 epilogue within tolerance of the fp16-chain op."""
