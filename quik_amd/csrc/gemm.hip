@@ -13,6 +13,7 @@ namespace {
 using CfgL = Cfg<256, 256, 2, 2, 2>;   // prefill: 128x128 per wave, 256 accumulator registers
 using CfgH = Cfg<256, 128, 2, 2, 2>;   // half-width tile that evens out the last round
 using CfgM = Cfg<128, 128, 2, 2, 2>;   // mid-size problems, two workgroups per CU
+using CfgN = Cfg<128, 64, 2, 2, 2>;    // few tiles: narrower ones put more CUs to work, three workgroups per CU
 using CfgLp = Cfg<256, 256, 2, 2, 0>;  // plain fallbacks
 using CfgMp = Cfg<128, 128, 2, 2, 0>;
 
@@ -130,7 +131,7 @@ int launch_decode(const FusedArgs &p, int32_t *C, int ldc, hipStream_t st) {
 // hardware hands the next workgroup to whichever CU frees up, so the run time is the makespan of
 // that list schedule; the narrow tiles even out its end.
 struct Plan {
-  enum Kind { kSmall, kMid, kMidPlain, kLargePlain, kSplit } kind;
+  enum Kind { kSmall, kMid, kNarrow, kMidPlain, kLargePlain, kSplit } kind;
   int64_t n_wide;
 };
 
@@ -197,7 +198,12 @@ Plan make_plan(int64_t M, int64_t N, bool dma_ok) {
       best_n = n_wide;
     }
   }
-  if (M <= 128 || mid < best) return {Plan::kMid, 0};
+  if (M <= 128 || mid < best) {
+    // with few 128x128 tiles most CUs would idle: 128x64 tiles put twice as many to work
+    // (measured: 15-20 % less time up to about 130 tiles, no gain at 224)
+    const int64_t mid_tiles = ((M + 127) / 128) * ((N + 127) / 128);
+    return {mid_tiles <= 160 ? Plan::kNarrow : Plan::kMid, 0};
+  }
   return {Plan::kSplit, best_n};
 }
 
@@ -228,6 +234,7 @@ int run_i32(const uint8_t *X, const uint8_t *W, int32_t *C, int64_t M, int64_t N
       return launch_decode<MODE, false, false>(p, C, a.ldc, st);
     }
     case Plan::kMid: return launch_i32<CfgM, MODE>(a, st);
+    case Plan::kNarrow: return launch_i32<CfgN, MODE>(a, st);
     case Plan::kMidPlain: return launch_i32<CfgMp, MODE>(a, st);
     case Plan::kLargePlain: return launch_i32<CfgLp, MODE>(a, st);
     default: break;
@@ -246,6 +253,7 @@ int run_fused(const FusedArgs &p, hipStream_t st) {
   switch (plan.kind) {
     case Plan::kSmall: return launch_decode<MODE, BF16, true>(p, nullptr, 0, st);
     case Plan::kMid: return launch_fused<CfgM, MODE, BF16>(p, st);
+    case Plan::kNarrow: return launch_fused<CfgN, MODE, BF16>(p, st);
     case Plan::kMidPlain: return launch_fused<CfgMp, MODE, BF16>(p, st);
     case Plan::kLargePlain: return launch_fused<CfgLp, MODE, BF16>(p, st);
     default: break;
