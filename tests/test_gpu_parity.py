@@ -554,6 +554,66 @@ def test_fused_group_equals_member_layers(tokens, bits):
         assert torch.equal(o, m(x))
 
 
+def test_packed_state_dict_round_trip():
+    """The packed module is its own checkpoint format: buffers under the reference's names
+    (experiments/qlinear.py:53-78), saved with torch.save and loaded into a freshly constructed
+    module (no from_float) reproduce the forward bit for bit."""
+    import io
+    from quik_amd.qlinear import MixedQLinear
+    rng = np.random.default_rng(77)
+    N, n_in, F = 192, 640, 64
+    for bits, with_bias in ((4, True), (8, False)):
+        W, s_w, ii, fi = _layer(rng, N, n_in, F, bits)
+        bias = rng.standard_normal(N).astype(np.float16) if with_bias else None
+        mod = _module(W, s_w, fi, bits, bias)
+        sd = mod.state_dict()
+        names = {"weights_scales", "int_weight", "int_indices", "fp_indices", "fp_weight", "reduced_w"}
+        assert set(sd) == names | ({"bias"} if with_bias else set())
+        assert sd["int_weight"].dtype == (torch.uint8 if bits == 4 else torch.int8)
+        buf = io.BytesIO()
+        torch.save(sd, buf)
+        buf.seek(0)
+        loaded = torch.load(buf, weights_only=True)
+        fresh = MixedQLinear(n_in, N, None, fp_features_num=F, symm=False, bits=bits, dtype=torch.float16)
+        if not with_bias:
+            fresh.bias = None
+        fresh.load_state_dict(loaded)
+        fresh = fresh.to(DEV)
+        x = _t(_acts(rng, 37, n_in, fi).astype(np.float16))
+        assert torch.equal(fresh(x), mod(x))
+
+
+@pytest.mark.parametrize("bits,bf16", [(4, False), (8, False), (4, True)])
+def test_kernel_path_vs_simulated_path(bits, bf16):
+    """Accuracy cross-check of the two ways the reference evaluates a QUIK layer: the kernel path
+    (this build, on the GPU) against the fake-quant simulated path (experiments/quant_sim.py:193-256,
+    restated in oracle/sim_path.py).  The two use different zero-point conventions, so they agree to
+    quantisation noise only: both errors against the unquantised float64 layer must be of the same
+    size, and 8 bits must be far more accurate than 4."""
+    from oracle import sim_path
+    from quik_amd.qlinear import MixedQLinear
+    rng = np.random.default_rng(50 + bits)
+    M, N, n_in, F = 256, 384, 2048, 128
+    W, s_w, ii, fi = _layer(rng, N, n_in, F, bits)
+    x = _acts(rng, M, n_in, fi, "student").astype(np.float16)
+    dt = torch.bfloat16 if bf16 else torch.float16
+    Wt, st, xt = torch.from_numpy(W).to(dt), torch.from_numpy(s_w).to(dt), torch.from_numpy(x).to(dt)
+    if bf16:   # codes * scale must round-trip in the storage type
+        codes = (torch.from_numpy(W[:, ii].astype(np.float32)) / torch.from_numpy(s_w.astype(np.float32))).round()
+        Wt[:, torch.from_numpy(ii)] = (codes * st.float()).to(dt)
+    lin = torch.nn.Linear(n_in, N, bias=False)
+    mod = MixedQLinear.from_float(lin, Wt, st, None, torch.from_numpy(fi), bits=bits).to(DEV)
+    out = mod(xt.to(DEV))[0].double().cpu().numpy()
+    sim = sim_path.sim_mixed_linear(xt, Wt, torch.from_numpy(ii),
+                                    torch.from_numpy(fi), bits).double().numpy()
+    full = xt.double().numpy() @ Wt.double().numpy().T
+    rms = np.sqrt((full ** 2).mean())
+    e_ker = np.sqrt(((out - full) ** 2).mean()) / rms
+    e_sim = np.sqrt(((sim - full) ** 2).mean()) / rms
+    assert 0.5 < e_sim / e_ker < 2.0, (e_sim, e_ker)
+    assert e_ker < (0.2 if bits == 4 else 0.02), e_ker
+
+
 def test_symmetric_mixed_qlinear():
     """Symmetric activations (scale = max|x| / 4 as the reference's expression evaluates):
     codes bit-exact with the oracle; fused fp32 epilogue within tolerance of the fp16-chain op."""
