@@ -35,7 +35,7 @@ constexpr int kThreads = 256;
 
 // ---------------------------------------------------------------------------------------
 // column map layout: [src_col: num_int idx][fp_col: num_fp idx][mask: ceil(cols/32) u32]
-//                    [grp: ceil(cols/8) u32][dirty: min(num_fp, ceil(cols/8)) u32][fp_slot: num_fp u16]
+//                    [grp: ceil(cols/8) u32][dirty: min(num_fp, ceil(cols/8)) u32][dirty_grp: same count, u16]
 //                    [flags: 4 u32]
 // idx is uint16_t when cols <= 65536, else uint32_t.  Section offsets are 16-byte aligned.
 // A "group" is 8 consecutive source columns (one 16-byte load).  A group without outliers is
@@ -43,10 +43,10 @@ constexpr int kThreads = 256;
 //   grp[g]   clean: (destination column of the group's first element) << 8
 //            dirty: (slot << 8) | mask byte (bit e set = column 8g+e is an outlier)
 //   dirty[s] (destination column of the group's first non-outlier element) << 8 | mask byte
-//   fp_slot[f] = 8 * slot + e: where outlier f sits when the dirty groups are laid out by slot
+//   dirty_grp[s] the group index of dirty group s
 //   flags[0] bit 0: int_indices ascending, the two lists partition the columns and the shape
 //            fits the streaming kernel;  flags[1] = number of dirty groups.
-// grp, dirty and fp_slot exist only when cols <= kStreamMaxCols.
+// grp, dirty and dirty_grp exist only when cols <= kStreamMaxCols.
 struct ColmapLayout {
   bool idx16;
   int64_t off_fp, off_mask, off_grp, off_dirty, off_slot, off_flags, bytes;
@@ -73,7 +73,7 @@ __host__ __device__ inline ColmapLayout colmap_layout(int64_t cols, int64_t num_
   const bool stream = cols <= kStreamMaxCols;
   l.off_dirty = l.off_grp + align16(stream ? ((cols + 7) / 8) * 4 : 0);
   l.off_slot = l.off_dirty + align16(stream ? max_dirty_groups(cols, num_fp) * 4 : 0);
-  l.off_flags = l.off_slot + align16(stream ? num_fp * 2 : 0);
+  l.off_flags = l.off_slot + align16(stream ? max_dirty_groups(cols, num_fp) * 2 : 0);
   l.bytes = l.off_flags + 16;
   return l;
 }
@@ -91,7 +91,7 @@ __global__ __launch_bounds__(1024) void colmap_build_kernel(const int64_t *__res
                                                             int64_t cols, IdxT *__restrict__ src_col,
                                                             IdxT *__restrict__ fp_col, uint32_t *__restrict__ mask,
                                                             uint32_t *__restrict__ grp, uint32_t *__restrict__ dirty,
-                                                            uint16_t *__restrict__ fp_slot,
+                                                            uint16_t *__restrict__ dirty_grp,
                                                             uint32_t *__restrict__ flags) {
   // single workgroup: the mask is cleared before any bit is set
   __shared__ int ascending;
@@ -144,14 +144,11 @@ __global__ __launch_bounds__(1024) void colmap_build_kernel(const int64_t *__res
         grp[g] = dest << 8;
       } else {
         grp[g] = (slot << 8) | mb;
-        if (slot < cap) dirty[slot] = (dest << 8) | mb;
+        if (slot < cap) {
+          dirty[slot] = (dest << 8) | mb;
+          dirty_grp[slot] = static_cast<uint16_t>(g);
+        }
       }
-    }
-    __syncthreads();
-    for (int64_t j = threadIdx.x; j < num_fp; j += blockDim.x) {
-      const int64_t c = static_cast<int64_t>(fp_col[j]);
-      const uint32_t slot = grp[c >> 3] >> 8;
-      fp_slot[j] = static_cast<uint16_t>(slot < cap ? slot * 8 + (c & 7) : 0);
     }
   }
 }
@@ -337,12 +334,12 @@ __device__ __forceinline__ void gather_rows(
 // All lanes run the same branch-free code on their groups as if they were clean: packed fp16
 // min/max (a dirty group's contribution is replaced by the neutral element with one select),
 // then 8 codes per group, written as 8 bytes to the group's destination position in an LDS byte
-// buffer (only that write is predicated).  Dirty groups are also copied raw to LDS, indexed by
-// their slot, and handled by lanes 0..ndirty-1, one group each, with per-element masking: that
-// keeps the expensive masked code off the all-lanes path, where a divergent branch would make
-// every wave pay for both sides.  A last pass reads 16 code bytes per lane, packs them to
-// nibbles (int4) and writes 8 or 16 contiguous bytes per lane; outliers are read from the row
-// early in the iteration and stored at its end.
+// buffer (only that write is predicated).  Dirty groups are handled a second time by lanes
+// 0..ndirty-1, one group each, with per-element masking: that keeps the expensive masked code off
+// the all-lanes path, where a divergent branch would make every wave pay for both sides.  Those
+// lanes load their group (and every lane its outlier value) straight from the row, right after
+// the row's own loads, so the data arrives with them (same cache lines).  A last pass reads 16
+// code bytes per lane, packs them to nibbles (int4) and writes 8 or 16 contiguous bytes per lane.
 typedef _Float16 h2 __attribute__((ext_vector_type(2)));
 typedef float f2 __attribute__((ext_vector_type(2)));
 
@@ -408,10 +405,10 @@ __device__ __forceinline__ uint2 group_codes(const uint4 &v, const RowQuant<BF16
 template <int BITS, bool BF16, int NV, int TPR>
 __device__ __forceinline__ void stream_rows(const uint16_t *__restrict__ x, int64_t rows, int64_t cols,
                                             const uint32_t *__restrict__ grp, const uint32_t *__restrict__ dirty,
-                                            int ndirty, const uint16_t *__restrict__ fp_slot, int64_t num_int,
-                                            int64_t num_fp, uint8_t *__restrict__ dst, uint16_t *__restrict__ meta,
-                                            uint16_t *__restrict__ fp_x, uint8_t *codes_s, uint4 *dirty_s,
-                                            float *red, int vec_out) {
+                                            const uint16_t *__restrict__ dirty_grp, int ndirty,
+                                            const uint16_t *__restrict__ fp_col, int64_t num_int, int64_t num_fp,
+                                            uint8_t *__restrict__ dst, uint16_t *__restrict__ meta,
+                                            uint16_t *__restrict__ fp_x, uint8_t *codes_s, float *red, int vec_out) {
   const int tid = threadIdx.x;
   const int nvec = static_cast<int>(cols >> 3);
   const float inf = __builtin_inff();
@@ -421,11 +418,12 @@ __device__ __forceinline__ void stream_rows(const uint16_t *__restrict__ x, int6
   // row-invariant tables of this lane's first ND dirty groups and outliers, kept in registers so
   // that the per-row loops below wait on no global load
   constexpr int ND = 256 / TPR;
-  uint32_t my_dirty[ND], my_slot[ND];
+  uint32_t my_dirty[ND], my_dgrp[ND], my_fpcol[ND];
 #pragma unroll
   for (int k = 0; k < ND; ++k) {
     my_dirty[k] = tid + k * TPR < ndirty ? dirty[tid + k * TPR] : 0u;
-    my_slot[k] = tid + k * TPR < num_fp ? fp_slot[tid + k * TPR] : 0u;
+    my_dgrp[k] = tid + k * TPR < ndirty ? dirty_grp[tid + k * TPR] : 0u;
+    my_fpcol[k] = tid + k * TPR < num_fp ? fp_col[tid + k * TPR] : 0u;
   }
 
   auto load_row = [&](int64_t row, uint4 (&v)[NV]) {
@@ -472,7 +470,9 @@ __device__ __forceinline__ void stream_rows(const uint16_t *__restrict__ x, int6
   };
 
   // one row; `cur` holds its groups, `parity` alternates so that two sets of reduction slots are used
-  auto process = [&](int64_t row, const uint4 (&cur)[NV], int parity) {
+  auto process = [&](int64_t row, const uint4 (&cur)[NV], const uint4 (&dv)[ND], const uint16_t (&fpv)[ND],
+                     int parity) {
+    const uint4 *xv = reinterpret_cast<const uint4 *>(x + row * cols);
     // ---- all lanes: min / max as if every group were clean
     float mn = inf, mx = -inf;
     const h2 pinf = h2{static_cast<_Float16>(inf), static_cast<_Float16>(inf)};
@@ -504,29 +504,17 @@ __device__ __forceinline__ void stream_rows(const uint16_t *__restrict__ x, int6
         mx = fmaxf(mx, clean ? hi : -inf);
       }
     }
-    // ---- dirty groups go to LDS, indexed by slot
-#pragma unroll
-    for (int i = 0; i < NV; ++i) {
-      if ((g[i] & 0xFFu) != 0u && tid + i * TPR < nvec) dirty_s[g[i] >> 8] = cur[i];
-    }
-    __syncthreads();  // dirty_s complete; also: the previous row's pack pass has finished reading codes_s
-    // ---- outliers, in the caller's order (before the next barrier: the next row overwrites dirty_s)
-    const uint16_t *dirty16 = reinterpret_cast<const uint16_t *>(dirty_s);
+    // ---- outliers, in the caller's order
 #pragma unroll
     for (int k = 0; k < ND; ++k)
-      if (tid + k * TPR < num_fp) fp_x[row * num_fp + tid + k * TPR] = dirty16[my_slot[k]];
-    for (int64_t f = tid + ND * TPR; f < num_fp; f += TPR) fp_x[row * num_fp + f] = dirty16[fp_slot[f]];
-    // ---- lanes 0 .. ndirty-1: one dirty group each (more when there are more than TPR of them)
-    uint4 dv[ND];
+      if (tid + k * TPR < num_fp) fp_x[row * num_fp + tid + k * TPR] = fpv[k];
+    for (int64_t f = tid + ND * TPR; f < num_fp; f += TPR) fp_x[row * num_fp + f] = x[row * cols + fp_col[f]];
+    // ---- lanes 0 .. ndirty-1: one dirty group each (more when there are more than ND * TPR of them)
 #pragma unroll
-    for (int k = 0; k < ND; ++k) {
-      dv[k] = make_uint4(0, 0, 0, 0);
-      if (tid + k * TPR < ndirty) {
-        dv[k] = dirty_s[tid + k * TPR];
-        dirty_minmax(dv[k], my_dirty[k] & 0xFFu, pmn, pmx, mn, mx);
-      }
-    }
-    for (int j = tid + ND * TPR; j < ndirty; j += TPR) dirty_minmax(dirty_s[j], dirty[j] & 0xFFu, pmn, pmx, mn, mx);
+    for (int k = 0; k < ND; ++k)
+      if (tid + k * TPR < ndirty) dirty_minmax(dv[k], my_dirty[k] & 0xFFu, pmn, pmx, mn, mx);
+    for (int j = tid + ND * TPR; j < ndirty; j += TPR)
+      dirty_minmax(xv[dirty_grp[j]], dirty[j] & 0xFFu, pmn, pmx, mn, mx);
     if constexpr (!BF16) {
       mn = fminf(static_cast<float>(pmn.x), static_cast<float>(pmn.y));
       mx = fmaxf(static_cast<float>(pmx.x), static_cast<float>(pmx.y));
@@ -566,7 +554,7 @@ __device__ __forceinline__ void stream_rows(const uint16_t *__restrict__ x, int6
 #pragma unroll
       for (int k = 0; k < ND; ++k)
         if (tid + k * TPR < ndirty) dirty_codes(dv[k], my_dirty[k], rq, slow_c);
-      for (int j = tid + ND * TPR; j < ndirty; j += TPR) dirty_codes(dirty_s[j], dirty[j], rq, slow_c);
+      for (int j = tid + ND * TPR; j < ndirty; j += TPR) dirty_codes(xv[dirty_grp[j]], dirty[j], rq, slow_c);
     };
     if (__builtin_amdgcn_readfirstlane(rq.slow ? 1 : 0)) {
       quantise(std::true_type{});
@@ -611,9 +599,18 @@ __device__ __forceinline__ void stream_rows(const uint16_t *__restrict__ x, int6
   // different rows overlap.
   int parity = 0;
   for (int64_t row = blockIdx.x; row < rows; row += gridDim.x, parity ^= 1) {
-    uint4 cur[NV];
+    uint4 cur[NV], dv[ND];
+    uint16_t fpv[ND];
     load_row(row, cur);
-    process(row, cur, parity);
+    const uint4 *xv = reinterpret_cast<const uint4 *>(x + row * cols);
+#pragma unroll
+    for (int k = 0; k < ND; ++k) {
+      dv[k] = make_uint4(0, 0, 0, 0);
+      fpv[k] = 0;
+      if (tid + k * TPR < ndirty) dv[k] = xv[my_dgrp[k]];
+      if (tid + k * TPR < num_fp) fpv[k] = x[row * cols + my_fpcol[k]];
+    }
+    process(row, cur, dv, fpv, parity);
   }
 }
 
@@ -629,12 +626,12 @@ __global__ __launch_bounds__(kThreads) void asym_quantize_kernel(
 }
 
 // Shapes that may stream: the column map's flag (known only on the device) picks the path.
-// Dynamic LDS: max(row bytes for the gather path, code bytes + 16 bytes per possible dirty group).
+// Dynamic LDS: the row (gather path) or one byte per code (streaming path), whichever is larger.
 template <typename IdxT, int BITS, bool BF16, int NV, int TPR>
 __global__ __launch_bounds__(TPR) void asym_quantize_stream_kernel(
     const uint16_t *__restrict__ x, int64_t rows, int64_t cols, const IdxT *__restrict__ src_col,
     const IdxT *__restrict__ fp_col, const uint32_t *__restrict__ mask, const uint32_t *__restrict__ grp,
-    const uint32_t *__restrict__ dirty, const uint16_t *__restrict__ fp_slot, const uint32_t *__restrict__ flags,
+    const uint32_t *__restrict__ dirty, const uint16_t *__restrict__ dirty_grp, const uint32_t *__restrict__ flags,
     int64_t num_int, int64_t num_fp, uint8_t *__restrict__ dst, uint16_t *__restrict__ meta,
     uint16_t *__restrict__ fp_x, int vec_out) {
   static_assert(sizeof(IdxT) == 2, "streaming needs cols <= 32768");
@@ -642,9 +639,9 @@ __global__ __launch_bounds__(TPR) void asym_quantize_stream_kernel(
   __shared__ float red[16];
   if (flags[0] & 1u) {
     uint8_t *codes_s = reinterpret_cast<uint8_t *>(row_s);
-    uint4 *dirty_s = reinterpret_cast<uint4 *>(codes_s + align16(num_int));
-    stream_rows<BITS, BF16, NV, TPR>(x, rows, cols, grp, dirty, static_cast<int>(flags[1]), fp_slot, num_int, num_fp,
-                                     dst, meta, fp_x, codes_s, dirty_s, red, vec_out);
+    stream_rows<BITS, BF16, NV, TPR>(x, rows, cols, grp, dirty, dirty_grp, static_cast<int>(flags[1]),
+                                     reinterpret_cast<const uint16_t *>(fp_col), num_int, num_fp, dst, meta, fp_x,
+                                     codes_s, red, vec_out);
   } else {
     gather_rows<IdxT, BITS, BF16, TPR>(x, rows, cols, src_col, fp_col, mask, num_int, num_fp, dst, meta, fp_x, 1,
                                        row_s, red);
@@ -788,8 +785,7 @@ template <typename IdxT, int BITS, bool BF16, int NV, int TPR>
 int launch_stream(const void *x, int64_t rows, int64_t cols, const uint8_t *cm, const ColmapLayout &l, int64_t num_int,
                   int64_t num_fp, void *dst, void *meta, void *fp_x, hipStream_t st) {
   auto kern = asym_quantize_stream_kernel<IdxT, BITS, BF16, NV, TPR>;
-  const int64_t lds_stream = align16(num_int) + 16 * max_dirty_groups(cols, num_fp);
-  const int64_t lds = lds_stream > align16(cols * 2) ? lds_stream : align16(cols * 2);
+  const int64_t lds = align16(cols * 2);  // >= align16(num_int)
   if (lds > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));

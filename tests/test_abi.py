@@ -38,7 +38,7 @@ def test_argument_validation_without_gpu():
     assert lib.quik_colmap_bytes(8192, 7936, 256) > 0
     assert lib.quik_colmap_bytes(8192, 7936, 255) == 0
     # idx16 layout: src_col (2 B each), fp_col, one mask bit per column, one u32 per 8-column group, one u32 per
-    # possible dirty group (at most one per outlier), one u16 per outlier, flags;
+    # possible dirty group (at most one per outlier), one u16 per possible dirty group, flags;
     # every section 16-byte aligned
     assert lib.quik_colmap_bytes(8192, 7936, 256) == 7936 * 2 + 512 + 1024 + 4096 + 1024 + 512 + 16
     a16 = lambda v: (v + 15) // 16 * 16
