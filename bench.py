@@ -195,6 +195,31 @@ def main():
     q_b2b = e0.elapsed_time(e1) / 50
     traffic = MEASURED_TRAFFIC_BYTES.get(name, {})
 
+    # the same step replayed from a HIP graph (extra figure: what a serving loop that captures the layer sees;
+    # for small token counts the eager step is bound by Python launch overhead, not by the kernels)
+    graph_ms = None
+    try:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            step()
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            step()
+        for _ in range(3):
+            graph.replay()
+        torch.cuda.synchronize()
+        g0, g1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        g0.record()
+        for _ in range(args.steps):
+            graph.replay()
+        g1.record()
+        torch.cuda.synchronize()
+        graph_ms = g0.elapsed_time(g1) / args.steps
+    except Exception as exc:  # the figure is optional
+        print(f"bench.py: graph replay skipped: {exc}", file=sys.stderr)
+
     int_ops = 2.0 * M * N * K
     tops = int_ops / (ms_step * 1e-3) / 1e12
     gemm_tops = int_ops / (g_avg * 1e-3) / 1e12
@@ -211,6 +236,7 @@ def main():
                                f"{'fused GEMM+dequant' if mod.fused else 'unfused three-op sequence'}",
                    "M": M, "in_features": n_in, "K": K, "N": N, "F": F, "bits": bits},
         "pct_int8_mfma_peak": round(100.0 * tops / PEAK_INT8_TOPS, 2),
+        "graph_replay_ms_per_step": None if graph_ms is None else round(graph_ms, 4),
         "roofline": {"kernel": "gemm_fused_split_kernel (one launch per step)" if mod.fused
                      else "gemm_i32_split_kernel + dequantize + F.linear",
                      "bound": "mfma", "achieved": round(gemm_tops, 2), "peak": PEAK_INT8_TOPS,
