@@ -127,7 +127,7 @@ def test_asym_quantize_bit_exact(case, bits, bf16):
 
 
 def test_asym_quantize_config1_shape_and_reference_invariants():
-    """BASELINE config 1 shape (512 x 4096, 128 outliers x50) plus the reference's own checks
+    """The reference-sized single layer (512 x 4096, 128 outliers x50) plus the reference's own checks
     (test/python/test_quant.py:24-39): indexed quantize == find_meta + quantizeOld on the gathered
     columns, fp_x == x[:, fp_indices]."""
     import quik
@@ -586,7 +586,7 @@ def test_packed_state_dict_round_trip():
 @pytest.mark.parametrize("bits,bf16", [(4, False), (8, False), (4, True)])
 def test_kernel_path_vs_simulated_path(bits, bf16):
     """Accuracy cross-check of the two ways the reference evaluates a QUIK layer: the kernel path
-    (this build, on the GPU) against the fake-quant simulated path (experiments/quant_sim.py:193-256,
+    (the HIP kernels, on the GPU) against the fake-quant simulated path (experiments/quant_sim.py:193-256,
     restated in oracle/sim_path.py).  The two use different zero-point conventions, so they agree to
     quantisation noise only: both errors against the unquantised float64 layer must be of the same
     size, and 8 bits must be far more accurate than 4."""
