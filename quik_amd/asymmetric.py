@@ -11,7 +11,7 @@ import torch
 
 from . import _lib as L
 
-__all__ = ["int4FusedDequantize", "int8FusedDequantize", "quantize", "dequantize", "find_meta", "quantizeOld", "build_colmap", "quantize_mapped"]
+__all__ = ["int4FusedDequantize", "int8FusedDequantize", "quantize", "dequantize", "find_meta", "quantizeOld", "build_colmap", "quantize_mapped", "quantize_mapped_fp6", "colmap_streams"]
 
 
 def _check_bits(bits):
@@ -61,6 +61,36 @@ def quantize_mapped(src: torch.Tensor, colmap: torch.Tensor, num_int: int, num_f
         L.check(lib.quik_asym_quantize(L.ptr(src), dt, rows, cols, L.ptr(colmap), num_int, num_fp, bits, L.ptr(dst),
                                        L.ptr(meta), L.ptr(fp_x), L.stream()), "quantize")
     return dst, meta, fp_x
+
+
+def colmap_streams(colmap: torch.Tensor, num_int: int, num_fp: int) -> bool:
+    """True if the column map selects the streaming kernel (ascending int_indices that partition the
+    columns with fp_indices, cols % 8 == 0, cols <= 32768).  Synchronises once: call per layer, not per step."""
+    lib = L.load()
+    with torch.cuda.device(colmap.device):
+        rc = lib.quik_colmap_streaming(L.ptr(colmap), num_int + num_fp, num_int, num_fp, L.stream())
+    if rc < 0:
+        L.check(rc, "colmap_streams")
+    return rc == 1
+
+
+def quantize_mapped_fp6(src: torch.Tensor, colmap: torch.Tensor, num_int: int, num_fp: int):
+    """quantize_mapped with bits = 4 whose codes go to a 6-bit operand buffer for matmul.mixed_linear_fp6
+    (internal format, see include/quik_hip.h).  Returns (x6 uint8 buffer, meta, fp_x)."""
+    L.check_cuda_contiguous("quantize", src=src)
+    dt = L.dtype_id(src, "quantize", allow_bf16=True)
+    rows, cols = src.shape
+    lib = L.load()
+    nbytes = lib.quik_fp6_operand_bytes(max(rows, 1), num_int)
+    if nbytes == 0:
+        raise RuntimeError("quantize: the 6-bit operand format needs a multiple of 128 integer columns")
+    with torch.cuda.device(src.device):
+        x6 = torch.empty((nbytes,), dtype=torch.uint8, device=src.device)
+        meta = torch.empty((2 * rows,), dtype=src.dtype, device=src.device)
+        fp_x = torch.empty((rows, num_fp), dtype=src.dtype, device=src.device)
+        L.check(lib.quik_asym_quantize_fp6(L.ptr(src), dt, rows, cols, L.ptr(colmap), num_int, num_fp, L.ptr(x6),
+                                           L.ptr(meta), L.ptr(fp_x) if num_fp else None, L.stream()), "quantize")
+    return x6, meta, fp_x
 
 
 def quantize(src: torch.Tensor, int_indices: torch.Tensor, fp_indices: torch.Tensor, bits: int):

@@ -1,0 +1,66 @@
+// int4 GEMM on the 6-bit matrix-core path: weight repacking and the entry points (kernels: gemm_fp6.h,
+// operand format: fp6_format.h; the activation side is produced by the quantize kernel).
+#include "gemm_fp6.h"
+
+namespace quik {
+namespace {
+
+constexpr int kThreads = 256;
+
+// 8 nibbles of a packed int4 dword (two's complement codes) -> two dwords of level bytes
+__device__ __forceinline__ void nibbles_to_level_bytes(uint32_t w, uint32_t &lo, uint32_t &hi) {
+  w ^= 0x88888888u;  // code + 8
+  // element 2i is the low nibble of byte i: bytes (e0 e1 e2 e3) come from nibbles 0..3 = bytes 0, 1 of w
+  const uint32_t even = w & 0x0F0F0F0Fu, odd = (w >> 4) & 0x0F0F0F0Fu;   // e0 e2 e4 e6 / e1 e3 e5 e7
+  lo = __builtin_amdgcn_perm(odd, even, 0x05010400u);   // e0 e1 e2 e3
+  hi = __builtin_amdgcn_perm(odd, even, 0x07030602u);   // e4 e5 e6 e7
+}
+
+// weights [N, K/2] packed int4 -> fp6 operand buffer; one lane per fragment
+__global__ __launch_bounds__(kThreads) void pack_weight_kernel(const uint8_t *__restrict__ qw, int64_t rows, int64_t K,
+                                                               uint8_t *__restrict__ out) {
+  const Fp6Layout l = fp6_layout(rows, K);
+  const int64_t frags_per_row = l.kblocks * 4;
+  const int64_t row = blockIdx.x;
+  __shared__ int total;
+  if (threadIdx.x == 0) total = 0;
+  __syncthreads();
+  int sum = 0;
+  for (int64_t f = threadIdx.x; f < frags_per_row; f += kThreads) {
+    const uint4 v = *reinterpret_cast<const uint4 *>(qw + row * (K / 2) + f * 16);  // 32 nibbles
+    uint32_t b[8];
+    nibbles_to_level_bytes(v.x, b[0], b[1]);
+    nibbles_to_level_bytes(v.y, b[2], b[3]);
+    nibbles_to_level_bytes(v.z, b[4], b[5]);
+    nibbles_to_level_bytes(v.w, b[6], b[7]);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) sum = __builtin_amdgcn_udot4(b[i], 0x01010101u, sum, false);
+    uint32_t o[6];
+    fp6_pack_fragment(b, o);
+    fp6_store_fragment(out, l, row, f, o);
+  }
+  atomicAdd(&total, sum);
+  __syncthreads();
+  if (threadIdx.x == 0) reinterpret_cast<int32_t *>(out + l.sums_off)[row] = total;
+}
+
+}  // namespace
+}  // namespace quik
+
+using namespace quik;
+
+extern "C" int64_t quik_fp6_operand_bytes(int64_t rows, int64_t K) {
+  if (rows <= 0 || K <= 0 || K % 128 != 0) return 0;
+  return fp6_layout(rows, K).bytes;
+}
+
+extern "C" int quik_fp6_pack_weight(const uint8_t *qw, int64_t N, int64_t K, void *out, void *stream) {
+  if (N <= 0 || K <= 0) return QUIK_ERR_SHAPE;
+  if (K % 128 != 0) return QUIK_ERR_ALIGN;
+  if (!qw || !out) return QUIK_ERR_NULL;
+  if (reinterpret_cast<uintptr_t>(qw) % 16 != 0 || reinterpret_cast<uintptr_t>(out) % 16 != 0) return QUIK_ERR_ALIGN;
+  if (N > (1 << 30) || K >= 131072) return QUIK_ERR_RANGE;
+  hipLaunchKernelGGL(pack_weight_kernel, dim3(static_cast<unsigned>(N)), dim3(kThreads), 0, as_stream(stream), qw, N, K,
+                     static_cast<uint8_t *>(out));
+  return check_launch();
+}

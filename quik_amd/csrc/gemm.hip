@@ -3,6 +3,7 @@
 #include <cstdint>
 
 #include "gemm_decode.h"
+#include "gemm_fp6.h"
 #include "gemm_kernels.h"
 
 namespace quik {
@@ -247,6 +248,50 @@ int run_i32(const uint8_t *X, const uint8_t *W, int32_t *C, int64_t M, int64_t N
   return launch_i32_split<CfgL, CfgH, MODE>(wide, tail, st);
 }
 
+template <class C, bool BF16>
+int launch_fused6(const Fused6Args &p, hipStream_t st) {
+  if (p.N <= 0) return QUIK_OK;
+  int tiles_m, tiles_n;
+  const int grid = grid_of<C>(p.M, p.N, tiles_m, tiles_n);
+  auto kern = gemm_fused6_kernel<C, BF16>;
+  constexpr int smem = fused6_smem<C>();
+  if (int rc = prepare(kern, smem)) return rc;
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(C::kThreads), smem, st, p, tiles_m, tiles_n);
+  return check_launch();
+}
+
+template <class CW, class CT, bool BF16>
+int launch_fused6_split(const Fused6Args &wide, const Fused6Args &tail, hipStream_t st) {
+  if (wide.N <= 0) return launch_fused6<CT, BF16>(tail, st);
+  if (tail.N <= 0) return launch_fused6<CW, BF16>(wide, st);
+  int tail_blocks;
+  const SplitGrid grid = split_grid<CW, CT>(wide.M, wide.N, tail.N, tail_blocks);
+  auto kern = gemm_fused6_split_kernel<CW, CT, BF16>;
+  constexpr int smem = fused6_smem<CW>() > fused6_smem<CT>() ? fused6_smem<CW>() : fused6_smem<CT>();
+  if (int rc = prepare(kern, smem)) return rc;
+  hipLaunchKernelGGL(kern, dim3(grid.wide_blocks + tail_blocks), dim3(CW::kThreads), smem, st, wide, tail, grid);
+  return check_launch();
+}
+
+// The 6-bit matrix-core path (gemm_fp6.h): same tile plan, 256x256 + 256x128 tiles or 128x128 tiles.
+template <bool BF16>
+int run_fused6(const Fused6Args &p, hipStream_t st) {
+  const Plan plan = make_plan(p.M, p.N, true);
+  if (plan.kind == Plan::kSmall) return QUIK_ERR_SHAPE;  // at most 32 rows: the weight-streaming kernel is the right one
+  if (plan.kind != Plan::kSplit) return launch_fused6<CfgM, BF16>(p, st);
+  Fused6Args wide = p, tail = p;
+  const int64_t nw = plan.n_wide;
+  wide.N = static_cast<int>(nw);
+  tail.N = static_cast<int>(p.N - nw);
+  tail.n_first = static_cast<int>(nw);
+  tail.s_col = p.s_col + nw;
+  tail.w_red = p.w_red + nw;
+  tail.bias = p.bias ? p.bias + nw : nullptr;
+  tail.fp_w = p.fp_w ? p.fp_w + nw * p.F : nullptr;
+  tail.out = p.out + nw;
+  return launch_fused6_split<CfgL, CfgH, BF16>(wide, tail, st);
+}
+
 template <int MODE, bool BF16>
 int run_fused(const FusedArgs &p, hipStream_t st) {
   const Plan plan = make_plan(p.M, p.N, p.kbytes % 64 == 0 && (p.F * 2) % 64 == 0);
@@ -325,4 +370,39 @@ extern "C" int quik_mixed_linear_fwd(const void *qx, const void *qw, const void 
   hipStream_t st = as_stream(stream);
   if (bits == 4) return dtype == QUIK_F16 ? run_fused<kInt4, false>(p, st) : run_fused<kInt4, true>(p, st);
   return dtype == QUIK_F16 ? run_fused<kInt8, false>(p, st) : run_fused<kInt8, true>(p, st);
+}
+
+extern "C" int quik_mixed_linear_fwd_fp6(const void *x6, const void *w6, const void *meta, const void *s_col,
+                                         const void *w_reduced, const void *fp_x, const void *fp_w, const void *bias,
+                                         int dtype, int64_t M, int64_t N, int64_t K, int64_t F, void *out,
+                                         void *stream) {
+  if (dtype != QUIK_F16 && dtype != QUIK_BF16) return QUIK_ERR_DTYPE;
+  if (M < 0 || N < 0 || K <= 0 || F < 0) return QUIK_ERR_SHAPE;
+  if (M == 0 || N == 0) return QUIK_OK;
+  if (M <= 32) return QUIK_ERR_SHAPE;
+  if (!x6 || !w6 || !meta || !s_col || !w_reduced || !out) return QUIK_ERR_NULL;
+  if (F > 0 && (!fp_x || !fp_w)) return QUIK_ERR_NULL;
+  if (K % 128 != 0 || F % 32 != 0) return QUIK_ERR_ALIGN;
+  auto misaligned = [](const void *p) { return reinterpret_cast<uintptr_t>(p) % 16 != 0; };
+  if (misaligned(x6) || misaligned(w6) || (F > 0 && (misaligned(fp_x) || misaligned(fp_w)))) return QUIK_ERR_ALIGN;
+  if (M > (1 << 30) || N > (1 << 30) || K >= 131072) return QUIK_ERR_RANGE;
+  Fused6Args p;
+  p.xbuf = static_cast<const uint8_t *>(x6);
+  p.wbuf = static_cast<const uint8_t *>(w6);
+  p.meta = static_cast<const uint16_t *>(meta);
+  p.s_col = static_cast<const uint16_t *>(s_col);
+  p.w_red = static_cast<const uint16_t *>(w_reduced);
+  p.fp_x = static_cast<const uint16_t *>(fp_x);
+  p.fp_w = static_cast<const uint16_t *>(fp_w);
+  p.bias = static_cast<const uint16_t *>(bias);
+  p.out = static_cast<uint16_t *>(out);
+  p.M = static_cast<int>(M);
+  p.N = static_cast<int>(N);
+  p.ldo = static_cast<int>(N);
+  p.K = static_cast<int>(K);
+  p.F = static_cast<int>(F);
+  p.n_first = 0;
+  p.N_total = static_cast<int>(N);
+  hipStream_t st = as_stream(stream);
+  return dtype == QUIK_F16 ? run_fused6<false>(p, st) : run_fused6<true>(p, st);
 }

@@ -27,6 +27,7 @@
 #include <type_traits>
 
 #include "common.h"
+#include "fp6_format.h"
 
 namespace quik {
 namespace {
@@ -408,7 +409,11 @@ __device__ __forceinline__ void stream_rows(const uint16_t *__restrict__ x, int6
                                             const uint16_t *__restrict__ dirty_grp, int ndirty,
                                             const uint16_t *__restrict__ fp_col, int64_t num_int, int64_t num_fp,
                                             uint8_t *__restrict__ dst, uint16_t *__restrict__ meta,
-                                            uint16_t *__restrict__ fp_x, uint8_t *codes_s, float *red, int vec_out) {
+                                            uint16_t *__restrict__ fp_x, uint8_t *codes_s, float *red, int vec_out,
+                                            int *rowsum_s) {
+  // vec_out: 0 byte-wise output, 1 16-byte output, 2 (4 bits only): dst is a 6-bit operand buffer
+  // (fp6_format.h) for the matrix-core path of gemm_fp6.h; needs num_int % 128 == 0
+  const Fp6Layout l6 = fp6_layout(rows, num_int);
   const int tid = threadIdx.x;
   const int nvec = static_cast<int>(cols >> 3);
   const float inf = __builtin_inff();
@@ -563,7 +568,33 @@ __device__ __forceinline__ void stream_rows(const uint16_t *__restrict__ x, int6
     }
     __syncthreads();
 
-    // ---- pack pass: 16 code bytes per lane -> 8 bytes (int4) or 16 bytes (int8)
+    // ---- pack pass: 16 code bytes per lane -> 8 bytes (int4) or 16 bytes (int8), or 32 code bytes -> one
+    // 24-byte fragment of 6-bit levels
+    if (BITS == 4 && vec_out == 2) {
+      const int frags = static_cast<int>(num_int >> 5);
+      int sum = 0;
+      for (int f = tid; f < frags; f += TPR) {
+        const uint4 c0 = *reinterpret_cast<const uint4 *>(codes_s + f * 32);
+        const uint4 c1 = *reinterpret_cast<const uint4 *>(codes_s + f * 32 + 16);
+        // code nibble (two's complement) -> level = code + 8
+        const uint32_t b[8] = {c0.x ^ 0x08080808u, c0.y ^ 0x08080808u, c0.z ^ 0x08080808u, c0.w ^ 0x08080808u,
+                               c1.x ^ 0x08080808u, c1.y ^ 0x08080808u, c1.z ^ 0x08080808u, c1.w ^ 0x08080808u};
+#pragma unroll
+        for (int i = 0; i < 8; ++i) sum = __builtin_amdgcn_udot4(b[i], 0x01010101u, sum, false);
+        uint32_t o[6];
+        fp6_pack_fragment(b, o);
+        fp6_store_fragment(dst, l6, row, f, o);
+      }
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+      if ((tid & 63) == 0) atomicAdd(rowsum_s, sum);
+      __syncthreads();
+      if (tid == 0) {
+        reinterpret_cast<int32_t *>(dst + l6.sums_off)[row] = *rowsum_s;
+        *rowsum_s = 0;   // for the next row of this workgroup (ordered by that row's barriers)
+      }
+      return;
+    }
     const int units = static_cast<int>((num_int + 15) >> 4);
     for (int u = tid; u < units; u += TPR) {
       const uint4 c = *reinterpret_cast<const uint4 *>(codes_s + u * 16);
@@ -637,11 +668,13 @@ __global__ __launch_bounds__(TPR) void asym_quantize_stream_kernel(
   static_assert(sizeof(IdxT) == 2, "streaming needs cols <= 32768");
   extern __shared__ __align__(16) uint16_t row_s[];
   __shared__ float red[16];
+  __shared__ int rowsum_s;
+  if (threadIdx.x == 0) rowsum_s = 0;
   if (flags[0] & 1u) {
     uint8_t *codes_s = reinterpret_cast<uint8_t *>(row_s);
     stream_rows<BITS, BF16, NV, TPR>(x, rows, cols, grp, dirty, dirty_grp, static_cast<int>(flags[1]),
                                      reinterpret_cast<const uint16_t *>(fp_col), num_int, num_fp, dst, meta, fp_x,
-                                     codes_s, red, vec_out);
+                                     codes_s, red, vec_out, &rowsum_s);
   } else {
     gather_rows<IdxT, BITS, BF16, TPR>(x, rows, cols, src_col, fp_col, mask, num_int, num_fp, dst, meta, fp_x, 1,
                                        row_s, red);
@@ -783,7 +816,7 @@ constexpr int64_t kMaxLdsRowBytes = 128 * 1024;  // of the 160 KB per CU
 
 template <typename IdxT, int BITS, bool BF16, int NV, int TPR>
 int launch_stream(const void *x, int64_t rows, int64_t cols, const uint8_t *cm, const ColmapLayout &l, int64_t num_int,
-                  int64_t num_fp, void *dst, void *meta, void *fp_x, hipStream_t st) {
+                  int64_t num_fp, void *dst, void *meta, void *fp_x, hipStream_t st, bool fp6) {
   auto kern = asym_quantize_stream_kernel<IdxT, BITS, BF16, NV, TPR>;
   const int64_t lds = align16(cols * 2);  // >= align16(num_int)
   if (lds > 48 * 1024) {
@@ -795,7 +828,7 @@ int launch_stream(const void *x, int64_t rows, int64_t cols, const uint8_t *cm, 
     }
   }
   const int grid = static_cast<int>(rows < (int64_t(1) << 30) ? rows : (int64_t(1) << 30));
-  const int vec_out = num_int % 16 == 0 && reinterpret_cast<uintptr_t>(dst) % 16 == 0;
+  const int vec_out = fp6 ? 2 : (num_int % 16 == 0 && reinterpret_cast<uintptr_t>(dst) % 16 == 0);
   hipLaunchKernelGGL(kern, dim3(grid), dim3(TPR), static_cast<size_t>(lds), st,
                      static_cast<const uint16_t *>(x), rows, cols, reinterpret_cast<const IdxT *>(cm),
                      reinterpret_cast<const IdxT *>(cm + l.off_fp), reinterpret_cast<const uint32_t *>(cm + l.off_mask),
@@ -809,7 +842,7 @@ int launch_stream(const void *x, int64_t rows, int64_t cols, const uint8_t *cm, 
 
 template <typename IdxT, int BITS, bool BF16>
 int launch_asym(const void *x, int64_t rows, int64_t cols, const uint8_t *cm, const ColmapLayout &l, int64_t num_int,
-                int64_t num_fp, void *dst, void *meta, void *fp_x, hipStream_t st) {
+                int64_t num_fp, void *dst, void *meta, void *fp_x, hipStream_t st, bool fp6 = false) {
   const IdxT *src_col = reinterpret_cast<const IdxT *>(cm);
   const IdxT *fp_col = reinterpret_cast<const IdxT *>(cm + l.off_fp);
   const uint32_t *mask = reinterpret_cast<const uint32_t *>(cm + l.off_mask);
@@ -818,13 +851,14 @@ int launch_asym(const void *x, int64_t rows, int64_t cols, const uint8_t *cm, co
     // better than fewer waves with less per-row fixed work (measured with 64, 128 and 256 threads).
     const int64_t groups = cols / 8;
 #define QUIK_STREAM(NV) \
-  return launch_stream<IdxT, BITS, BF16, NV, kThreads>(x, rows, cols, cm, l, num_int, num_fp, dst, meta, fp_x, st)
+  return launch_stream<IdxT, BITS, BF16, NV, kThreads>(x, rows, cols, cm, l, num_int, num_fp, dst, meta, fp_x, st, fp6)
     if (groups <= 512) QUIK_STREAM(2);
     if (groups <= 1024) QUIK_STREAM(4);
     if (groups <= 2048) QUIK_STREAM(8);
     QUIK_STREAM(16);
 #undef QUIK_STREAM
   }
+  if (fp6) return QUIK_ERR_SHAPE;  // the 6-bit output exists on the streaming path only
   const int grid = static_cast<int>(rows < 65535 * 8 ? rows : 65535 * 8);
   const int64_t lds = align16(cols * 2);
   if (lds <= kMaxLdsRowBytes) {
@@ -913,6 +947,37 @@ extern "C" int quik_asym_quantize(const void *x, int dtype, int64_t rows, int64_
     QUIK_DISPATCH(uint32_t)
   }
 #undef QUIK_DISPATCH
+}
+
+extern "C" int quik_colmap_streaming(const void *colmap, int64_t cols, int64_t num_int, int64_t num_fp, void *stream) {
+  if (!colmap || cols <= 0 || num_int < 0 || num_fp < 0 || num_int + num_fp != cols) return QUIK_ERR_SHAPE;
+  const ColmapLayout l = colmap_layout(cols, num_int, num_fp);
+  uint32_t flags = 0;
+  hipStream_t st = as_stream(stream);
+  if (hipMemcpyAsync(&flags, static_cast<const uint8_t *>(colmap) + l.off_flags, sizeof(flags), hipMemcpyDeviceToHost,
+                     st) != hipSuccess ||
+      hipStreamSynchronize(st) != hipSuccess) {
+    set_last_hip_error(hipGetLastError());
+    return QUIK_ERR_LAUNCH;
+  }
+  return (flags & 1u) ? 1 : 0;
+}
+
+extern "C" int quik_asym_quantize_fp6(const void *x, int dtype, int64_t rows, int64_t cols, const void *colmap,
+                                      int64_t num_int, int64_t num_fp, void *out6, void *meta, void *fp_x,
+                                      void *stream) {
+  if (dtype != QUIK_F16 && dtype != QUIK_BF16) return QUIK_ERR_DTYPE;
+  if (rows < 0 || cols <= 0 || num_int <= 0 || num_fp < 0 || num_int + num_fp != cols) return QUIK_ERR_SHAPE;
+  if (num_int % 128 != 0 || cols % 8 != 0 || cols > kStreamMaxCols) return QUIK_ERR_ALIGN;
+  if (rows == 0) return QUIK_OK;
+  if (!x || !colmap || !out6 || !meta || (num_fp > 0 && !fp_x)) return QUIK_ERR_NULL;
+  if (reinterpret_cast<uintptr_t>(x) % 16 != 0 || reinterpret_cast<uintptr_t>(out6) % 16 != 0) return QUIK_ERR_ALIGN;
+  const ColmapLayout l = colmap_layout(cols, num_int, num_fp);
+  const uint8_t *cm = static_cast<const uint8_t *>(colmap);
+  hipStream_t st = as_stream(stream);
+  return dtype == QUIK_F16
+             ? launch_asym<uint16_t, 4, false>(x, rows, cols, cm, l, num_int, num_fp, out6, meta, fp_x, st, true)
+             : launch_asym<uint16_t, 4, true>(x, rows, cols, cm, l, num_int, num_fp, out6, meta, fp_x, st, true);
 }
 
 extern "C" int quik_asym_find_meta(const void *x, int64_t rows, int64_t cols, int bits, void *meta, void *stream) {
