@@ -123,29 +123,32 @@ int quik_sym_fused_dequantize(const void *A, const void *B, const void *scale_ro
  * and GEMM kernels.  int4 levels (code + 8) are E2M3 numbers; v_mfma_f32_32x32x64_f8f6f4 multiplies
  * them exactly at twice the int8 rate, and the integer accumulator is recovered exactly from the
  * fp32 sum and the per-row / per-column level sums, so the results are those of
- * quik_mixed_linear_fwd bit for bit.  Needs K % 128 == 0, F % 32 == 0, M > 32. */
+ * quik_mixed_linear_fwd bit for bit.  An operand buffer holds a [rows, K] int4 matrix, its [rows, F]
+ * fp16/bf16 outlier columns and the per-row level sums, in the order the GEMM tiles read them.
+ * Needs K % 128 == 0, F % 32 == 0, M > 32; operand buffers aligned to 256 bytes. */
 
-/* bytes of a 6-bit operand buffer for a [rows, K] matrix (0 if the shape is not supported) */
-int64_t quik_fp6_operand_bytes(int64_t rows, int64_t K);
+/* bytes of an operand buffer for [rows, K] int4 + [rows, F] outliers (0 if the shape is not supported) */
+int64_t quik_fp6_operand_bytes(int64_t rows, int64_t K, int64_t F);
 
-/* weights [N, K/2] nibble-packed int4 (MixedQLinear.int_weight) -> 6-bit operand buffer; once per layer */
-int quik_fp6_pack_weight(const uint8_t *qw, int64_t N, int64_t K, void *out, void *stream);
+/* weights [N, K/2] nibble-packed int4 (MixedQLinear.int_weight) and [N, F] fp16/bf16
+ * (MixedQLinear.fp_weight, may be NULL when F == 0) -> operand buffer; once per layer */
+int quik_fp6_pack_weight(const uint8_t *qw, const void *fp_w, int64_t N, int64_t K, int64_t F, void *out,
+                         void *stream);
 
 /* 1 if the column map selects the streaming quantize kernel (ascending int_indices, ...), 0 if not,
  * negative on error; copies one word from the device and synchronises the stream: call once per layer */
 int quik_colmap_streaming(const void *colmap, int64_t cols, int64_t num_int, int64_t num_fp, void *stream);
 
-/* as quik_asym_quantize with bits = 4, but the codes go to a 6-bit operand buffer [rows, num_int];
- * the column map must select the streaming kernel (quik_colmap_streaming) */
+/* as quik_asym_quantize with bits = 4, but codes and outlier values go to an operand buffer
+ * (quik_fp6_operand_bytes(rows, num_int, num_fp)); the column map must select the streaming kernel
+ * (quik_colmap_streaming) */
 int quik_asym_quantize_fp6(const void *x, int dtype, int64_t rows, int64_t cols, const void *colmap,
-                           int64_t num_int, int64_t num_fp, void *out6, void *meta, void *fp_x,
-                           void *stream);
+                           int64_t num_int, int64_t num_fp, void *out6, void *meta, void *stream);
 
-/* as quik_mixed_linear_fwd (asymmetric form, bits = 4) on 6-bit operand buffers */
+/* as quik_mixed_linear_fwd (asymmetric form, bits = 4) on operand buffers */
 int quik_mixed_linear_fwd_fp6(const void *x6, const void *w6, const void *meta, const void *s_col,
-                              const void *w_reduced, const void *fp_x, const void *fp_w,
-                              const void *bias, int dtype, int64_t M, int64_t N, int64_t K,
-                              int64_t F, void *out, void *stream);
+                              const void *w_reduced, const void *bias, int dtype, int64_t M, int64_t N,
+                              int64_t K, int64_t F, void *out, void *stream);
 
 /* quik.matmul.int4Matmul(A, B) -> C int32 [M, N]
  * replaces int4MatmulCUDA, src/matmul/matmul.cu:17-55.

@@ -75,22 +75,22 @@ def colmap_streams(colmap: torch.Tensor, num_int: int, num_fp: int) -> bool:
 
 
 def quantize_mapped_fp6(src: torch.Tensor, colmap: torch.Tensor, num_int: int, num_fp: int):
-    """quantize_mapped with bits = 4 whose codes go to a 6-bit operand buffer for matmul.mixed_linear_fp6
-    (internal format, see include/quik_hip.h).  Returns (x6 uint8 buffer, meta, fp_x)."""
+    """quantize_mapped with bits = 4 whose codes and outlier values go to an operand buffer for
+    matmul.mixed_linear_fp6 (internal format, see include/quik_hip.h).  Returns (x6 uint8 buffer, meta)."""
     L.check_cuda_contiguous("quantize", src=src)
     dt = L.dtype_id(src, "quantize", allow_bf16=True)
     rows, cols = src.shape
     lib = L.load()
-    nbytes = lib.quik_fp6_operand_bytes(max(rows, 1), num_int)
+    nbytes = lib.quik_fp6_operand_bytes(max(rows, 1), num_int, num_fp)
     if nbytes == 0:
-        raise RuntimeError("quantize: the 6-bit operand format needs a multiple of 128 integer columns")
+        raise RuntimeError("quantize: the 6-bit operand format needs a multiple of 128 integer columns and a "
+                           "multiple of 32 outlier columns")
     with torch.cuda.device(src.device):
         x6 = torch.empty((nbytes,), dtype=torch.uint8, device=src.device)
         meta = torch.empty((2 * rows,), dtype=src.dtype, device=src.device)
-        fp_x = torch.empty((rows, num_fp), dtype=src.dtype, device=src.device)
         L.check(lib.quik_asym_quantize_fp6(L.ptr(src), dt, rows, cols, L.ptr(colmap), num_int, num_fp, L.ptr(x6),
-                                           L.ptr(meta), L.ptr(fp_x) if num_fp else None, L.stream()), "quantize")
-    return x6, meta, fp_x
+                                           L.ptr(meta), L.stream()), "quantize")
+    return x6, meta
 
 
 def quantize(src: torch.Tensor, int_indices: torch.Tensor, fp_indices: torch.Tensor, bits: int):

@@ -16,12 +16,17 @@ __device__ __forceinline__ void nibbles_to_level_bytes(uint32_t w, uint32_t &lo,
   hi = __builtin_amdgcn_perm(odd, even, 0x07030602u);   // e4 e5 e6 e7
 }
 
-// weights [N, K/2] packed int4 -> fp6 operand buffer; one lane per fragment
-__global__ __launch_bounds__(kThreads) void pack_weight_kernel(const uint8_t *__restrict__ qw, int64_t rows, int64_t K,
-                                                               uint8_t *__restrict__ out) {
-  const Fp6Layout l = fp6_layout(rows, K);
-  const int64_t frags_per_row = l.kblocks * 4;
+// weights [N, K/2] packed int4 and outlier weights [N, F] (16-bit patterns) -> operand buffer; one
+// workgroup per row, one lane per fragment / 16-byte outlier chunk
+__global__ __launch_bounds__(kThreads) void pack_weight_kernel(const uint8_t *__restrict__ qw,
+                                                               const uint16_t *__restrict__ fp_w, int64_t rows,
+                                                               int64_t K, int64_t F, uint8_t *__restrict__ out) {
+  const Fp6Layout l = fp6_layout(rows, K, F);
+  const int64_t frags_per_row = l.steps * 2;
   const int64_t row = blockIdx.x;
+  for (int64_t c = threadIdx.x; c < F / 8; c += kThreads)
+    *reinterpret_cast<uint4 *>(out + fp6_outlier_offset(l, row, c >> 1, static_cast<int>(c & 1))) =
+        *reinterpret_cast<const uint4 *>(fp_w + row * F + c * 8);
   __shared__ int total;
   if (threadIdx.x == 0) total = 0;
   __syncthreads();
@@ -49,18 +54,21 @@ __global__ __launch_bounds__(kThreads) void pack_weight_kernel(const uint8_t *__
 
 using namespace quik;
 
-extern "C" int64_t quik_fp6_operand_bytes(int64_t rows, int64_t K) {
-  if (rows <= 0 || K <= 0 || K % 128 != 0) return 0;
-  return fp6_layout(rows, K).bytes;
+extern "C" int64_t quik_fp6_operand_bytes(int64_t rows, int64_t K, int64_t F) {
+  if (rows <= 0 || K <= 0 || K % 128 != 0 || F < 0 || F % 32 != 0) return 0;
+  return fp6_layout(rows, K, F).bytes;
 }
 
-extern "C" int quik_fp6_pack_weight(const uint8_t *qw, int64_t N, int64_t K, void *out, void *stream) {
-  if (N <= 0 || K <= 0) return QUIK_ERR_SHAPE;
-  if (K % 128 != 0) return QUIK_ERR_ALIGN;
-  if (!qw || !out) return QUIK_ERR_NULL;
-  if (reinterpret_cast<uintptr_t>(qw) % 16 != 0 || reinterpret_cast<uintptr_t>(out) % 16 != 0) return QUIK_ERR_ALIGN;
+extern "C" int quik_fp6_pack_weight(const uint8_t *qw, const void *fp_w, int64_t N, int64_t K, int64_t F, void *out,
+                                    void *stream) {
+  if (N <= 0 || K <= 0 || F < 0) return QUIK_ERR_SHAPE;
+  if (K % 128 != 0 || F % 32 != 0) return QUIK_ERR_ALIGN;
+  if (!qw || !out || (F > 0 && !fp_w)) return QUIK_ERR_NULL;
+  if (reinterpret_cast<uintptr_t>(qw) % 16 != 0 || reinterpret_cast<uintptr_t>(out) % 256 != 0 ||
+      reinterpret_cast<uintptr_t>(fp_w) % 16 != 0)
+    return QUIK_ERR_ALIGN;
   if (N > (1 << 30) || K >= 131072) return QUIK_ERR_RANGE;
-  hipLaunchKernelGGL(pack_weight_kernel, dim3(static_cast<unsigned>(N)), dim3(kThreads), 0, as_stream(stream), qw, N, K,
-                     static_cast<uint8_t *>(out));
+  hipLaunchKernelGGL(pack_weight_kernel, dim3(static_cast<unsigned>(N)), dim3(kThreads), 0, as_stream(stream), qw,
+                     static_cast<const uint16_t *>(fp_w), N, K, F, static_cast<uint8_t *>(out));
   return check_launch();
 }

@@ -1,27 +1,54 @@
 // 6-bit operand format of the int4 GEMM on the E2M3 matrix-core path (consumer: gemm_fp6.h).
 //
 // A level L = code + 8 (0 .. 15) is stored as a 6-bit field holding L: as an E2M3 number that is
-// L / 8.  32 fields make a 24-byte fragment, element e in bits [6 e, 6 e + 6).  Fragment g (0..3)
-// of 128-element block kb of row r keeps its first 16 bytes in heads[r][kb][16 g .. 16 g + 16)
-// and its last 8 bytes in tails[kb][g][r] (plane-major, rows padded to a multiple of 256 so that
-// a tile's 128-row loads never leave the plane); the buffer ends with one int32 per row, the sum
-// of the row's levels.
+// L / 8.  32 fields make a 24-byte fragment, element e in bits [6 e, 6 e + 6): a 16-byte head and
+// an 8-byte tail.  One MFMA k-step covers 64 elements, fragment h = 0 / 1 of the step.
+//
+// The buffer is stored in the order the GEMM copies it into LDS, so that every wave-wide copy
+// (64 lanes x 16 bytes) reads one contiguous, 1 KB aligned kilobyte: whole cache lines, each
+// fetched exactly once per tile.  Rows are grouped in blocks of 64; unit (block B, step s) is 3 KB:
+//   [0, 1024)     heads of rows 0..31 of the block: row r at 32 r, fragment h in 16-byte slot
+//                 h ^ ((r >> 3) & 1)  (the slot swap keeps 16 consecutive rows of one fragment in 16
+//                 different 16-byte bank groups of the 64-bank LDS)
+//   [1024, 2048)  the same for rows 32..63
+//   [2048, 3072)  tails: fragment h of row q (0..63) at 512 h + 8 q
+// The outlier columns (fp16 / bf16, 16 per step t, i.e. two 16-byte chunks c per row and step) follow as
+// further units of the same size whose third kilobyte is unused:
+//   [0, 1024) rows 0..31, [1024, 2048) rows 32..63, row r at 32 r, chunk c in slot c ^ ((r >> 3) & 1).
+// A block's units are contiguous: K / 64 integer steps, then F / 16 outlier steps, so the GEMM walks one
+// pointer per block through all its steps.  The buffer ends with one int32 per row: the sum of the row's
+// levels.
+// Rows of the last block beyond the matrix are never written; any bit pattern is a finite E2M3
+// or half value times results that are never stored.
 #pragma once
 #include "common.h"
 
 namespace quik {
 
 struct Fp6Layout {
-  int64_t rows_pad, kblocks, tails_off, sums_off, bytes;
+  int64_t blocks, steps, fsteps, block_bytes, sums_off, bytes;
 };
-__host__ __device__ inline Fp6Layout fp6_layout(int64_t rows, int64_t K) {
+__host__ __device__ inline Fp6Layout fp6_layout(int64_t rows, int64_t K, int64_t F) {
   Fp6Layout l;
-  l.rows_pad = (rows + 255) / 256 * 256;
-  l.kblocks = K / 128;
-  l.tails_off = (rows * l.kblocks * 64 + 255) / 256 * 256;
-  l.sums_off = l.tails_off + l.kblocks * 4 * l.rows_pad * 8;
+  l.blocks = (rows + 63) / 64;
+  l.steps = K / 64;
+  l.fsteps = F / 16;
+  l.block_bytes = (l.steps + l.fsteps) * 3072;
+  l.sums_off = l.blocks * l.block_bytes;
   l.bytes = l.sums_off + rows * 4;
   return l;
+}
+
+__host__ __device__ inline int64_t fp6_head_offset(const Fp6Layout &l, int64_t row, int64_t step, int h) {
+  return (row >> 6) * l.block_bytes + step * 3072 + ((row >> 5) & 1) * 1024 + (row & 31) * 32 +
+         ((h ^ ((row >> 3) & 1)) << 4);
+}
+__host__ __device__ inline int64_t fp6_tail_offset(const Fp6Layout &l, int64_t row, int64_t step, int h) {
+  return (row >> 6) * l.block_bytes + step * 3072 + 2048 + h * 512 + (row & 63) * 8;
+}
+// 16-byte chunk c (8 values) of outlier step t
+__host__ __device__ inline int64_t fp6_outlier_offset(const Fp6Layout &l, int64_t row, int64_t t, int c) {
+  return fp6_head_offset(l, row, l.steps + t, c);
 }
 
 // 4 levels in the bytes of w -> 24 bits, 6 per level
@@ -42,11 +69,11 @@ __device__ __forceinline__ void fp6_pack_fragment(const uint32_t (&b)[8], uint32
   out[5] = (t[6] >> 16) | (t[7] << 8);
 }
 
-// writes one fragment (index f = 4 kb + g of row `row`) into an operand buffer
+// writes fragment f = 2 step + h of row `row` into an operand buffer
 __device__ __forceinline__ void fp6_store_fragment(uint8_t *buf, const Fp6Layout &l, int64_t row, int64_t f,
                                                    const uint32_t (&o)[6]) {
-  *reinterpret_cast<uint4 *>(buf + row * l.kblocks * 64 + f * 16) = make_uint4(o[0], o[1], o[2], o[3]);
-  *reinterpret_cast<uint2 *>(buf + l.tails_off + (f * l.rows_pad + row) * 8) = make_uint2(o[4], o[5]);
+  *reinterpret_cast<uint4 *>(buf + fp6_head_offset(l, row, f >> 1, f & 1)) = make_uint4(o[0], o[1], o[2], o[3]);
+  *reinterpret_cast<uint2 *>(buf + fp6_tail_offset(l, row, f >> 1, f & 1)) = make_uint2(o[4], o[5]);
 }
 
 }  // namespace quik

@@ -287,7 +287,6 @@ int run_fused6(const Fused6Args &p, hipStream_t st) {
   tail.s_col = p.s_col + nw;
   tail.w_red = p.w_red + nw;
   tail.bias = p.bias ? p.bias + nw : nullptr;
-  tail.fp_w = p.fp_w ? p.fp_w + nw * p.F : nullptr;
   tail.out = p.out + nw;
   return launch_fused6_split<CfgL, CfgH, BF16>(wide, tail, st);
 }
@@ -373,18 +372,16 @@ extern "C" int quik_mixed_linear_fwd(const void *qx, const void *qw, const void 
 }
 
 extern "C" int quik_mixed_linear_fwd_fp6(const void *x6, const void *w6, const void *meta, const void *s_col,
-                                         const void *w_reduced, const void *fp_x, const void *fp_w, const void *bias,
-                                         int dtype, int64_t M, int64_t N, int64_t K, int64_t F, void *out,
-                                         void *stream) {
+                                         const void *w_reduced, const void *bias, int dtype, int64_t M, int64_t N,
+                                         int64_t K, int64_t F, void *out, void *stream) {
   if (dtype != QUIK_F16 && dtype != QUIK_BF16) return QUIK_ERR_DTYPE;
   if (M < 0 || N < 0 || K <= 0 || F < 0) return QUIK_ERR_SHAPE;
   if (M == 0 || N == 0) return QUIK_OK;
   if (M <= 32) return QUIK_ERR_SHAPE;
   if (!x6 || !w6 || !meta || !s_col || !w_reduced || !out) return QUIK_ERR_NULL;
-  if (F > 0 && (!fp_x || !fp_w)) return QUIK_ERR_NULL;
   if (K % 128 != 0 || F % 32 != 0) return QUIK_ERR_ALIGN;
-  auto misaligned = [](const void *p) { return reinterpret_cast<uintptr_t>(p) % 16 != 0; };
-  if (misaligned(x6) || misaligned(w6) || (F > 0 && (misaligned(fp_x) || misaligned(fp_w)))) return QUIK_ERR_ALIGN;
+  auto misaligned = [](const void *p) { return reinterpret_cast<uintptr_t>(p) % 256 != 0; };
+  if (misaligned(x6) || misaligned(w6)) return QUIK_ERR_ALIGN;
   if (M > (1 << 30) || N > (1 << 30) || K >= 131072) return QUIK_ERR_RANGE;
   Fused6Args p;
   p.xbuf = static_cast<const uint8_t *>(x6);
@@ -392,8 +389,6 @@ extern "C" int quik_mixed_linear_fwd_fp6(const void *x6, const void *w6, const v
   p.meta = static_cast<const uint16_t *>(meta);
   p.s_col = static_cast<const uint16_t *>(s_col);
   p.w_red = static_cast<const uint16_t *>(w_reduced);
-  p.fp_x = static_cast<const uint16_t *>(fp_x);
-  p.fp_w = static_cast<const uint16_t *>(fp_w);
   p.bias = static_cast<const uint16_t *>(bias);
   p.out = static_cast<uint16_t *>(out);
   p.M = static_cast<int>(M);

@@ -9,14 +9,17 @@
 // recovers the integer accumulator exactly (every term is an integer below 2^24).  From there
 // the epilogue is the one of gemm_kernels.h, so the output is bit-identical to the int8-MFMA path.
 //
-// Operand format: fp6_format.h (heads [R][K/128][64 bytes], tails plane-major, level sums).  One MFMA
-// k-step (64 elements) of a lane is fragment 2 s + h of a 128-element block: the head is one 16-byte
-// LDS read, the tail one 8-byte read, both conflict-free.
+// Operand format: fp6_format.h.  Both operand buffers are stored as the sequence of LDS images the
+// tiles need, so a copy instruction moves one contiguous kilobyte and every cache line is requested
+// once per tile (with row-major operands a 32-byte piece per row and step asks for each line four
+// times, and the 64 KB a tile touches in four steps do not survive in the 32 KB vector cache: the
+// loop was bound by the cache-to-CU path at a quarter of its rate).  One MFMA k-step (64 elements)
+// of a lane is a 16-byte head read plus an 8-byte tail read, both free of bank conflicts.
 //
 // Pipeline: a ring of 6 LDS slots, one per k-step, filled by global_load_lds_dwordx4.  While step j
 // feeds the MFMAs, the fragments of step j + 1 are read into registers, steps j + 2 .. j + 4 are
 // landing and step j + 5 is being issued; the outlier GEMM's fp16/bf16 steps (16 elements each,
-// same 32 bytes per row) run through the same ring after the integer steps.
+// 32 bytes per row like a head) run through the same ring after the integer steps.
 #pragma once
 #include "fp6_format.h"
 #include "gemm_kernels.h"
@@ -29,154 +32,141 @@ typedef int v8i __attribute__((ext_vector_type(8)));
 template <class C>
 struct Fp6Pipe {
   static constexpr int MI = C::MI, NI = C::NI, NS = 6, NF = MI + NI;
-  // per step: heads (BM + BN) x 32 bytes, tails 2 planes x (BM + BN) x 8 bytes
-  static constexpr int XH = C::BM * 32, WH = C::BN * 32, XT = C::BM * 16, WT = C::BN * 16;
-  static constexpr int XH_OFF = 0, WH_OFF = XH, XT_OFF = XH + WH, WT_OFF = XH + WH + XT;
-  static constexpr int STAGE = XH + WH + XT + WT;
+  static_assert(C::WM % 64 == 0 && C::WN % 64 == 0, "a wave's rows start at a 64-row block");
+  static_assert(C::WAVES == 4, "copy assignment below");
+  // LDS slot of one step: head images (1 KB per 32 rows) of X then W, tail images (1 KB per 64 rows) of X then W
+  static constexpr int XH_OFF = 0, WH_OFF = C::BM * 32, XT_OFF = (C::BM + C::BN) * 32, WT_OFF = XT_OFF + C::BM * 16;
+  static constexpr int STAGE = (C::BM + C::BN) * 48;
   static constexpr int SMEM = NS * STAGE;
-  static constexpr int per_wave(int bytes) { return (bytes / 1024 + C::WAVES - 1) / C::WAVES; }
-  static constexpr int XH_I = per_wave(XH), WH_I = per_wave(WH), XT_I = per_wave(XT), WT_I = per_wave(WT);
-  static constexpr int P = XH_I + WH_I + XT_I + WT_I;  // loads per wave and step
+  // Copies per step: 3 per 64-row block (head image of rows 0..31, of rows 32..63, tail image), XB + WB blocks.
+  // Every wave copies one whole block from its source A (X block w, or W block w - XB when the tile has
+  // fewer than 4 X blocks), and NB further kilobytes from its source B:
+  //   256x256: W block w (3);  256x128: W block w % 2, pieces w / 2 and w / 2 + 1 (piece 1 is copied twice);
+  //   128x128: none.
+  static constexpr int XB = C::BM / 64, WB = C::BN / 64;
+  static constexpr int NB = XB + WB == 8 ? 3 : XB + WB == 6 ? 2 : 0;
+  static_assert((XB == 4 && (WB == 4 || WB == 2)) || (XB == 2 && WB == 2), "supported tile shapes");
+  static constexpr int P = 3 + NB;  // copies per wave and step
   static_assert(3 * P <= 63, "three steps in flight must fit the vmcnt counter");
 
   uint8_t *smem;
   uint32_t lds0;
-  int wave;
-  const uint8_t *Xh, *Wh, *Xt, *Wt;      // set 0: heads / tails of the integer operands
-  const uint8_t *Xf, *Wf;                // set 1: fp16 / bf16 outlier operands
-  int64_t xt_plane, wt_plane;            // bytes from one tail plane to the next
-  uint32_t vxh[XH_I], vwh[WH_I], vxt[XT_I], vwt[WT_I], vxf[XH_I], vwf[WH_I];
-  int steps0, steps;                     // steps of set 0, of both sets
-  int x_head, w_head, x_tail, w_tail;    // this lane's fragment offsets inside a slot
+  const uint8_t *pa, *pb;   // wave-uniform: sources of the next step to be copied
+  uint32_t da[3], db[3];    // wave-uniform: destinations inside a slot
+  uint32_t fill;            // wave-uniform: LDS address of the slot the next copy fills
+  int left;                 // steps whose copy has not been issued yet
+  uint32_t voff[3];         // lane * 16 + 1024 k
+  uint32_t rd;              // byte offset of the slot the next fragment read looks at
+  int steps0, steps;        // integer steps, all steps
+  uint32_t x_head, w_head, x_tail, w_tail;  // this lane's fragment offsets inside a slot
 
-  // heads / outlier rows: 32 bytes per row and step, two 16-byte chunks; lane -> (row = lane / 2, chunk = lane % 2);
-  // chunk c of row r sits in slot c ^ ((r >> 2) & 1): eight consecutive lanes of a 16-byte read then cover all
-  // eight 16-byte bank groups
-  __device__ __forceinline__ void init(uint8_t *smem_, const uint8_t *xbuf, const Fp6Layout &lx, const uint8_t *wbuf,
-                                       const Fp6Layout &lw, int m0, int n0, int rows_x, int rows_w,
-                                       const uint8_t *fx, const uint8_t *fw, int fbytes) {
+  static __device__ __forceinline__ uint32_t dst_of(bool is_x, int blk, int piece) {
+    return piece < 2 ? (is_x ? XH_OFF : WH_OFF) + (2 * blk + piece) * 1024 : (is_x ? XT_OFF : WT_OFF) + blk * 1024;
+  }
+
+  // xb0 / wb0: first 64-row block of the tile in each operand buffer
+  __device__ __forceinline__ void init(uint8_t *smem_, const uint8_t *xbuf, const Fp6Layout &lx, int64_t xb0,
+                                       const uint8_t *wbuf, const Fp6Layout &lw, int64_t wb0) {
     smem = smem_;
     lds0 = lds_address(smem_);
     const int lane = threadIdx.x & 63;
-    wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int wm = wave / C::WAVES_N, wn = wave % C::WAVES_N;
-    const int64_t ldx = lx.kblocks * 64, ldw = lw.kblocks * 64;
-    Xh = xbuf + int64_t(m0) * ldx;
-    Wh = wbuf + int64_t(n0) * ldw;
-    Xt = xbuf + lx.tails_off + int64_t(m0) * 8;
-    Wt = wbuf + lw.tails_off + int64_t(n0) * 8;
-    xt_plane = lx.rows_pad * 8;
-    wt_plane = lw.rows_pad * 8;
-    Xf = fx, Wf = fw;
-    const int lrow = lane >> 1;
-    const int gchunk = (lane & 1) ^ ((lrow >> 2) & 1);
-    auto head_off = [&](int instr, int total, int rows_valid, int64_t ld) {
-      const int i = instr < total ? instr : total - 1;  // surplus waves repeat the last load
-      const int row = i * 32 + lrow;
-      return static_cast<uint32_t>((row < rows_valid ? row : rows_valid - 1) * ld + gchunk * 16);
+    auto block_ptr = [&](bool is_x, int blk) {
+      const Fp6Layout &l = is_x ? lx : lw;
+      int64_t B = (is_x ? xb0 : wb0) + blk;
+      B = B < l.blocks ? B : l.blocks - 1;  // blocks past the matrix: any valid block, results never stored
+      return (is_x ? xbuf : wbuf) + B * l.block_bytes;
     };
+    {
+      const bool is_x = wave < XB;
+      const int blk = is_x ? wave : wave - XB;
+      pa = block_ptr(is_x, blk);
 #pragma unroll
-    for (int j = 0; j < XH_I; ++j) {
-      vxh[j] = head_off(wave * XH_I + j, XH / 1024, rows_x, ldx);
-      vxf[j] = head_off(wave * XH_I + j, XH / 1024, rows_x, fbytes);
+      for (int k = 0; k < 3; ++k) da[k] = dst_of(is_x, blk, k);
+    }
+    pb = pa;
+    if constexpr (NB == 3) {
+      pb = block_ptr(false, wave);
+#pragma unroll
+      for (int k = 0; k < 3; ++k) db[k] = dst_of(false, wave, k);
+    } else if constexpr (NB == 2) {
+      pb = block_ptr(false, wave & 1) + (wave >> 1) * 1024;
+#pragma unroll
+      for (int k = 0; k < 2; ++k) db[k] = dst_of(false, wave & 1, (wave >> 1) + k);
     }
 #pragma unroll
-    for (int j = 0; j < WH_I; ++j) {
-      vwh[j] = head_off(wave * WH_I + j, WH / 1024, rows_w, ldw);
-      vwf[j] = head_off(wave * WH_I + j, WH / 1024, rows_w, fbytes);
-    }
-    // tails: a plane holds 8 bytes per row; one load covers 128 rows; loads [0, BM/128) are plane h = 0
-    auto tail_off = [&](int instr, int rows_tile, int64_t plane) {
-      const int per_plane = rows_tile / 128 > 0 ? rows_tile / 128 : 1;
-      const int total = 2 * per_plane;
-      const int i = instr < total ? instr : total - 1;
-      const int h = i / per_plane, part = i % per_plane;
-      return static_cast<uint32_t>(h * plane + (part * 128) * 8 + lane * 16);
-    };
-#pragma unroll
-    for (int j = 0; j < XT_I; ++j) vxt[j] = tail_off(wave * XT_I + j, C::BM, xt_plane);
-#pragma unroll
-    for (int j = 0; j < WT_I; ++j) vwt[j] = tail_off(wave * WT_I + j, C::BN, wt_plane);
-    steps0 = static_cast<int>(lx.kblocks) * 2;
-    steps = steps0 + fbytes / 32;
+    for (int k = 0; k < 3; ++k) voff[k] = lane * 16 + k * 1024;
+    fill = lds0;
+    rd = 0;
+    steps0 = static_cast<int>(lx.steps);
+    steps = steps0 + static_cast<int>(lx.fsteps);
+    left = steps;
     const int r = lane & 31, h = lane >> 5;
-    x_head = XH_OFF + (wm * C::WM + r) * 32 + ((h ^ ((r >> 2) & 1)) << 4);
-    w_head = WH_OFF + (wn * C::WN + r) * 32 + ((h ^ ((r >> 2) & 1)) << 4);
-    x_tail = XT_OFF + (h * C::BM + wm * C::WM + r) * 8;
-    w_tail = WT_OFF + (h * C::BN + wn * C::WN + r) * 8;
+    const int slot16 = (h ^ ((r >> 3) & 1)) << 4;
+    x_head = XH_OFF + (wm * C::WM + r) * 32 + slot16;
+    w_head = WH_OFF + (wn * C::WN + r) * 32 + slot16;
+    x_tail = XT_OFF + (wm * C::WM / 64) * 1024 + h * 512 + r * 8;
+    w_tail = WT_OFF + (wn * C::WN / 64) * 1024 + h * 512 + r * 8;
   }
 
-  // LDS destination of load `instr` of an operand region (surplus loads repeat the last one)
-  template <int IDX>
-  __device__ __forceinline__ void issue_one(int step) const {
-    const int st = step < steps ? step : steps - 1;
-    const uint32_t slot = lds0 + (step % NS) * STAGE;
-    const bool second = st >= steps0;
-    const int s0 = second ? steps0 - 1 : st;          // tails of outlier steps: a harmless re-load
-    const int64_t hb = second ? int64_t(st - steps0) * 32 : int64_t(st) * 32;
-    if constexpr (IDX < XH_I) {
-      const int i = wave * XH_I + IDX;
-      const int total = XH / 1024;
-      dma_load16((second ? Xf : Xh) + hb, second ? vxf[IDX] : vxh[IDX], slot + XH_OFF + (i < total ? i : total - 1) * 1024);
-    } else if constexpr (IDX < XH_I + WH_I) {
-      constexpr int J = IDX - XH_I;
-      const int i = wave * WH_I + J;
-      const int total = WH / 1024;
-      dma_load16((second ? Wf : Wh) + hb, second ? vwf[J] : vwh[J], slot + WH_OFF + (i < total ? i : total - 1) * 1024);
-    } else if constexpr (IDX < XH_I + WH_I + XT_I) {
-      constexpr int J = IDX - XH_I - WH_I;
-      const int i = wave * XT_I + J;
-      const int total = XT / 1024;
-      dma_load16(Xt + int64_t(s0) * 2 * xt_plane, vxt[J], slot + XT_OFF + (i < total ? i : total - 1) * 1024);
-    } else {
-      constexpr int J = IDX - XH_I - WH_I - XT_I;
-      const int i = wave * WT_I + J;
-      const int total = WT / 1024;
-      dma_load16(Wt + int64_t(s0) * 2 * wt_plane, vwt[J], slot + WT_OFF + (i < total ? i : total - 1) * 1024);
-    }
+  // Copies of the next step (scalar bookkeeping only: two pointer bumps, one slot bump).  Past the last step
+  // the pointers stop and the last step is copied again into a slot nobody reads.
+  __device__ __forceinline__ void issue() {
+#pragma unroll
+    for (int k = 0; k < 3; ++k) dma_load16(pa, voff[k], fill + da[k]);
+#pragma unroll
+    for (int k = 0; k < NB; ++k) dma_load16(pb, voff[k], fill + db[k]);
+    const int adv = left > 1 ? 3072 : 0;
+    left -= 1;
+    pa += adv;
+    pb += adv;
+    fill += STAGE;
+    fill = fill == lds0 + NS * STAGE ? lds0 : fill;
   }
-  template <int FIRST, int COUNT>
-  __device__ __forceinline__ void issue_range(int step) const {
-    if constexpr (COUNT > 0) {
-      issue_one<FIRST>(step);
-      issue_range<FIRST + 1, COUNT - 1>(step);
-    }
-  }
-  __device__ __forceinline__ void issue(int step) const { issue_range<0, P>(step); }
 
   // Fill the ring: afterwards steps 0 and 1 are visible and steps 2 .. 4 are in flight.
-  __device__ __forceinline__ void start() const {
-    issue(0);
-    issue(1);
-    issue(2);
-    issue(3);
-    issue(4);
+  __device__ __forceinline__ void start() {
+    issue();
+    issue();
+    issue();
+    issue();
+    issue();
     __builtin_amdgcn_s_waitcnt(vmcnt_imm(3 * P));
     __syncthreads();
   }
 
-  __device__ __forceinline__ void read6(int step, v4i (&fh)[NF], v2i (&ft)[NF]) const {
-    const uint8_t *s = smem + (step % NS) * STAGE;
+  __device__ __forceinline__ void next_read_slot() {
+    rd += STAGE;
+    rd = rd == NS * STAGE ? 0 : rd;
+  }
+  __device__ __forceinline__ void previous_read_slot() { rd = rd == 0 ? (NS - 1) * STAGE : rd - STAGE; }
+
+  // fragment j (32 rows) of this wave: head image j, tail image j / 2 at row offset 32 (j % 2)
+  __device__ __forceinline__ void read6(v4i (&fh)[NF], v2i (&ft)[NF]) {
+    const uint8_t *s = smem + rd;
 #pragma unroll
     for (int j = 0; j < NF; ++j) {
-      const int ho = j < MI ? x_head + j * 32 * 32 : w_head + (j - MI) * 32 * 32;
-      const int to = j < MI ? x_tail + j * 32 * 8 : w_tail + (j - MI) * 32 * 8;
-      fh[j] = *reinterpret_cast<const v4i *>(s + ho);
-      ft[j] = *reinterpret_cast<const v2i *>(s + to);
+      const int jj = j < MI ? j : j - MI;
+      fh[j] = *reinterpret_cast<const v4i *>(s + (j < MI ? x_head : w_head) + jj * 1024);
+      ft[j] = *reinterpret_cast<const v2i *>(s + (j < MI ? x_tail : w_tail) + (jj >> 1) * 1024 + (jj & 1) * 256);
     }
+    next_read_slot();
   }
-  __device__ __forceinline__ void read16(int step, v4i (&f)[NF]) const {
-    const uint8_t *s = smem + (step % NS) * STAGE;
+  __device__ __forceinline__ void read16(v4i (&f)[NF]) {
+    const uint8_t *s = smem + rd;
 #pragma unroll
-    for (int j = 0; j < NF; ++j) f[j] = *reinterpret_cast<const v4i *>(s + (j < MI ? x_head + j * 32 * 32 : w_head + (j - MI) * 32 * 32));
+    for (int j = 0; j < NF; ++j)
+      f[j] = *reinterpret_cast<const v4i *>(s + (j < MI ? x_head : w_head) + (j < MI ? j : j - MI) * 1024);
+    next_read_slot();
   }
 
-  // One pipeline turn after the MFMAs of step j were put in program order: the loads of step j + 5 and
-  // the scheduling pattern that spreads fragment reads and loads between the MFMAs; then wait until
+  // One pipeline turn after the MFMAs of step j were put in program order: the copies of step j + 5 and
+  // the scheduling pattern that spreads fragment reads and copies between the MFMAs; then wait until
   // step j + 2 has landed (three newer steps may stay in flight) and a barrier makes it visible.
   template <int READS>
-  __device__ __forceinline__ void turn(int j) const {
-    issue(j + 5);
+  __device__ __forceinline__ void turn() {
+    issue();
     constexpr int mfmas = MI * NI;
 #pragma unroll
     for (int i = 0; i < mfmas; ++i) {
@@ -198,18 +188,19 @@ struct Fp6Pipe {
         acc[mi][ni] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(w, x, acc[mi][ni], 2, 2, 0, 127, 0, 127);
       }
   }
-  __device__ __forceinline__ void run_fp6(v16f (&acc)[MI][NI]) const {
+  __device__ __forceinline__ void run_fp6(v16f (&acc)[MI][NI]) {
     v4i h0[NF], h1[NF];
     v2i t0[NF], t1[NF];
-    read6(0, h0, t0);
+    read6(h0, t0);
     for (int j = 0; j < steps0; j += 2) {
-      read6(j + 1, h1, t1);
+      read6(h1, t1);
       mfmas6(h0, t0, acc);
-      turn<2 * NF>(j);
-      read6(j + 2, h0, t0);
+      turn<2 * NF>();
+      read6(h0, t0);
       mfmas6(h1, t1, acc);
-      turn<2 * NF>(j + 1);
+      turn<2 * NF>();
     }
+    previous_read_slot();  // the last read looked at the first outlier step (or a dead slot) as 6-bit data
   }
 
   // Outlier steps [steps0, steps): acc += fp_w fp_x^T, 16 elements per MFMA.
@@ -222,16 +213,16 @@ struct Fp6Pipe {
       for (int mi = 0; mi < MI; ++mi) Ops::mma(f[mi], f[MI + ni], acc[mi][ni]);
   }
   template <bool BF16>
-  __device__ __forceinline__ void run_f16(v16f (&acc)[MI][NI]) const {
+  __device__ __forceinline__ void run_f16(v16f (&acc)[MI][NI]) {
     v4i f0[NF], f1[NF];
-    read16(steps0, f0);
+    read16(f0);
     for (int j = steps0; j < steps; j += 2) {
-      read16(j + 1, f1);
+      read16(f1);
       mfmas16<BF16>(f0, acc);
-      turn<NF>(j);
-      read16(j + 2, f0);
+      turn<NF>();
+      read16(f0);
       mfmas16<BF16>(f1, acc);
-      turn<NF>(j + 1);
+      turn<NF>();
     }
   }
 
@@ -242,8 +233,8 @@ struct Fp6Pipe {
 };
 
 struct Fused6Args {
-  const uint8_t *xbuf, *wbuf;  // fp6 operand buffers (activations, weights)
-  const uint16_t *meta, *s_col, *w_red, *fp_x, *fp_w, *bias;
+  const uint8_t *xbuf, *wbuf;  // operand buffers (activations, weights), outlier columns included
+  const uint16_t *meta, *s_col, *w_red, *bias;
   uint16_t *out;
   int M, N, ldo, K, F;  // N: columns of this launch (wbuf, s_col, ... start at its first column)
   int n_first;          // first column of this launch inside the weight buffer's row numbering
@@ -278,7 +269,7 @@ __device__ __forceinline__ void fused6_tile(const Fused6Args &p, int tm, int tn,
   const int m0 = tm * C::BM, n0 = tn * C::BN;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = wave / C::WAVES_N, wn = wave % C::WAVES_N;
-  const Fp6Layout lx = fp6_layout(p.M, p.K), lw = fp6_layout(p.N_total, p.K);
+  const Fp6Layout lx = fp6_layout(p.M, p.K, p.F), lw = fp6_layout(p.N_total, p.K, p.F);
   const TileVectors6<C> tv(smem + Pipe::SMEM);
   {
     const int32_t *xs = reinterpret_cast<const int32_t *>(p.xbuf + lx.sums_off);
@@ -308,10 +299,7 @@ __device__ __forceinline__ void fused6_tile(const Fused6Args &p, int tm, int tn,
       for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0.0f;
 
   Pipe pipe;
-  const int fbytes = p.F * 2;
-  pipe.init(smem, p.xbuf, lx, p.wbuf + 0, lw, m0, p.n_first + n0, p.M - m0, p.N_total - (p.n_first + n0),
-            reinterpret_cast<const uint8_t *>(p.fp_x) + int64_t(m0) * fbytes,
-            reinterpret_cast<const uint8_t *>(p.fp_w) + int64_t(n0) * fbytes, fbytes);
+  pipe.init(smem, p.xbuf, lx, m0 / 64, p.wbuf, lw, (p.n_first + n0) / 64);
   pipe.start();
   pipe.run_fp6(acc);
 

@@ -412,8 +412,10 @@ __device__ __forceinline__ void stream_rows(const uint16_t *__restrict__ x, int6
                                             uint16_t *__restrict__ fp_x, uint8_t *codes_s, float *red, int vec_out,
                                             int *rowsum_s) {
   // vec_out: 0 byte-wise output, 1 16-byte output, 2 (4 bits only): dst is a 6-bit operand buffer
-  // (fp6_format.h) for the matrix-core path of gemm_fp6.h; needs num_int % 128 == 0
-  const Fp6Layout l6 = fp6_layout(rows, num_int);
+  // (fp6_format.h) for the matrix-core path of gemm_fp6.h, which also takes the outlier values (fp_x is
+  // not written); needs num_int % 128 == 0 and num_fp % 32 == 0
+  const Fp6Layout l6 = fp6_layout(rows, num_int, num_fp);
+  const bool to6 = BITS == 4 && vec_out == 2;
   const int tid = threadIdx.x;
   const int nvec = static_cast<int>(cols >> 3);
   const float inf = __builtin_inff();
@@ -510,10 +512,14 @@ __device__ __forceinline__ void stream_rows(const uint16_t *__restrict__ x, int6
       }
     }
     // ---- outliers, in the caller's order
+    auto fp_slot = [&](int64_t f) -> uint16_t * {
+      if (!to6) return fp_x + row * num_fp + f;
+      return reinterpret_cast<uint16_t *>(dst + fp6_outlier_offset(l6, row, f >> 4, static_cast<int>((f >> 3) & 1))) + (f & 7);
+    };
 #pragma unroll
     for (int k = 0; k < ND; ++k)
-      if (tid + k * TPR < num_fp) fp_x[row * num_fp + tid + k * TPR] = fpv[k];
-    for (int64_t f = tid + ND * TPR; f < num_fp; f += TPR) fp_x[row * num_fp + f] = x[row * cols + fp_col[f]];
+      if (tid + k * TPR < num_fp) *fp_slot(tid + k * TPR) = fpv[k];
+    for (int64_t f = tid + ND * TPR; f < num_fp; f += TPR) *fp_slot(f) = x[row * cols + fp_col[f]];
     // ---- lanes 0 .. ndirty-1: one dirty group each (more when there are more than ND * TPR of them)
 #pragma unroll
     for (int k = 0; k < ND; ++k)
@@ -570,7 +576,7 @@ __device__ __forceinline__ void stream_rows(const uint16_t *__restrict__ x, int6
 
     // ---- pack pass: 16 code bytes per lane -> 8 bytes (int4) or 16 bytes (int8), or 32 code bytes -> one
     // 24-byte fragment of 6-bit levels
-    if (BITS == 4 && vec_out == 2) {
+    if (to6) {
       const int frags = static_cast<int>(num_int >> 5);
       int sum = 0;
       for (int f = tid; f < frags; f += TPR) {
@@ -628,8 +634,16 @@ __device__ __forceinline__ void stream_rows(const uint16_t *__restrict__ x, int6
   // No software prefetch: the launch makes one workgroup per row (up to the grid limit), several of
   // them are resident per CU, and their phases drift apart, so loads, arithmetic and stores of
   // different rows overlap.
+  // 6-bit output: a cache line of the operand buffer takes pieces of 4 (heads) or 16 (tails) consecutive rows.
+  // Workgroups are dealt round-robin to the 8 XCDs, so workgroup w takes row (w % 8) * rows / 8 + w / 8: rows
+  // that share lines then run at about the same time on the same XCD and meet in its L2.
+  const int64_t per_xcd = (rows + 7) >> 3;
+  const int64_t items = to6 ? per_xcd * 8 : rows;
   int parity = 0;
-  for (int64_t row = blockIdx.x; row < rows; row += gridDim.x, parity ^= 1) {
+  for (int64_t w = blockIdx.x; w < items; w += gridDim.x) {
+    const int64_t row = to6 ? (w & 7) * per_xcd + (w >> 3) : w;
+    if (row >= rows) continue;
+    parity ^= 1;
     uint4 cur[NV], dv[ND];
     uint16_t fpv[ND];
     load_row(row, cur);
@@ -827,7 +841,8 @@ int launch_stream(const void *x, int64_t rows, int64_t cols, const uint8_t *cm, 
       return QUIK_ERR_LAUNCH;
     }
   }
-  const int grid = static_cast<int>(rows < (int64_t(1) << 30) ? rows : (int64_t(1) << 30));
+  const int64_t items = fp6 ? (rows + 7) / 8 * 8 : rows;
+  const int grid = static_cast<int>(items < (int64_t(1) << 30) ? items : (int64_t(1) << 30));
   const int vec_out = fp6 ? 2 : (num_int % 16 == 0 && reinterpret_cast<uintptr_t>(dst) % 16 == 0);
   hipLaunchKernelGGL(kern, dim3(grid), dim3(TPR), static_cast<size_t>(lds), st,
                      static_cast<const uint16_t *>(x), rows, cols, reinterpret_cast<const IdxT *>(cm),
@@ -964,14 +979,14 @@ extern "C" int quik_colmap_streaming(const void *colmap, int64_t cols, int64_t n
 }
 
 extern "C" int quik_asym_quantize_fp6(const void *x, int dtype, int64_t rows, int64_t cols, const void *colmap,
-                                      int64_t num_int, int64_t num_fp, void *out6, void *meta, void *fp_x,
-                                      void *stream) {
+                                      int64_t num_int, int64_t num_fp, void *out6, void *meta, void *stream) {
   if (dtype != QUIK_F16 && dtype != QUIK_BF16) return QUIK_ERR_DTYPE;
   if (rows < 0 || cols <= 0 || num_int <= 0 || num_fp < 0 || num_int + num_fp != cols) return QUIK_ERR_SHAPE;
-  if (num_int % 128 != 0 || cols % 8 != 0 || cols > kStreamMaxCols) return QUIK_ERR_ALIGN;
+  if (num_int % 128 != 0 || num_fp % 32 != 0 || cols > kStreamMaxCols) return QUIK_ERR_ALIGN;
   if (rows == 0) return QUIK_OK;
-  if (!x || !colmap || !out6 || !meta || (num_fp > 0 && !fp_x)) return QUIK_ERR_NULL;
-  if (reinterpret_cast<uintptr_t>(x) % 16 != 0 || reinterpret_cast<uintptr_t>(out6) % 16 != 0) return QUIK_ERR_ALIGN;
+  if (!x || !colmap || !out6 || !meta) return QUIK_ERR_NULL;
+  if (reinterpret_cast<uintptr_t>(x) % 16 != 0 || reinterpret_cast<uintptr_t>(out6) % 256 != 0) return QUIK_ERR_ALIGN;
+  void *fp_x = nullptr;
   const ColmapLayout l = colmap_layout(cols, num_int, num_fp);
   const uint8_t *cm = static_cast<const uint8_t *>(colmap);
   hipStream_t st = as_stream(stream);

@@ -85,29 +85,33 @@ def mixed_linear(qx, int_weight, meta, weights_scales, reduced_w, fp_x, fp_weigh
     return out
 
 
-def pack_weight_fp6(int_weight: torch.Tensor) -> torch.Tensor:
-    """Nibble-packed int4 weights [N, K/2] -> 6-bit operand buffer for mixed_linear_fp6 (once per layer)."""
-    L.check_cuda_contiguous("pack_weight_fp6", int_weight=int_weight)
+def pack_weight_fp6(int_weight: torch.Tensor, fp_weight: torch.Tensor) -> torch.Tensor:
+    """Nibble-packed int4 weights [N, K/2] and outlier weights [N, F] -> operand buffer for mixed_linear_fp6
+    (once per layer)."""
+    L.check_cuda_contiguous("pack_weight_fp6", int_weight=int_weight, fp_weight=fp_weight)
     if int_weight.dtype != torch.uint8 or int_weight.dim() != 2:
-        raise RuntimeError("pack_weight_fp6: expected a uint8 [N, K/2] tensor")
-    N, K = int_weight.size(0), int_weight.size(1) * 2
+        raise RuntimeError("pack_weight_fp6: expected a uint8 [N, K/2] int_weight")
+    if fp_weight.dtype not in (torch.float16, torch.bfloat16) or fp_weight.dim() != 2 or \
+            fp_weight.size(0) != int_weight.size(0):
+        raise RuntimeError("pack_weight_fp6: expected an fp16/bf16 [N, F] fp_weight")
+    N, K, F = int_weight.size(0), int_weight.size(1) * 2, fp_weight.size(1)
     lib = L.load()
-    nbytes = lib.quik_fp6_operand_bytes(N, K)
+    nbytes = lib.quik_fp6_operand_bytes(N, K, F)
     if nbytes == 0:
-        raise RuntimeError("pack_weight_fp6: K must be a multiple of 128")
+        raise RuntimeError("pack_weight_fp6: K must be a multiple of 128 and F a multiple of 32")
     with torch.cuda.device(int_weight.device):
         out = torch.empty((nbytes,), dtype=torch.uint8, device=int_weight.device)
-        L.check(lib.quik_fp6_pack_weight(L.ptr(int_weight), N, K, L.ptr(out), L.stream()), "pack_weight_fp6")
+        L.check(lib.quik_fp6_pack_weight(L.ptr(int_weight), L.ptr(fp_weight) if F else None, N, K, F, L.ptr(out),
+                                         L.stream()), "pack_weight_fp6")
     return out
 
 
-def mixed_linear_fp6(x6, w6, meta, weights_scales, reduced_w, fp_x, fp_weight, bias, M, N, K, out_dtype):
-    """mixed_linear (asymmetric, 4 bits) on 6-bit operand buffers: the int4 products run on the E2M3
-    matrix-core path at twice the int8 rate; same result bit for bit."""
+def mixed_linear_fp6(x6, w6, meta, weights_scales, reduced_w, bias, M, N, K, F, out_dtype):
+    """mixed_linear (asymmetric, 4 bits) on operand buffers (asymmetric.quantize_mapped_fp6, pack_weight_fp6):
+    the int4 products run on the E2M3 matrix-core path at twice the int8 rate; same result bit for bit."""
     tensors = dict(x6=x6, w6=w6, meta=meta, weights_scales=weights_scales, reduced_w=reduced_w)
-    for name, t in (("fp_x", fp_x), ("fp_weight", fp_weight), ("bias", bias)):
-        if t is not None and t.numel() > 0:
-            tensors[name] = t
+    if bias is not None and bias.numel() > 0:
+        tensors["bias"] = bias
     L.check_cuda_contiguous("mixed_linear_fp6", **tensors)
     dt = L.QUIK_F16 if out_dtype == torch.float16 else L.QUIK_BF16 if out_dtype == torch.bfloat16 else None
     if dt is None:
@@ -115,16 +119,14 @@ def mixed_linear_fp6(x6, w6, meta, weights_scales, reduced_w, fp_x, fp_weight, b
     for name, t in tensors.items():
         if name not in ("x6", "w6") and t.dtype != out_dtype:
             raise RuntimeError(f"mixed_linear_fp6: expected {name} of dtype {out_dtype} but got {t.dtype}")
-    F = 0 if "fp_x" not in tensors else fp_x.size(1)
     lib = L.load()
-    if x6.numel() != lib.quik_fp6_operand_bytes(M, K) or w6.numel() != lib.quik_fp6_operand_bytes(N, K):
-        raise RuntimeError("mixed_linear_fp6: operand buffers do not match M, N, K")
+    if x6.numel() != lib.quik_fp6_operand_bytes(M, K, F) or w6.numel() != lib.quik_fp6_operand_bytes(N, K, F):
+        raise RuntimeError("mixed_linear_fp6: operand buffers do not match M, N, K, F")
     if meta.numel() != 2 * M or weights_scales.numel() != N or reduced_w.numel() != N:
         raise RuntimeError("mixed_linear_fp6: meta / weights_scales / reduced_w sizes are inconsistent with M, N")
     with torch.cuda.device(x6.device):
         out = torch.empty((M, N), dtype=out_dtype, device=x6.device)
         L.check(lib.quik_mixed_linear_fwd_fp6(L.ptr(x6), L.ptr(w6), L.ptr(meta), L.ptr(weights_scales),
-                                              L.ptr(reduced_w), L.ptr(fp_x) if F else None,
-                                              L.ptr(fp_weight) if F else None, L.ptr(tensors.get("bias")), dt, M, N, K,
-                                              F, L.ptr(out), L.stream()), "mixed_linear_fp6")
+                                              L.ptr(reduced_w), L.ptr(tensors.get("bias")), dt, M, N, K, F,
+                                              L.ptr(out), L.stream()), "mixed_linear_fp6")
     return out
