@@ -29,13 +29,29 @@ namespace quik {
 typedef int v2i __attribute__((ext_vector_type(2)));
 typedef int v8i __attribute__((ext_vector_type(8)));
 
+// N consecutive kilobytes global -> LDS with one LDS base: the instruction offset moves both addresses
+template <int N>
+__device__ __forceinline__ void dma_load16x(const uint8_t *sbase, uint32_t voff, uint32_t lds_addr) {
+  static_assert(N >= 1 && N <= 3, "offsets up to 2048");
+  if constexpr (N == 1) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(sbase) : "memory", "m0");
+  } else if constexpr (N == 2) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2\n\tglobal_load_lds_dwordx4 %1, %2 offset:1024"
+                 : : "s"(lds_addr), "v"(voff), "s"(sbase) : "memory", "m0");
+  } else {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2\n\tglobal_load_lds_dwordx4 %1, %2 offset:1024\n\t"
+                 "global_load_lds_dwordx4 %1, %2 offset:2048"
+                 : : "s"(lds_addr), "v"(voff), "s"(sbase) : "memory", "m0");
+  }
+}
+
 template <class C>
 struct Fp6Pipe {
   static constexpr int MI = C::MI, NI = C::NI, NS = 6, NF = MI + NI;
   static_assert(C::WM % 64 == 0 && C::WN % 64 == 0, "a wave's rows start at a 64-row block");
   static_assert(C::WAVES == 4, "copy assignment below");
-  // LDS slot of one step: head images (1 KB per 32 rows) of X then W, tail images (1 KB per 64 rows) of X then W
-  static constexpr int XH_OFF = 0, WH_OFF = C::BM * 32, XT_OFF = (C::BM + C::BN) * 32, WT_OFF = XT_OFF + C::BM * 16;
+  // LDS slot of one step: the 3 KB units of the tile's X blocks, then of its W blocks, as they are in memory
+  static constexpr int W_OFF = C::BM * 48;
   static constexpr int STAGE = (C::BM + C::BN) * 48;
   static constexpr int SMEM = NS * STAGE;
   // Copies per step: 3 per 64-row block (head image of rows 0..31, of rows 32..63, tail image), XB + WB blocks.
@@ -52,17 +68,16 @@ struct Fp6Pipe {
   uint8_t *smem;
   uint32_t lds0;
   const uint8_t *pa, *pb;   // wave-uniform: sources of the next step to be copied
-  uint32_t da[3], db[3];    // wave-uniform: destinations inside a slot
+  uint32_t da, db;          // wave-uniform: destinations inside a slot
   uint32_t fill;            // wave-uniform: LDS address of the slot the next copy fills
   int left;                 // steps whose copy has not been issued yet
-  uint32_t voff[3];         // lane * 16 + 1024 k
+  uint32_t lane16;
   uint32_t rd;              // byte offset of the slot the next fragment read looks at
   int steps0, steps;        // integer steps, all steps
-  uint32_t x_head, w_head, x_tail, w_tail;  // this lane's fragment offsets inside a slot
-
-  static __device__ __forceinline__ uint32_t dst_of(bool is_x, int blk, int piece) {
-    return piece < 2 ? (is_x ? XH_OFF : WH_OFF) + (2 * blk + piece) * 1024 : (is_x ? XT_OFF : WT_OFF) + blk * 1024;
-  }
+  uint32_t x_head, w_head;  // this lane's head offsets inside a slot (fragment j: + 1024 j)
+  uint32_t tail[NF];        // this lane's tail offsets inside a slot, one register per fragment: reads that share
+                            // a base register are paired into one 4-register read by the compiler, and the halves
+                            // then have to be copied into the operand tuples behind an exposed LDS round trip
 
   // xb0 / wb0: first 64-row block of the tile in each operand buffer
   __device__ __forceinline__ void init(uint8_t *smem_, const uint8_t *xbuf, const Fp6Layout &lx, int64_t xb0,
@@ -82,21 +97,18 @@ struct Fp6Pipe {
       const bool is_x = wave < XB;
       const int blk = is_x ? wave : wave - XB;
       pa = block_ptr(is_x, blk);
-#pragma unroll
-      for (int k = 0; k < 3; ++k) da[k] = dst_of(is_x, blk, k);
+      da = (is_x ? 0 : W_OFF) + blk * 3072;
     }
     pb = pa;
+    db = da;
     if constexpr (NB == 3) {
       pb = block_ptr(false, wave);
-#pragma unroll
-      for (int k = 0; k < 3; ++k) db[k] = dst_of(false, wave, k);
+      db = W_OFF + wave * 3072;
     } else if constexpr (NB == 2) {
       pb = block_ptr(false, wave & 1) + (wave >> 1) * 1024;
-#pragma unroll
-      for (int k = 0; k < 2; ++k) db[k] = dst_of(false, wave & 1, (wave >> 1) + k);
+      db = W_OFF + (wave & 1) * 3072 + (wave >> 1) * 1024;
     }
-#pragma unroll
-    for (int k = 0; k < 3; ++k) voff[k] = lane * 16 + k * 1024;
+    lane16 = lane * 16;
     fill = lds0;
     rd = 0;
     steps0 = static_cast<int>(lx.steps);
@@ -104,19 +116,22 @@ struct Fp6Pipe {
     left = steps;
     const int r = lane & 31, h = lane >> 5;
     const int slot16 = (h ^ ((r >> 3) & 1)) << 4;
-    x_head = XH_OFF + (wm * C::WM + r) * 32 + slot16;
-    w_head = WH_OFF + (wn * C::WN + r) * 32 + slot16;
-    x_tail = XT_OFF + (wm * C::WM / 64) * 1024 + h * 512 + r * 8;
-    w_tail = WT_OFF + (wn * C::WN / 64) * 1024 + h * 512 + r * 8;
+    x_head = (wm * C::WM / 64) * 3072 + r * 32 + slot16;
+    w_head = W_OFF + (wn * C::WN / 64) * 3072 + r * 32 + slot16;
+#pragma unroll
+    for (int j = 0; j < NF; ++j) {
+      const int jj = j < MI ? j : j - MI;
+      tail[j] = (j < MI ? (wm * C::WM / 64) * 3072 : W_OFF + (wn * C::WN / 64) * 3072) + (jj >> 1) * 3072 + 2048 +
+                h * 512 + ((jj & 1) * 32 + r) * 8;
+      asm volatile("" : "+v"(tail[j]));  // unrelated values as far as the compiler can tell
+    }
   }
 
   // Copies of the next step (scalar bookkeeping only: two pointer bumps, one slot bump).  Past the last step
   // the pointers stop and the last step is copied again into a slot nobody reads.
   __device__ __forceinline__ void issue() {
-#pragma unroll
-    for (int k = 0; k < 3; ++k) dma_load16(pa, voff[k], fill + da[k]);
-#pragma unroll
-    for (int k = 0; k < NB; ++k) dma_load16(pb, voff[k], fill + db[k]);
+    dma_load16x<3>(pa, lane16, fill + da);
+    if constexpr (NB > 0) dma_load16x<NB>(pb, lane16, fill + db);
     const int adv = left > 1 ? 3072 : 0;
     left -= 1;
     pa += adv;
@@ -148,8 +163,8 @@ struct Fp6Pipe {
 #pragma unroll
     for (int j = 0; j < NF; ++j) {
       const int jj = j < MI ? j : j - MI;
-      fh[j] = *reinterpret_cast<const v4i *>(s + (j < MI ? x_head : w_head) + jj * 1024);
-      ft[j] = *reinterpret_cast<const v2i *>(s + (j < MI ? x_tail : w_tail) + (jj >> 1) * 1024 + (jj & 1) * 256);
+      fh[j] = *reinterpret_cast<const v4i *>(s + (j < MI ? x_head : w_head) + (jj >> 1) * 3072 + (jj & 1) * 1024);
+      ft[j] = *reinterpret_cast<const v2i *>(s + tail[j]);
     }
     next_read_slot();
   }
@@ -157,7 +172,8 @@ struct Fp6Pipe {
     const uint8_t *s = smem + rd;
 #pragma unroll
     for (int j = 0; j < NF; ++j)
-      f[j] = *reinterpret_cast<const v4i *>(s + (j < MI ? x_head : w_head) + (j < MI ? j : j - MI) * 1024);
+      f[j] = *reinterpret_cast<const v4i *>(s + (j < MI ? x_head : w_head) + ((j < MI ? j : j - MI) >> 1) * 3072 +
+                                            ((j < MI ? j : j - MI) & 1) * 1024);
     next_read_slot();
   }
 
