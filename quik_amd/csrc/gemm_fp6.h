@@ -17,9 +17,10 @@
 // of a lane is a 16-byte head read plus an 8-byte tail read, both free of bank conflicts.
 //
 // Pipeline: a ring of 6 LDS slots, one per k-step, filled by global_load_lds_dwordx4.  While step j
-// feeds the MFMAs, the fragments of step j + 1 are read into registers, steps j + 2 .. j + 4 are
-// landing and step j + 5 is being issued; the outlier GEMM's fp16/bf16 steps (16 elements each,
-// 32 bytes per row like a head) run through the same ring after the integer steps.
+// feeds the MFMAs, the fragments of step j + 1 are read into registers and steps j + 2 .. j + 5 are
+// landing (the slot of step j was handed to step j + 6 when step j's reads were done); the outlier
+// GEMM's fp16/bf16 steps (16 elements each, 32 bytes per row like a head) run through the same ring
+// after the integer steps.
 #pragma once
 #include "fp6_format.h"
 #include "gemm_kernels.h"
@@ -29,20 +30,12 @@ namespace quik {
 typedef int v2i __attribute__((ext_vector_type(2)));
 typedef int v8i __attribute__((ext_vector_type(8)));
 
-// N consecutive kilobytes global -> LDS with one LDS base: the instruction offset moves both addresses
-template <int N>
-__device__ __forceinline__ void dma_load16x(const uint8_t *sbase, uint32_t voff, uint32_t lds_addr) {
-  static_assert(N >= 1 && N <= 3, "offsets up to 2048");
-  if constexpr (N == 1) {
-    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(sbase) : "memory", "m0");
-  } else if constexpr (N == 2) {
-    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2\n\tglobal_load_lds_dwordx4 %1, %2 offset:1024"
-                 : : "s"(lds_addr), "v"(voff), "s"(sbase) : "memory", "m0");
-  } else {
-    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2\n\tglobal_load_lds_dwordx4 %1, %2 offset:1024\n\t"
-                 "global_load_lds_dwordx4 %1, %2 offset:2048"
-                 : : "s"(lds_addr), "v"(voff), "s"(sbase) : "memory", "m0");
-  }
+// One wave-wide copy global -> LDS (see dma_load16) whose instruction offset moves both addresses: the three
+// kilobytes of a block unit are copied with one source pointer and one LDS base.
+template <int OFFSET>
+__device__ __forceinline__ void dma_load16k(const uint8_t *sbase, uint32_t voff, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2 offset:%3"
+               : : "s"(lds_addr), "v"(voff), "s"(sbase), "n"(OFFSET) : "memory", "m0");
 }
 
 template <class C>
@@ -127,20 +120,35 @@ struct Fp6Pipe {
     }
   }
 
-  // Copies of the next step (scalar bookkeeping only: two pointer bumps, one slot bump).  Past the last step
-  // the pointers stop and the last step is copied again into a slot nobody reads.
+  // Copy G (0 .. P-1) of the step being copied; after the last one the scalar bookkeeping: two pointer
+  // bumps and one slot bump.  Past the last step the pointers stop and the last step is copied again into
+  // a slot nobody reads.
+  template <int G>
+  __device__ __forceinline__ void issue_one() {
+    if constexpr (G < 3) {
+      dma_load16k<G * 1024>(pa, lane16, fill + da);
+    } else {
+      dma_load16k<(G - 3) * 1024>(pb, lane16, fill + db);
+    }
+    if constexpr (G == P - 1) {
+      const int adv = left > 1 ? 3072 : 0;
+      left -= 1;
+      pa += adv;
+      pb += adv;
+      fill += STAGE;
+      fill = fill == lds0 + NS * STAGE ? lds0 : fill;
+    }
+  }
+  template <int G = 0>
   __device__ __forceinline__ void issue() {
-    dma_load16x<3>(pa, lane16, fill + da);
-    if constexpr (NB > 0) dma_load16x<NB>(pb, lane16, fill + db);
-    const int adv = left > 1 ? 3072 : 0;
-    left -= 1;
-    pa += adv;
-    pb += adv;
-    fill += STAGE;
-    fill = fill == lds0 + NS * STAGE ? lds0 : fill;
+    if constexpr (G < P) {
+      issue_one<G>();
+      issue<G + 1>();
+    }
   }
 
-  // Fill the ring: afterwards steps 0 and 1 are visible and steps 2 .. 4 are in flight.
+  // Fill the ring: afterwards steps 0 and 1 are visible and steps 2 .. 4 are in flight; the copies of step 5
+  // are made during the MFMAs of step 0.
   __device__ __forceinline__ void start() {
     issue();
     issue();
@@ -158,87 +166,153 @@ struct Fp6Pipe {
   __device__ __forceinline__ void previous_read_slot() { rd = rd == 0 ? (NS - 1) * STAGE : rd - STAGE; }
 
   // fragment j (32 rows) of this wave: head image j, tail image j / 2 at row offset 32 (j % 2)
-  __device__ __forceinline__ void read6(v4i (&fh)[NF], v2i (&ft)[NF]) {
+  template <int J>
+  __device__ __forceinline__ void read6_one(v4i (&fh)[NF], v2i (&ft)[NF]) const {
+    constexpr int jj = J < MI ? J : J - MI;
     const uint8_t *s = smem + rd;
-#pragma unroll
-    for (int j = 0; j < NF; ++j) {
-      const int jj = j < MI ? j : j - MI;
-      fh[j] = *reinterpret_cast<const v4i *>(s + (j < MI ? x_head : w_head) + (jj >> 1) * 3072 + (jj & 1) * 1024);
-      ft[j] = *reinterpret_cast<const v2i *>(s + tail[j]);
-    }
-    next_read_slot();
+    fh[J] = *reinterpret_cast<const v4i *>(s + (J < MI ? x_head : w_head) + (jj >> 1) * 3072 + (jj & 1) * 1024);
+    ft[J] = *reinterpret_cast<const v2i *>(s + tail[J]);
   }
+  template <int J>
+  __device__ __forceinline__ void read16_one(v4i (&f)[NF]) const {
+    constexpr int jj = J < MI ? J : J - MI;
+    f[J] = *reinterpret_cast<const v4i *>(smem + rd + (J < MI ? x_head : w_head) + (jj >> 1) * 3072 + (jj & 1) * 1024);
+  }
+  template <int J = 0>
+  __device__ __forceinline__ void read6(v4i (&fh)[NF], v2i (&ft)[NF]) {
+    if constexpr (J < NF) {
+      read6_one<J>(fh, ft);
+      read6<J + 1>(fh, ft);
+    } else {
+      next_read_slot();
+    }
+  }
+  template <int J = 0>
   __device__ __forceinline__ void read16(v4i (&f)[NF]) {
-    const uint8_t *s = smem + rd;
-#pragma unroll
-    for (int j = 0; j < NF; ++j)
-      f[j] = *reinterpret_cast<const v4i *>(s + (j < MI ? x_head : w_head) + ((j < MI ? j : j - MI) >> 1) * 3072 +
-                                            ((j < MI ? j : j - MI) & 1) * 1024);
-    next_read_slot();
+    if constexpr (J < NF) {
+      read16_one<J>(f);
+      read16<J + 1>(f);
+    } else {
+      next_read_slot();
+    }
   }
 
-  // One pipeline turn after the MFMAs of step j were put in program order: the copies of step j + 5 and
-  // the scheduling pattern that spreads fragment reads and copies between the MFMAs; then wait until
-  // step j + 2 has landed (three newer steps may stay in flight) and a barrier makes it visible.
-  template <int READS>
-  __device__ __forceinline__ void turn() {
-    issue();
-    constexpr int mfmas = MI * NI;
+  // MFMA I (0 .. MI NI - 1) of a step: block (mi, ni) = (I % MI, I / MI)
+  template <int I>
+  static __device__ __forceinline__ void mfma6_one(const v4i (&fh)[NF], const v2i (&ft)[NF], v16f (&acc)[MI][NI]) {
+    constexpr int mi = I % MI, ni = I / MI;
+    const v8i w = v8i{fh[MI + ni].x, fh[MI + ni].y, fh[MI + ni].z, fh[MI + ni].w, ft[MI + ni].x, ft[MI + ni].y, 0, 0};
+    const v8i x = v8i{fh[mi].x, fh[mi].y, fh[mi].z, fh[mi].w, ft[mi].x, ft[mi].y, 0, 0};
+    acc[mi][ni] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(w, x, acc[mi][ni], 2, 2, 0, 127, 0, 127);
+  }
+  template <bool BF16, int I>
+  static __device__ __forceinline__ void mfma16_one(const v4i (&f)[NF], v16f (&acc)[MI][NI]) {
+    constexpr int mi = I % MI, ni = I / MI;
+    FragOps<BF16 ? kBF16 : kF16>::mma(f[mi], f[MI + ni], acc[mi][ni]);
+  }
+
+  // One step, cut into P chunks: chunk G holds its share of the step's MFMAs (on the fragments in `cur`),
+  // of the next step's fragment reads (into `nxt`) and one of the P copies of the step five ahead of the
+  // one in the MFMAs.  A copy instruction occupies the wave until the memory pipeline has taken its 64
+  // addresses; six of them in a row at the start of a step stall the MFMA issue for as long as the copies
+  // take, so they go one by one between groups of MFMAs.  Then: wait until the step after next has
+  // landed (the three newer ones stay in flight) and a barrier makes it visible; behind it every wave has
+  // issued the MFMAs of this step, which waited for their fragments, so this step's slot may be overwritten
+  // by the copies issued during the next step.
+  template <int G = 0>
+  __device__ __forceinline__ void step6(const v4i (&ch)[NF], const v2i (&ct)[NF], v4i (&nh)[NF], v2i (&nt)[NF],
+                                        v16f (&acc)[MI][NI]) {
+    constexpr int MM = MI * NI;
+    if constexpr (G < P) {
+      constexpr int r_lo = G * NF / P, r_hi = (G + 1) * NF / P, m_lo = G * MM / P, m_hi = (G + 1) * MM / P;
+      chunk_reads6<r_lo, r_hi>(nh, nt);
+      chunk_mfmas6<m_lo, m_hi>(ch, ct, acc);
 #pragma unroll
-    for (int i = 0; i < mfmas; ++i) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                   // one MFMA
-      if (i < READS) __builtin_amdgcn_sched_group_barrier(0x100, (READS + mfmas - 1) / mfmas, 0);  // LDS reads
+      for (int i = m_lo; i < m_hi; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, (2 * (r_hi - r_lo) + (m_hi - m_lo) - 1) / (m_hi - m_lo), 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      issue_one<G>();
+      __builtin_amdgcn_sched_barrier(0);
+      step6<G + 1>(ch, ct, nh, nt, acc);
+    } else {
+      next_read_slot();
+      __builtin_amdgcn_s_waitcnt(vmcnt_imm(3 * P));
+      __builtin_amdgcn_s_barrier();
     }
-    __builtin_amdgcn_s_waitcnt(vmcnt_imm(3 * P));
-    __builtin_amdgcn_s_barrier();
+  }
+  template <int LO, int HI>
+  __device__ __forceinline__ void chunk_reads6(v4i (&nh)[NF], v2i (&nt)[NF]) const {
+    if constexpr (LO < HI) {
+      read6_one<LO>(nh, nt);
+      chunk_reads6<LO + 1, HI>(nh, nt);
+    }
+  }
+  template <int LO, int HI>
+  static __device__ __forceinline__ void chunk_mfmas6(const v4i (&ch)[NF], const v2i (&ct)[NF], v16f (&acc)[MI][NI]) {
+    if constexpr (LO < HI) {
+      mfma6_one<LO>(ch, ct, acc);
+      chunk_mfmas6<LO + 1, HI>(ch, ct, acc);
+    }
+  }
+  template <bool BF16, int G = 0>
+  __device__ __forceinline__ void step16(const v4i (&cf)[NF], v4i (&nf)[NF], v16f (&acc)[MI][NI]) {
+    constexpr int MM = MI * NI;
+    if constexpr (G < P) {
+      constexpr int r_lo = G * NF / P, r_hi = (G + 1) * NF / P, m_lo = G * MM / P, m_hi = (G + 1) * MM / P;
+      chunk_reads16<r_lo, r_hi>(nf);
+      chunk_mfmas16<BF16, m_lo, m_hi>(cf, acc);
+#pragma unroll
+      for (int i = m_lo; i < m_hi; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, ((r_hi - r_lo) + (m_hi - m_lo) - 1) / (m_hi - m_lo), 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      issue_one<G>();
+      __builtin_amdgcn_sched_barrier(0);
+      step16<BF16, G + 1>(cf, nf, acc);
+    } else {
+      next_read_slot();
+      __builtin_amdgcn_s_waitcnt(vmcnt_imm(3 * P));
+      __builtin_amdgcn_s_barrier();
+    }
+  }
+  template <int LO, int HI>
+  __device__ __forceinline__ void chunk_reads16(v4i (&nf)[NF]) const {
+    if constexpr (LO < HI) {
+      read16_one<LO>(nf);
+      chunk_reads16<LO + 1, HI>(nf);
+    }
+  }
+  template <bool BF16, int LO, int HI>
+  static __device__ __forceinline__ void chunk_mfmas16(const v4i (&cf)[NF], v16f (&acc)[MI][NI]) {
+    if constexpr (LO < HI) {
+      mfma16_one<BF16, LO>(cf, acc);
+      chunk_mfmas16<BF16, LO + 1, HI>(cf, acc);
+    }
   }
 
   // Integer steps [0, steps0): acc += (Lw / 8)(Lx / 8) summed over 64 elements per MFMA.
-  static __device__ __forceinline__ void mfmas6(const v4i (&fh)[NF], const v2i (&ft)[NF], v16f (&acc)[MI][NI]) {
-#pragma unroll
-    for (int ni = 0; ni < NI; ++ni)
-#pragma unroll
-      for (int mi = 0; mi < MI; ++mi) {
-        const v8i w = v8i{fh[MI + ni].x, fh[MI + ni].y, fh[MI + ni].z, fh[MI + ni].w, ft[MI + ni].x, ft[MI + ni].y, 0, 0};
-        const v8i x = v8i{fh[mi].x, fh[mi].y, fh[mi].z, fh[mi].w, ft[mi].x, ft[mi].y, 0, 0};
-        acc[mi][ni] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(w, x, acc[mi][ni], 2, 2, 0, 127, 0, 127);
-      }
-  }
   __device__ __forceinline__ void run_fp6(v16f (&acc)[MI][NI]) {
     v4i h0[NF], h1[NF];
     v2i t0[NF], t1[NF];
     read6(h0, t0);
     for (int j = 0; j < steps0; j += 2) {
-      read6(h1, t1);
-      mfmas6(h0, t0, acc);
-      turn<2 * NF>();
-      read6(h0, t0);
-      mfmas6(h1, t1, acc);
-      turn<2 * NF>();
+      step6(h0, t0, h1, t1, acc);
+      step6(h1, t1, h0, t0, acc);
     }
     previous_read_slot();  // the last read looked at the first outlier step (or a dead slot) as 6-bit data
   }
 
   // Outlier steps [steps0, steps): acc += fp_w fp_x^T, 16 elements per MFMA.
   template <bool BF16>
-  static __device__ __forceinline__ void mfmas16(const v4i (&f)[NF], v16f (&acc)[MI][NI]) {
-    using Ops = FragOps<BF16 ? kBF16 : kF16>;
-#pragma unroll
-    for (int ni = 0; ni < NI; ++ni)
-#pragma unroll
-      for (int mi = 0; mi < MI; ++mi) Ops::mma(f[mi], f[MI + ni], acc[mi][ni]);
-  }
-  template <bool BF16>
   __device__ __forceinline__ void run_f16(v16f (&acc)[MI][NI]) {
     v4i f0[NF], f1[NF];
     read16(f0);
     for (int j = steps0; j < steps; j += 2) {
-      read16(f1);
-      mfmas16<BF16>(f0, acc);
-      turn<NF>();
-      read16(f0);
-      mfmas16<BF16>(f1, acc);
-      turn<NF>();
+      step16<BF16>(f0, f1, acc);
+      step16<BF16>(f1, f0, acc);
     }
   }
 
