@@ -490,6 +490,20 @@ struct BlockStore {
                                                int cols_valid, bool vec) {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
+    if (vec && rows_valid >= 32 && cols_valid >= C::WN) {  // interior block (wave-uniform): straight-line code
+      constexpr int kIters = 32 / kRowsPerInstr;
+      v4i piece[kIters];
+#pragma unroll
+      for (int it = 0; it < kIters; ++it)
+        piece[it] = *reinterpret_cast<const v4i *>(stage + (it * kRowsPerInstr + lane / kLanesPerRow) * kRowBytes +
+                                                   (lane % kLanesPerRow) * 16);
+#pragma unroll
+      for (int it = 0; it < kIters; ++it)
+        *reinterpret_cast<v4i *>(g + int64_t(it * kRowsPerInstr + lane / kLanesPerRow) * ld +
+                                 (lane % kLanesPerRow) * kElems) = piece[it];
+      __builtin_amdgcn_wave_barrier();
+      return;
+    }
 #pragma unroll
     for (int it = 0; it < 32 / kRowsPerInstr; ++it) {
       const int r = it * kRowsPerInstr + lane / kLanesPerRow;
