@@ -45,6 +45,7 @@ class SharedQuantizedInput:
         self.fp_x = None
         self.qscale_x = None
         self.meta = None
+        self.x6 = None  # activation in the 6-bit operand format (codes and outlier values), see MixedQLinear
         self.group_size = group_size
         self.cur_group_elem = 0
 
@@ -55,13 +56,29 @@ class SharedQuantizedInput:
             self.qscale_x = None
             self.meta = None
             self.fp_x = None
+            self.x6 = None
             self.cur_group_elem = 0
 
 
 class MixedQLinear(torch.nn.Module):
+    """The reference's layer (qlinear.py:40-145) on the HIP kernels.
+
+    W4A4 asymmetric layers with at least `six_bit_min_rows` token rows run their int4 products on the
+    6-bit (E2M3) matrix-core path, which has twice the int8 rate: levels code + 8 are exact E2M3 numbers
+    and the integer accumulator is recovered exactly, so the output is bit-identical to the int8-MFMA
+    path.  It needs int_features % 128 == 0, fp_features % 32 == 0 and ascending int_indices, and keeps a
+    second copy of the weights in the operand format of that path (0.75 bytes per int4 weight plus the
+    outlier columns, built on first use); `six_bit_path = False` turns it off."""
+
+    six_bit_min_rows = 256
+
     def __init__(self, in_features, out_features, shared_input=None,
                  fp_features_num=0, symm=False, bits=4, dtype=torch.float16, fused=True):
         super().__init__()
+        self.six_bit_path = True
+        self._w6 = None
+        self._w6_key = None
+        self._streams = None
         self.fp_features_num = fp_features_num
         self.int_features_num = in_features - fp_features_num
         self.in_features = in_features
@@ -95,7 +112,29 @@ class MixedQLinear(torch.nn.Module):
         if self._colmap is None or self._colmap_key != key:
             self._colmap = asymmetric.build_colmap(self.int_indices, self.fp_indices, self.in_features)
             self._colmap_key = key
+            self._streams = None
         return self._colmap
+
+    # -- 6-bit matrix-core path: eligibility and the cached weight operand
+    def _six_bit_ok(self, rows):
+        if not (self.six_bit_path and self.fused and not self.symmetric and self.bits == 4):
+            return False
+        if rows < self.six_bit_min_rows or self.int_features_num % 128 != 0 or self.fp_features_num % 32 != 0:
+            return False
+        colmap = self._column_map()
+        if self._streams is None:  # one device-to-host word and a stream synchronisation, once per column map
+            self._streams = asymmetric.colmap_streams(colmap, self.int_features_num, self.fp_features_num)
+        return self._streams
+
+    def _weight6(self):
+        fp_w = self.fp_weight if self.fp_features_num > 0 else \
+            torch.empty((self.out_features, 0), dtype=self.dtype, device=self.int_weight.device)
+        key = (self.int_weight.data_ptr(), self.int_weight._version, fp_w.data_ptr(), fp_w._version,
+               self.int_weight.device)
+        if self._w6 is None or self._w6_key != key:
+            self._w6 = matmul.pack_weight_fp6(self.int_weight, fp_w)
+            self._w6_key = key
+        return self._w6
 
     def _quantize_input(self, x, shared_input):
         if self.symmetric:
@@ -123,6 +162,16 @@ class MixedQLinear(torch.nn.Module):
             x2 = x2.contiguous()
         shared_input = self.shared_input if self.shared_input is not None else SharedQuantizedInput(1)
         with torch.cuda.device(x.device):
+            if x2.data_ptr() % 16 == 0 and self._six_bit_ok(x2.shape[0]):
+                if shared_input.x6 is None:
+                    shared_input.x6, shared_input.meta = asymmetric.quantize_mapped_fp6(
+                        x2, self._column_map(), self.int_features_num, self.fp_features_num)
+                output = matmul.mixed_linear_fp6(shared_input.x6, self._weight6(), shared_input.meta,
+                                                 self.weights_scales, self.reduced_w, self.bias, x2.shape[0],
+                                                 self.out_features, self.int_features_num, self.fp_features_num,
+                                                 self.dtype)
+                shared_input.finish()
+                return output.reshape(*lead, self.out_features)
             if shared_input.qint_x is None:
                 self._quantize_input(x2, shared_input)
             if self.fused:

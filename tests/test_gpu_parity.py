@@ -614,7 +614,7 @@ def test_kernel_path_vs_simulated_path(bits, bf16):
     assert e_ker < (0.2 if bits == 4 else 0.02), e_ker
 
 
-@pytest.mark.parametrize("tokens", [200, 4])
+@pytest.mark.parametrize("tokens", [300, 200, 4])     # 6-bit matrix-core path, int8-MFMA path, decode kernel
 def test_forward_under_hip_graph_replays(tokens):
     """The forward (quantize + GEMM, no allocation or synchronisation inside the library) captured in a
     HIP graph: every replay, with new input contents and eager work in between, equals the eager result."""
@@ -877,3 +877,144 @@ def test_fused_dequantize_vs_oracle_full_operand_range(bits, spread):
     want = qo.asym_fused_dequantize(acc, scale_row, scale_col, 8.0, zero_row, w_reduce, y)
     assert np.array_equal(np.isnan(got), np.isnan(want))
     assert np.array_equal(got[~np.isnan(want)].view(np.uint16), want[~np.isnan(want)].view(np.uint16))
+
+
+# ------------------------------------------------------------------------------ 6-bit matrix-core path
+def _decode_operand6(buf, rows, K, F):
+    """Operand buffer of the 6-bit path -> (levels [rows, K], outlier bit patterns [rows, F], level sums [rows]),
+    following the layout documented in quik_amd/csrc/fp6_format.h (restated here, not imported)."""
+    steps, fsteps, blocks = K // 64, F // 16, (rows + 63) // 64
+    block_bytes = (steps + fsteps) * 3072
+    assert buf.size == blocks * block_bytes + 4 * rows
+    levels = np.zeros((rows, K), np.int64)
+    outl = np.zeros((rows, F), np.uint16)
+    for r in range(rows):
+        base = (r >> 6) * block_bytes
+        head_row = ((r >> 5) & 1) * 1024 + (r & 31) * 32
+        swap = (r >> 3) & 1
+        for s in range(steps):
+            for h in range(2):
+                head = buf[base + s * 3072 + head_row + ((h ^ swap) << 4):][:16]
+                tail = buf[base + s * 3072 + 2048 + h * 512 + (r & 63) * 8:][:8]
+                word = int.from_bytes(bytes(head) + bytes(tail), "little")
+                levels[r, s * 64 + h * 32: s * 64 + h * 32 + 32] = [(word >> (6 * e)) & 63 for e in range(32)]
+        for t in range(fsteps):
+            for c in range(2):
+                chunk = buf[base + (steps + t) * 3072 + head_row + ((c ^ swap) << 4):][:16]
+                outl[r, t * 16 + c * 8: t * 16 + c * 8 + 8] = np.frombuffer(bytes(chunk), np.uint16)
+    sums = np.frombuffer(bytes(buf[blocks * block_bytes:]), np.int32)
+    return levels, outl, sums
+
+
+@pytest.mark.parametrize("rows,K,F,bf16", [(70, 256, 32, False), (130, 128, 64, True), (64, 384, 0, False)])
+def test_six_bit_operand_buffers_hold_the_int4_codes(rows, K, F, bf16):
+    """quantize_mapped_fp6 and pack_weight_fp6 write the codes of quantize_mapped / int_weight (bit-exact against
+    the oracle elsewhere) as levels code + 8, the outlier values and the level sums, in the documented layout."""
+    from quik_amd import asymmetric, matmul
+    rng = np.random.default_rng(rows + K + F)
+    n_in = K + F
+    ii, fi = _split(rng, n_in, F)
+    x = _acts(rng, rows, n_in, fi).astype(np.float16)
+    if rows >= 8:
+        x = _edge_rows(x, ii)
+    xt = _bf16_t(x.astype(np.float32)) if bf16 else _t(x)
+    colmap = asymmetric.build_colmap(_t(ii), _t(fi), n_in)
+    assert asymmetric.colmap_streams(colmap, K, F)
+    q, meta, fp_x = asymmetric.quantize_mapped(xt, colmap, K, F, 4)
+    x6, meta6 = asymmetric.quantize_mapped_fp6(xt, colmap, K, F)
+    assert np.array_equal(_bits(meta), _bits(meta6))
+    qn = q.cpu().numpy()
+    want = np.empty((rows, K), np.int64)
+    want[:, 0::2] = (qn & 0xF) ^ 8
+    want[:, 1::2] = (qn >> 4) ^ 8
+    levels, outl, sums = _decode_operand6(x6.cpu().numpy(), rows, K, F)
+    assert np.array_equal(levels, want)
+    assert np.array_equal(outl, _bits(fp_x).reshape(rows, F))
+    assert np.array_equal(sums, want.sum(1))
+    # weights
+    N = rows
+    qw = rng.integers(0, 256, (N, K // 2)).astype(np.uint8)
+    fpw = (0.02 * rng.standard_normal((N, F))).astype(np.float16)
+    fpw_t = _bf16_t(fpw.astype(np.float32)) if bf16 else _t(fpw)
+    w6 = matmul.pack_weight_fp6(_t(qw), fpw_t)
+    want = np.empty((N, K), np.int64)
+    want[:, 0::2] = (qw & 0xF) ^ 8
+    want[:, 1::2] = (qw >> 4) ^ 8
+    levels, outl, sums = _decode_operand6(w6.cpu().numpy(), N, K, F)
+    assert np.array_equal(levels, want)
+    assert np.array_equal(outl, _bits(fpw_t).reshape(N, F))
+    assert np.array_equal(sums, want.sum(1))
+
+
+SIX_CASES = [
+    # M, N, in, F, bias, kind: K = in - F a multiple of 128, F a multiple of 32, M >= 256
+    (256, 256, 384, 128, True, "x50"),        # one 128x128-tile round, two integer steps
+    (300, 520, 1088, 64, False, "student"),   # ragged M and N
+    (257, 130, 544, 32, True, "x50"),         # two outlier steps, N below a tile
+    (512, 1024, 1024, 0, True, "x50"),        # no outlier columns
+    (1000, 4160, 4096, 256, True, "x50"),     # 256x256 and 256x128 tiles in one launch, ragged M, N = 32.5 tiles
+    (2048, 1280, 2048 + 96, 96, False, "x50"),
+]
+
+
+@pytest.mark.parametrize("case", SIX_CASES)
+@pytest.mark.parametrize("bf16", [False, True])
+def test_six_bit_path_is_bit_identical_to_the_int8_path(case, bf16):
+    """MixedQLinear on the 6-bit (E2M3) matrix-core path against the same layer on the int8-MFMA path (which the
+    other tests hold against the oracle): identical output bits, NaN / Inf rows included."""
+    from quik_amd.qlinear import MixedQLinear
+    M, N, n_in, F, with_bias, kind = case
+    rng = np.random.default_rng(sum(case[:4]) + bf16)
+    W, s_w, ii, fi = _layer(rng, N, n_in, F, 4)
+    bias = rng.standard_normal(N).astype(np.float16) if with_bias else None
+    x = _edge_rows(_acts(rng, M, n_in, fi, kind).astype(np.float16), ii)
+    mods = []
+    for six in (True, False):
+        mod = _module(W, s_w, fi, 4, bias)
+        if bf16:
+            mod = mod.to(torch.bfloat16)
+            mod.dtype = torch.bfloat16
+        mod.six_bit_path = six
+        mods.append(mod)
+    xt = _bf16_t(x.astype(np.float32)) if bf16 else _t(x)
+    out6, out8 = mods[0](xt), mods[1](xt)
+    assert mods[0]._w6 is not None and mods[1]._w6 is None      # the paths that were meant to run did run
+    assert out6.shape == out8.shape == (1, M, N)
+    assert np.array_equal(_bits(out6), _bits(out8))
+    if not bf16:                                                # and against the oracle, on a slice of the rows
+        omod = qo.from_float(W, s_w, fi, 4)
+        rows = np.r_[0:24, M - 8:M]
+        want, _ = qo.mixed_qlinear_forward(x[rows], omod, 4, bias)
+        got = out6[0].float().cpu().numpy()[rows]
+        fin = np.isfinite(want)
+        assert np.array_equal(np.isfinite(got), fin)
+        rms = np.sqrt((want[fin].astype(np.float64) ** 2).mean())
+        assert np.abs(got[fin].astype(np.float64) - want[fin]).max() <= 1e-2 * rms
+
+
+def test_six_bit_path_shared_input_and_fallbacks():
+    """A q/k/v-style group on the 6-bit path quantizes once into the operand format; a member with the path
+    switched off, or a call with fewer rows than the threshold, takes the int4 path, with the same results."""
+    from quik_amd.qlinear import SharedQuantizedInput
+    rng = np.random.default_rng(77)
+    n_in, F, M = 1024 + 64, 64, 320
+    shared = SharedQuantizedInput(3)
+    mods, singles = [], []
+    for N in (256, 128, 384):
+        W, s_w, ii, fi = _layer(np.random.default_rng(6), N, n_in, F, 4)
+        mods.append(_module(W, s_w, fi, 4, shared=shared))
+        single = _module(W, s_w, fi, 4)
+        single.six_bit_path = False
+        singles.append(single)
+    xt = _t(_acts(rng, M, n_in, fi).astype(np.float16))
+    for i, (m, s) in enumerate(zip(mods, singles)):
+        out = m(xt)
+        assert (shared.x6 is None) == (i == 2) and shared.qint_x is None
+        assert torch.equal(out, s(xt))
+    mods[1].six_bit_path = False                               # mixed group: member 1 re-quantizes to int4
+    for i, (m, s) in enumerate(zip(mods, singles)):
+        assert torch.equal(m(xt), s(xt))
+    assert shared.x6 is None and shared.qint_x is None
+    small = xt[:40].contiguous()                               # below the row threshold: int4 path, decode-size kernels
+    assert torch.equal(mods[0](small), singles[0](small))
+    shared.finish(), shared.finish()
