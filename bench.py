@@ -2,14 +2,17 @@
 """Benchmark of the MixedQLinear forward path on one MI355X.
 
 A step is one forward of the layer: the per-token asymmetric quantize kernel followed by the
-fused GEMM kernel (int4 x int4 on int8 MFMA + fp16 outlier GEMM + dequantize epilogue), on
-synthetic inputs already resident in HBM.  The default workload is the one the headline
+fused GEMM kernel (int4 x int4 + fp16 outlier GEMM + dequantize epilogue), on synthetic inputs
+already resident in HBM.  W4A4 layers with 256 or more token rows take the path MixedQLinear takes:
+the int4 products run on the 6-bit (E2M3) matrix-core instructions, exactly (--int8-mfma forces the
+int8 MFMA path, which has the same output bits).  The default workload is the one the headline
 metric is quoted on: Llama-2-70B gate_proj, 8192 -> 28672, 2048 tokens, 256 fp16 outlier
 columns, W4A4 asymmetric activations.
 
 Prints ONE JSON line.  value = 2*M*N*K / t_step in TOPS (the integer GEMM's operations over the
 whole forward time; the outlier GEMM's 2*M*N*F flops are not counted).  `roofline` is for the
-dominant kernel (the fused GEMM, bounded by the int8 MFMA peak); `roofline_quantize` for the
+dominant kernel (the fused GEMM, priced against the peak of the MFMA instructions it issues: 10.1 POP/s
+for the 6-bit path, 5.0 POP/s for int8); `roofline_quantize` for the
 quantize kernel (bounded by HBM).  Kernel durations are measured with HIP events recorded on
 the stream the kernels run on, inside the timed region.  `cpu_baseline` times the CPU
 restatement of the reference's fake-quant path (oracle/sim_path.py) on the host cores.
@@ -46,13 +49,15 @@ WORKLOADS = {
 }
 
 PEAK_INT8_TOPS = 5000.0   # MI355X dense int8 MFMA, published
+PEAK_FP6_TOPS = 10100.0   # MI355X dense fp6 / fp4 MFMA, published
 PEAK_HBM_GBPS = 8000.0    # MI355X HBM3E, published
 
 # HBM/fabric bytes per launch from rocprofv3 counter runs of this file (FETCH_SIZE and WRITE_SIZE, each
 # scaled by what the same counter reads for a plain 256 MiB copy): offline figures, kept per workload;
-# the summaries with the commands are profiles/*__llama2-70b.gate_proj.md and profiles/copy_calibration__256MiB.md
+# the summaries with the commands are profiles/*__llama2-70b.gate_proj*.md and profiles/copy_calibration__256MiB.md
+# (gemm6 / quantize6: the kernels of the 6-bit matrix-core path, the default; gemm / quantize: --int8-mfma)
 MEASURED_TRAFFIC_BYTES = {
-    "llama2-70b.gate_proj": {"gemm": 831.3e6, "quantize": 43.0e6},
+    "llama2-70b.gate_proj": {"gemm": 831.3e6, "quantize": 43.0e6, "gemm6": 1088.6e6, "quantize6": 47.1e6},
 }
 
 
@@ -115,6 +120,8 @@ def main():
     ap.add_argument("--workload", default="llama2-70b.gate_proj", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--unfused", action="store_true", help="run the reference's three-op sequence instead")
+    ap.add_argument("--int8-mfma", action="store_true",
+                    help="W4A4: keep the int4 products on the int8 MFMA path (same output bits as the 6-bit path)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run only plain device-to-device copies of a 256 MiB buffer (known traffic: 256 MiB read, "
                          "256 MiB written per launch) to scale the FETCH_SIZE / WRITE_SIZE counters")
@@ -151,10 +158,26 @@ def main():
 
     from quik_amd import asymmetric, matmul
     colmap = mod._column_map()
+    six = mod.fused and not args.int8_mfma and mod._six_bit_ok(M)   # the path MixedQLinear.forward takes
+    w6 = mod._weight6() if six else None
+
+    def quantize_only():
+        if six:
+            return asymmetric.quantize_mapped_fp6(x, colmap, K, F)
+        return asymmetric.quantize_mapped(x, colmap, K, F, bits)
 
     def step(ev=None):
         if ev is not None:
             ev[0].record()
+        if six:
+            x6, meta = asymmetric.quantize_mapped_fp6(x, colmap, K, F)
+            if ev is not None:
+                ev[1].record()
+            out = matmul.mixed_linear_fp6(x6, w6, meta, mod.weights_scales, mod.reduced_w, mod.bias, M, N, K, F,
+                                          torch.float16)
+            if ev is not None:
+                ev[2].record()
+            return out
         q, meta, fp = asymmetric.quantize_mapped(x, colmap, K, F, bits)
         if ev is not None:
             ev[1].record()
@@ -189,7 +212,7 @@ def main():
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record()
     for _ in range(50):
-        asymmetric.quantize_mapped(x, colmap, K, F, bits)
+        quantize_only()
     e1.record()
     torch.cuda.synchronize()
     q_b2b = e0.elapsed_time(e1) / 50
@@ -223,31 +246,45 @@ def main():
     int_ops = 2.0 * M * N * K
     tops = int_ops / (ms_step * 1e-3) / 1e12
     gemm_tops = int_ops / (g_avg * 1e-3) / 1e12
-    quant_bytes = M * n_in * 2 + M * K * bits // 8 + M * F * 2 + M * 4
+    # read the row once; write the codes (6 bits each in the operand format of the 6-bit path, plus a 4-byte
+    # level sum per row), the outlier values and the (scale, zero) pair
+    quant_bytes = M * n_in * 2 + (M * K * 6 // 8 + M * 4 if six else M * K * bits // 8) + M * F * 2 + M * 4
     quant_gbps = quant_bytes / (q_avg * 1e-3) / 1e9
+    peak = PEAK_FP6_TOPS if six else PEAK_INT8_TOPS
+    if six:
+        gemm_kernel = "gemm_fused6_split_kernel (one launch per step)"
+        dtype = "int4 (exact, as E2M3 on the 6-bit MFMA path)"
+    elif mod.fused:
+        gemm_kernel = "gemm_fused_split_kernel (one launch per step)"
+        dtype = "int8" if bits == 8 else "int4 (on int8 MFMA)"
+    else:
+        gemm_kernel = "gemm_i32_split_kernel + dequantize + F.linear"
+        dtype = "int8" if bits == 8 else "int4 (on int8 MFMA)"
 
     res = {
         "metric": "MixedQLinear fwd TOPS (2*M*N*K / forward time), 1 GPU",
         "value": round(tops, 2), "unit": "TOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "int8" if bits == 8 else "int4 (on int8 MFMA)", "data": "synthetic",
+        "dtype": dtype, "data": "synthetic",
         "config": {"workload": f"{name}: MixedQLinear fwd, tokens={M}, in={n_in}, out={N}, fp16 outliers={F}, "
                                f"W{bits}A{bits} asymmetric per-token, fp16 activations, "
-                               f"{'fused GEMM+dequant' if mod.fused else 'unfused three-op sequence'}",
+                               f"{'fused GEMM+dequant' if mod.fused else 'unfused three-op sequence'}"
+                               f"{', 6-bit matrix-core path' if six else ''}",
                    "M": M, "in_features": n_in, "K": K, "N": N, "F": F, "bits": bits},
         "pct_int8_mfma_peak": round(100.0 * tops / PEAK_INT8_TOPS, 2),
         "graph_replay_ms_per_step": None if graph_ms is None else round(graph_ms, 4),
-        "roofline": {"kernel": "gemm_fused_split_kernel (one launch per step)" if mod.fused
-                     else "gemm_i32_split_kernel + dequantize + F.linear",
-                     "bound": "mfma", "achieved": round(gemm_tops, 2), "peak": PEAK_INT8_TOPS,
-                     "unit": "TOP/s", "frac": round(gemm_tops / PEAK_INT8_TOPS, 4),
-                     "traffic": traffic.get("gemm") if mod.fused else None,
+        "roofline": {"kernel": gemm_kernel,
+                     "bound": "mfma", "achieved": round(gemm_tops, 2), "peak": peak,
+                     "unit": "TOP/s", "frac": round(gemm_tops / peak, 4),
+                     "frac_of_int8_peak": round(gemm_tops / PEAK_INT8_TOPS, 4),
+                     "traffic": traffic.get("gemm6" if six else "gemm") if mod.fused else None,
                      "avg_ms": round(g_avg, 4), "median_ms": round(g_ms[len(g_ms) // 2], 4),
                      "algorithmic_ops": int_ops},
-        "roofline_quantize": {"kernel": "asym_quantize_stream_kernel", "bound": "hbm",
+        "roofline_quantize": {"kernel": "asym_quantize_stream_kernel" + (" (6-bit operand output)" if six else ""),
+                              "bound": "hbm",
                               "achieved": round(quant_gbps, 1),
                               "peak": PEAK_HBM_GBPS, "unit": "GB/s", "frac": round(quant_gbps / PEAK_HBM_GBPS, 4),
-                              "traffic": traffic.get("quantize"), "avg_ms": round(q_avg, 5),
+                              "traffic": traffic.get("quantize6" if six else "quantize"), "avg_ms": round(q_avg, 5),
                               "median_ms": round(q_ms[len(q_ms) // 2], 5), "algorithmic_bytes": quant_bytes,
                               "back_to_back_ms": round(q_b2b, 5),
                               "note": "avg_ms: two event records around one ~15 us launch inside the step "
