@@ -424,31 +424,54 @@ __device__ __forceinline__ void fused6_tile(const Fused6Args &p, int tm, int tn,
   pipe.template run_f16<BF16>(acc);
   pipe.drain();
 
-  // out = storage(acc + (zs * w_red + bias)), written through the staging area
+  // out = storage(acc + (zs * w_red + bias)), written through a staging area in the (now idle) ring: all MI row
+  // blocks of the wave are staged, then read back as whole row segments, then stored, so the LDS round trip and
+  // the store issue are paid once per tile and not once per row block.  The per-column vectors are read once;
+  // the fragment registers are free by now.
   using Store = BlockStore<C, uint16_t>;
-  static_assert(Store::kBytes * C::WAVES <= Pipe::SMEM, "staging fits in the (now idle) ring");
-  uint8_t *stage = smem + wave * Store::kBytes;
+  static_assert(Store::kBytes * C::MI * C::WAVES <= Pipe::SMEM, "staging fits in the ring");
+  uint8_t *stage = smem + wave * (Store::kBytes * C::MI);
   const bool vec = (p.ldo & 7) == 0 && (reinterpret_cast<uintptr_t>(p.out) & 15) == 0;
-  const int nw = n0 + wn * C::WN;
+  const int nw = n0 + wn * C::WN, mw = m0 + wm * C::WM;
+  float4 wr[C::NI][4], bs[C::NI][4];
+#pragma unroll
+  for (int ni = 0; ni < C::NI; ++ni)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int c = wn * C::WN + ni * 32 + acc_col(g, lane);
+      wr[ni][g] = *reinterpret_cast<const float4 *>(tv.wred + c);
+      bs[ni][g] = *reinterpret_cast<const float4 *>(tv.bias + c);
+    }
 #pragma unroll
   for (int mi = 0; mi < C::MI; ++mi) {
-    const int mb = m0 + wm * C::WM + mi * 32;
     const float zs = tv.zs[wm * C::WM + mi * 32 + (lane & 31)];
 #pragma unroll
     for (int ni = 0; ni < C::NI; ++ni)
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        const int c = wn * C::WN + ni * 32 + acc_col(g, lane);
-        const float4 wr = *reinterpret_cast<const float4 *>(tv.wred + c);
-        const float4 bs = *reinterpret_cast<const float4 *>(tv.bias + c);
-        const uint16_t v[4] = {from_f32<BF16>(acc[mi][ni][4 * g] + (zs * wr.x + bs.x)),
-                               from_f32<BF16>(acc[mi][ni][4 * g + 1] + (zs * wr.y + bs.y)),
-                               from_f32<BF16>(acc[mi][ni][4 * g + 2] + (zs * wr.z + bs.z)),
-                               from_f32<BF16>(acc[mi][ni][4 * g + 3] + (zs * wr.w + bs.w))};
-        Store::put(stage, lane, ni, g, v);
+        const uint16_t v[4] = {from_f32<BF16>(acc[mi][ni][4 * g] + (zs * wr[ni][g].x + bs[ni][g].x)),
+                               from_f32<BF16>(acc[mi][ni][4 * g + 1] + (zs * wr[ni][g].y + bs[ni][g].y)),
+                               from_f32<BF16>(acc[mi][ni][4 * g + 2] + (zs * wr[ni][g].z + bs[ni][g].z)),
+                               from_f32<BF16>(acc[mi][ni][4 * g + 3] + (zs * wr[ni][g].w + bs[ni][g].w))};
+        Store::put(stage + mi * Store::kBytes, lane, ni, g, v);
       }
-    if (mb < p.M && nw < p.N) Store::flush(stage, lane, p.out + int64_t(mb) * p.ldo + nw, p.ldo, p.M - mb, p.N - nw, vec);
-    __builtin_amdgcn_sched_barrier(0);
+  }
+  if (vec && p.M - mw >= C::WM && p.N - nw >= C::WN) {  // interior (wave-uniform): straight-line code
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    v4i piece[C::MI][Store::kIters];
+#pragma unroll
+    for (int mi = 0; mi < C::MI; ++mi) Store::read_block(stage + mi * Store::kBytes, lane, piece[mi]);
+#pragma unroll
+    for (int mi = 0; mi < C::MI; ++mi)
+      Store::write_block(piece[mi], lane, p.out + int64_t(mw + mi * 32) * p.ldo + nw, p.ldo);
+  } else {
+#pragma unroll
+    for (int mi = 0; mi < C::MI; ++mi) {
+      const int mb = mw + mi * 32;
+      if (mb < p.M && nw < p.N)
+        Store::flush(stage + mi * Store::kBytes, lane, p.out + int64_t(mb) * p.ldo + nw, p.ldo, p.M - mb, p.N - nw, vec);
+    }
   }
 }
 

@@ -485,6 +485,21 @@ struct BlockStore {
     }
   }
 
+  // interior block: the 32 / kRowsPerInstr pieces of a staged block, and their places in global memory
+  static constexpr int kIters = 32 / kRowsPerInstr;
+  static __device__ __forceinline__ void read_block(const uint8_t *stage, int lane, v4i (&piece)[kIters]) {
+#pragma unroll
+    for (int it = 0; it < kIters; ++it)
+      piece[it] = *reinterpret_cast<const v4i *>(stage + (it * kRowsPerInstr + lane / kLanesPerRow) * kRowBytes +
+                                                 (lane % kLanesPerRow) * 16);
+  }
+  static __device__ __forceinline__ void write_block(const v4i (&piece)[kIters], int lane, T *g, int64_t ld) {
+#pragma unroll
+    for (int it = 0; it < kIters; ++it)
+      *reinterpret_cast<v4i *>(g + int64_t(it * kRowsPerInstr + lane / kLanesPerRow) * ld +
+                               (lane % kLanesPerRow) * kElems) = piece[it];
+  }
+
   // staged block -> g[row * ld + col], rows < rows_valid, cols < cols_valid
   static __device__ __forceinline__ void flush(const uint8_t *stage, int lane, T *g, int64_t ld, int rows_valid,
                                                int cols_valid, bool vec) {
