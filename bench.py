@@ -3,7 +3,7 @@
 
 A step is one forward of the layer: the per-token asymmetric quantize kernel followed by the
 fused GEMM kernel (int4 x int4 + fp16 outlier GEMM + dequantize epilogue), on synthetic inputs
-already resident in HBM.  W4A4 layers with 256 or more token rows take the path MixedQLinear takes:
+already resident in HBM.  W4A4 layers with more than 32 token rows take the path MixedQLinear takes:
 the int4 products run on the 6-bit (E2M3) matrix-core instructions, exactly (--int8-mfma forces the
 int8 MFMA path, which has the same output bits).  The default workload is the one the headline
 metric is quoted on: Llama-2-70B gate_proj, 8192 -> 28672, 2048 tokens, 256 fp16 outlier

@@ -63,14 +63,14 @@ class SharedQuantizedInput:
 class MixedQLinear(torch.nn.Module):
     """The reference's layer (qlinear.py:40-145) on the HIP kernels.
 
-    W4A4 asymmetric layers with at least `six_bit_min_rows` token rows run their int4 products on the
+    W4A4 asymmetric calls with at least `six_bit_min_rows` token rows (everything above decode size) run their int4 products on the
     6-bit (E2M3) matrix-core path, which has twice the int8 rate: levels code + 8 are exact E2M3 numbers
     and the integer accumulator is recovered exactly, so the output is bit-identical to the int8-MFMA
     path.  It needs int_features % 128 == 0, fp_features % 32 == 0 and ascending int_indices, and keeps a
     second copy of the weights in the operand format of that path (0.75 bytes per int4 weight plus the
     outlier columns, built on first use); `six_bit_path = False` turns it off."""
 
-    six_bit_min_rows = 256
+    six_bit_min_rows = 33    # up to 32 rows the weight-streaming decode kernel on the packed int4 weights is the right one
 
     def __init__(self, in_features, out_features, shared_input=None,
                  fp_features_num=0, symm=False, bits=4, dtype=torch.float16, fused=True):

@@ -614,7 +614,7 @@ def test_kernel_path_vs_simulated_path(bits, bf16):
     assert e_ker < (0.2 if bits == 4 else 0.02), e_ker
 
 
-@pytest.mark.parametrize("tokens", [300, 200, 4])     # 6-bit matrix-core path, int8-MFMA path, decode kernel
+@pytest.mark.parametrize("tokens", [300, 40, 4])     # 6-bit matrix-core path (two tile plans), decode kernel
 def test_forward_under_hip_graph_replays(tokens):
     """The forward (quantize + GEMM, no allocation or synchronisation inside the library) captured in a
     HIP graph: every replay, with new input contents and eager work in between, equals the eager result."""
@@ -947,7 +947,9 @@ def test_six_bit_operand_buffers_hold_the_int4_codes(rows, K, F, bf16):
 
 
 SIX_CASES = [
-    # M, N, in, F, bias, kind: K = in - F a multiple of 128, F a multiple of 32, M >= 256
+    # M, N, in, F, bias, kind: K = in - F a multiple of 128, F a multiple of 32, M > 32
+    (33, 200, 544, 32, True, "x50"),          # smallest row count of the path
+    (100, 1056, 1024 + 64, 64, False, "student"),
     (256, 256, 384, 128, True, "x50"),        # one 128x128-tile round, two integer steps
     (300, 520, 1088, 64, False, "student"),   # ragged M and N
     (257, 130, 544, 32, True, "x50"),         # two outlier steps, N below a tile
@@ -1015,6 +1017,6 @@ def test_six_bit_path_shared_input_and_fallbacks():
     for i, (m, s) in enumerate(zip(mods, singles)):
         assert torch.equal(m(xt), s(xt))
     assert shared.x6 is None and shared.qint_x is None
-    small = xt[:40].contiguous()                               # below the row threshold: int4 path, decode-size kernels
+    small = xt[:20].contiguous()                               # decode size: int4 path, weight-streaming kernel
     assert torch.equal(mods[0](small), singles[0](small))
     shared.finish(), shared.finish()
