@@ -43,6 +43,19 @@ __device__ __forceinline__ uint16_t from_f32(float f) {
   }
 }
 
+// Two fp32 values -> two storage values in one dword (first value in the low half).  fp16: the packed
+// convert instruction of gfx950, same round-to-nearest-even as the scalar one.
+template <bool BF16>
+__device__ __forceinline__ uint32_t pack2_from_f32(float a, float b) {
+  if constexpr (BF16) {
+    return static_cast<uint32_t>(f32_to_bf16_bits(a)) | (static_cast<uint32_t>(f32_to_bf16_bits(b)) << 16);
+  } else {
+    typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+    typedef float float2_t __attribute__((ext_vector_type(2)));
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(float2_t{a, b}, half2_t));
+  }
+}
+
 // Round an fp32 value to the storage type and return it as fp32 again.
 template <bool BF16>
 __device__ __forceinline__ float round_storage(float f) {

@@ -449,11 +449,11 @@ __device__ __forceinline__ void fused6_tile(const Fused6Args &p, int tm, int tn,
     for (int ni = 0; ni < C::NI; ++ni)
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        const uint16_t v[4] = {from_f32<BF16>(acc[mi][ni][4 * g] + (zs * wr[ni][g].x + bs[ni][g].x)),
-                               from_f32<BF16>(acc[mi][ni][4 * g + 1] + (zs * wr[ni][g].y + bs[ni][g].y)),
-                               from_f32<BF16>(acc[mi][ni][4 * g + 2] + (zs * wr[ni][g].z + bs[ni][g].z)),
-                               from_f32<BF16>(acc[mi][ni][4 * g + 3] + (zs * wr[ni][g].w + bs[ni][g].w))};
-        Store::put(stage + mi * Store::kBytes, lane, ni, g, v);
+        Store::put_pairs(stage + mi * Store::kBytes, lane, ni, g,
+                         pack2_from_f32<BF16>(acc[mi][ni][4 * g] + (zs * wr[ni][g].x + bs[ni][g].x),
+                                              acc[mi][ni][4 * g + 1] + (zs * wr[ni][g].y + bs[ni][g].y)),
+                         pack2_from_f32<BF16>(acc[mi][ni][4 * g + 2] + (zs * wr[ni][g].z + bs[ni][g].z),
+                                              acc[mi][ni][4 * g + 3] + (zs * wr[ni][g].w + bs[ni][g].w)));
       }
   }
   if (vec && p.M - mw >= C::WM && p.N - nw >= C::WN) {  // interior (wave-uniform): straight-line code

@@ -485,6 +485,12 @@ struct BlockStore {
     }
   }
 
+  // the same for 16-bit elements that are already packed in pairs
+  static __device__ __forceinline__ void put_pairs(uint8_t *stage, int lane, int ni, int g, uint32_t lo, uint32_t hi) {
+    static_assert(sizeof(T) == 2, "16-bit elements");
+    *reinterpret_cast<uint2 *>(stage + (lane & 31) * kRowBytes + (ni * 32 + acc_col(g, lane)) * 2) = make_uint2(lo, hi);
+  }
+
   // interior block: the 32 / kRowsPerInstr pieces of a staged block, and their places in global memory
   static constexpr int kIters = 32 / kRowsPerInstr;
   static __device__ __forceinline__ void read_block(const uint8_t *stage, int lane, v4i (&piece)[kIters]) {
@@ -768,11 +774,11 @@ __device__ __forceinline__ void fused_tile(const FusedArgs &p, int tm, int tn, u
         const int c = wn * C::WN + ni * 32 + acc_col(g, lane);
         const float4 wr = *reinterpret_cast<const float4 *>(tv.wred + c);
         const float4 bs = *reinterpret_cast<const float4 *>(tv.bias + c);
-        const uint16_t v[4] = {from_f32<BF16>(accf[mi][ni][4 * g] + (zs * wr.x + bs.x)),
-                               from_f32<BF16>(accf[mi][ni][4 * g + 1] + (zs * wr.y + bs.y)),
-                               from_f32<BF16>(accf[mi][ni][4 * g + 2] + (zs * wr.z + bs.z)),
-                               from_f32<BF16>(accf[mi][ni][4 * g + 3] + (zs * wr.w + bs.w))};
-        Store::put(stage, lane, ni, g, v);
+        Store::put_pairs(stage, lane, ni, g,
+                         pack2_from_f32<BF16>(accf[mi][ni][4 * g] + (zs * wr.x + bs.x),
+                                              accf[mi][ni][4 * g + 1] + (zs * wr.y + bs.y)),
+                         pack2_from_f32<BF16>(accf[mi][ni][4 * g + 2] + (zs * wr.z + bs.z),
+                                              accf[mi][ni][4 * g + 3] + (zs * wr.w + bs.w)));
       }
     if (mb < p.M && nw < p.N) Store::flush(stage, lane, p.out + int64_t(mb) * p.ldo + nw, p.ldo, p.M - mb, p.N - nw, vec);
     __builtin_amdgcn_sched_barrier(0);
