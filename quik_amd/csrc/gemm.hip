@@ -15,6 +15,7 @@ using CfgL = Cfg<256, 256, 2, 2, 2>;   // prefill: 128x128 per wave, 256 accumul
 using CfgH = Cfg<256, 128, 2, 2, 2>;   // half-width tile that evens out the last round
 using CfgM = Cfg<128, 128, 2, 2, 2>;   // mid-size problems, two workgroups per CU
 using CfgN = Cfg<128, 64, 2, 2, 2>;    // few tiles: narrower ones put more CUs to work, three workgroups per CU
+using CfgL8 = Cfg<256, 256, 2, 4, 2>;  // 6-bit path, launches of 256x256 tiles only: two waves per SIMD (1-5 % faster than CfgL)
 using CfgLp = Cfg<256, 256, 2, 2, 0>;  // plain fallbacks
 using CfgMp = Cfg<128, 128, 2, 2, 0>;
 
@@ -140,42 +141,42 @@ struct Plan {
 constexpr int kCostWide = 100, kCostHalf = 55, kCostMid = 28;
 
 // Makespan of `wide` tiles followed by `half` tiles on kCUs CUs under greedy list scheduling.
-int64_t makespan(int64_t wide, int64_t half) {
+int64_t makespan(int64_t wide, int64_t half, int cost_half = kCostHalf) {
   // after the wide tiles: `rem` CUs carry one tile more than the others
   const int64_t full = wide / kCUs, rem = wide % kCUs;
   int64_t lo_level = full * kCostWide, lo_count = kCUs - rem;  // less loaded CUs
   int64_t hi_level = lo_level + kCostWide, hi_count = rem;
   // the half tiles go to the least loaded CUs, a whole level at a time
   while (half > 0) {
-    if (hi_count == 0 || lo_level + kCostHalf <= hi_level) {
-      if (half >= lo_count && lo_level + kCostHalf < hi_level && hi_count > 0) {
-        lo_level += kCostHalf;
+    if (hi_count == 0 || lo_level + cost_half <= hi_level) {
+      if (half >= lo_count && lo_level + cost_half < hi_level && hi_count > 0) {
+        lo_level += cost_half;
         half -= lo_count;
       } else if (hi_count == 0) {
         const int64_t rounds = half / lo_count, left = half % lo_count;
-        return lo_level + rounds * kCostHalf + (left ? kCostHalf : 0);
+        return lo_level + rounds * cost_half + (left ? cost_half : 0);
       } else if (half >= lo_count) {  // lo reaches hi's level exactly
-        lo_level += kCostHalf;
+        lo_level += cost_half;
         half -= lo_count;
         if (lo_level == hi_level) {
           lo_count += hi_count;
           hi_count = 0;
         }
       } else {
-        const int64_t top = lo_level + kCostHalf;
+        const int64_t top = lo_level + cost_half;
         return top > hi_level ? top : hi_level;
       }
     } else {
       // adding a half tile to the lower level overtakes the higher one: swap roles afterwards
       if (half >= lo_count) {
         half -= lo_count;
-        const int64_t new_hi = lo_level + kCostHalf, new_hi_count = lo_count;
+        const int64_t new_hi = lo_level + cost_half, new_hi_count = lo_count;
         lo_level = hi_level;
         lo_count = hi_count;
         hi_level = new_hi;
         hi_count = new_hi_count;
       } else {
-        return lo_level + kCostHalf;
+        return lo_level + cost_half;
       }
     }
   }
@@ -248,6 +249,27 @@ int run_i32(const uint8_t *X, const uint8_t *W, int32_t *C, int64_t M, int64_t N
   return launch_i32_split<CfgL, CfgH, MODE>(wide, tail, st);
 }
 
+// Tile plan of the 6-bit path (gemm_fp6.h).  Costs in percent of a 256x256 tile, measured at K = 7936, F = 256:
+// a 256x128 tile 59; 128x128 tiles run two to a CU, 66 for a pair, 36 for one that has the CU to itself.
+Plan make_plan6(int64_t M, int64_t N) {
+  if (M <= 32) return {Plan::kSmall, 0};
+  const int64_t tiles_m = (M + 255) / 256;
+  const int64_t mid_tiles = ((M + 127) / 128) * ((N + 127) / 128);
+  const int64_t pairs = mid_tiles / (2 * kCUs), left = mid_tiles % (2 * kCUs);
+  const int64_t mid = pairs * 66 + (left == 0 ? 0 : left <= kCUs ? 36 : 66);
+  int64_t best = INT64_MAX, best_n = 0;
+  for (int64_t n_wide = 0; n_wide <= N + 255; n_wide += 256) {
+    const int64_t nw = n_wide < N ? n_wide : N;   // the last candidate: wide tiles only, the last one ragged
+    const int64_t c = makespan(tiles_m * ((nw + 255) / 256), tiles_m * ((N - nw + 127) / 128), 59);
+    if (c <= best) {
+      best = c;
+      best_n = nw;
+    }
+  }
+  if (mid < best) return {Plan::kMid, 0};
+  return {Plan::kSplit, best_n};
+}
+
 template <class C, bool BF16>
 int launch_fused6(const Fused6Args &p, hipStream_t st) {
   if (p.N <= 0) return QUIK_OK;
@@ -265,7 +287,8 @@ int launch_fused6_split(const Fused6Args &wide, const Fused6Args &tail, hipStrea
   if (wide.N <= 0) return launch_fused6<CT, BF16>(tail, st);
   if (tail.N <= 0) return launch_fused6<CW, BF16>(wide, st);
   int tail_blocks;
-  const SplitGrid grid = split_grid<CW, CT>(wide.M, wide.N, tail.N, tail_blocks);
+  SplitGrid grid = split_grid<CW, CT>(wide.M, wide.N, tail.N, tail_blocks);
+  grid.lead = 0;  // this kernel lives on L2 hits between the tiles of an XCD that share operand rows: keep them in step
   auto kern = gemm_fused6_split_kernel<CW, CT, BF16>;
   constexpr int smem = fused6_smem<CW>() > fused6_smem<CT>() ? fused6_smem<CW>() : fused6_smem<CT>();
   if (int rc = prepare(kern, smem)) return rc;
@@ -273,11 +296,13 @@ int launch_fused6_split(const Fused6Args &wide, const Fused6Args &tail, hipStrea
   return check_launch();
 }
 
-// The 6-bit matrix-core path (gemm_fp6.h): same tile plan, 256x256 + 256x128 tiles or 128x128 tiles.
+// The 6-bit matrix-core path (gemm_fp6.h): 256x256 tiles alone (eight waves), 256x256 + 256x128 tiles in one
+// launch (four waves), or 128x128 tiles.
 template <bool BF16>
 int run_fused6(const Fused6Args &p, hipStream_t st) {
-  const Plan plan = make_plan(p.M, p.N, true);
+  const Plan plan = make_plan6(p.M, p.N);
   if (plan.kind == Plan::kSmall) return QUIK_ERR_SHAPE;  // at most 32 rows: the weight-streaming kernel is the right one
+  if (plan.kind == Plan::kSplit && plan.n_wide >= p.N) return launch_fused6<CfgL8, BF16>(p, st);
   if (plan.kind != Plan::kSplit) return launch_fused6<CfgM, BF16>(p, st);
   Fused6Args wide = p, tail = p;
   const int64_t nw = plan.n_wide;

@@ -42,7 +42,7 @@ template <class C>
 struct Fp6Pipe {
   static constexpr int MI = C::MI, NI = C::NI, NS = 6, NF = MI + NI;
   static_assert(C::WM % 64 == 0 && C::WN % 64 == 0, "a wave's rows start at a 64-row block");
-  static_assert(C::WAVES == 4, "copy assignment below");
+  static_assert(C::WAVES == 4 || C::WAVES == 8, "copy assignment below");
   // LDS slot of one step: the 3 KB units of the tile's X blocks, then of its W blocks, as they are in memory
   static constexpr int W_OFF = C::BM * 48;
   static constexpr int STAGE = (C::BM + C::BN) * 48;
@@ -53,8 +53,10 @@ struct Fp6Pipe {
   //   256x256: W block w (3);  256x128: W block w % 2, pieces w / 2 and w / 2 + 1 (piece 1 is copied twice);
   //   128x128: none.
   static constexpr int XB = C::BM / 64, WB = C::BN / 64;
-  static constexpr int NB = XB + WB == 8 ? 3 : XB + WB == 6 ? 2 : 0;
+  // (eight waves, 256x256: one block per wave, no source B)
+  static constexpr int NB = C::WAVES == 8 ? 0 : XB + WB == 8 ? 3 : XB + WB == 6 ? 2 : 0;
   static_assert((XB == 4 && (WB == 4 || WB == 2)) || (XB == 2 && WB == 2), "supported tile shapes");
+  static_assert(C::WAVES == 4 || XB + WB == 8, "eight waves copy eight blocks");
   static constexpr int P = 3 + NB;  // copies per wave and step
   static_assert(3 * P <= 63, "three steps in flight must fit the vmcnt counter");
 
