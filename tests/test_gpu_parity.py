@@ -956,6 +956,8 @@ SIX_CASES = [
     (512, 1024, 1024, 0, True, "x50"),        # no outlier columns
     (1000, 4160, 4096, 256, True, "x50"),     # 256x256 and 256x128 tiles in one launch, ragged M, N = 32.5 tiles
     (2048, 1280, 2048 + 96, 96, False, "x50"),
+    (2048, 8192, 1024 + 128, 128, True, "x50"),   # one full round of 256x256 tiles: the eight-wave tile
+    (2040, 8192 - 64, 512 + 32, 32, False, "x50"),   # eight-wave tiles, ragged last tile row and column
 ]
 
 
