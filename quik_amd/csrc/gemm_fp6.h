@@ -70,6 +70,8 @@ struct Fp6Pipe {
   uint32_t rd;              // byte offset of the slot the next fragment read looks at
   int steps0, steps;        // integer steps, all steps
   uint32_t x_head, w_head;  // this lane's head offsets inside a slot (fragment j: + 1024 j)
+  uint32_t x_head3[3], w_head3[3], tail3[3][NF];  // the same offsets inside slots 0, 2 and 4 (for steps whose slot is
+                                                  // known at compile time: the odd slot is an immediate offset away)
   uint32_t tail[NF];        // this lane's tail offsets inside a slot, one register per fragment: reads that share
                             // a base register are paired into one 4-register read by the compiler, and the halves
                             // then have to be copied into the operand tuples behind an exposed LDS round trip
@@ -120,25 +122,39 @@ struct Fp6Pipe {
                 h * 512 + ((jj & 1) * 32 + r) * 8;
       asm volatile("" : "+v"(tail[j]));  // unrelated values as far as the compiler can tell
     }
+#pragma unroll
+    for (int q = 0; q < 3; ++q) {
+      x_head3[q] = x_head + q * 2 * STAGE;
+      w_head3[q] = w_head + q * 2 * STAGE;
+#pragma unroll
+      for (int j = 0; j < NF; ++j) {
+        tail3[q][j] = tail[j] + q * 2 * STAGE;
+        asm volatile("" : "+v"(tail3[q][j]));
+      }
+    }
   }
 
   // Copy G (0 .. P-1) of the step being copied; after the last one the scalar bookkeeping: two pointer
   // bumps and one slot bump.  Past the last step the pointers stop and the last step is copied again into
   // a slot nobody reads.
-  template <int G>
+  // FS: slot being filled when known at compile time (the caller keeps `fill` consistent), -1: `fill`
+  template <int G, int FS = -1>
   __device__ __forceinline__ void issue_one() {
+    const uint32_t slot = FS < 0 ? fill : lds0 + (FS < 0 ? 0 : FS) * STAGE;
     if constexpr (G < 3) {
-      dma_load16k<G * 1024>(pa, lane16, fill + da);
+      dma_load16k<G * 1024>(pa, lane16, slot + da);
     } else {
-      dma_load16k<(G - 3) * 1024>(pb, lane16, fill + db);
+      dma_load16k<(G - 3) * 1024>(pb, lane16, slot + db);
     }
     if constexpr (G == P - 1) {
       const int adv = left > 1 ? 3072 : 0;
       left -= 1;
       pa += adv;
       pb += adv;
-      fill += STAGE;
-      fill = fill == lds0 + NS * STAGE ? lds0 : fill;
+      if constexpr (FS < 0) {
+        fill += STAGE;
+        fill = fill == lds0 + NS * STAGE ? lds0 : fill;
+      }
     }
   }
   template <int G = 0>
@@ -168,12 +184,20 @@ struct Fp6Pipe {
   __device__ __forceinline__ void previous_read_slot() { rd = rd == 0 ? (NS - 1) * STAGE : rd - STAGE; }
 
   // fragment j (32 rows) of this wave: head image j, tail image j / 2 at row offset 32 (j % 2)
-  template <int J>
+  // RS: slot being read when known at compile time, -1: `rd`
+  template <int J, int RS = -1>
   __device__ __forceinline__ void read6_one(v4i (&fh)[NF], v2i (&ft)[NF]) const {
     constexpr int jj = J < MI ? J : J - MI;
-    const uint8_t *s = smem + rd;
-    fh[J] = *reinterpret_cast<const v4i *>(s + (J < MI ? x_head : w_head) + (jj >> 1) * 3072 + (jj & 1) * 1024);
-    ft[J] = *reinterpret_cast<const v2i *>(s + tail[J]);
+    if constexpr (RS < 0) {
+      const uint8_t *s = smem + rd;
+      fh[J] = *reinterpret_cast<const v4i *>(s + (J < MI ? x_head : w_head) + (jj >> 1) * 3072 + (jj & 1) * 1024);
+      ft[J] = *reinterpret_cast<const v2i *>(s + tail[J]);
+    } else {
+      constexpr int q = (RS < 0 ? 0 : RS) / 2, odd = ((RS < 0 ? 0 : RS) % 2) * STAGE;
+      fh[J] = *reinterpret_cast<const v4i *>(smem + (J < MI ? x_head3[q] : w_head3[q]) + odd + (jj >> 1) * 3072 +
+                                             (jj & 1) * 1024);
+      ft[J] = *reinterpret_cast<const v2i *>(smem + tail3[q][J] + odd);
+    }
   }
   template <int J>
   __device__ __forceinline__ void read16_one(v4i (&f)[NF]) const {
@@ -221,13 +245,15 @@ struct Fp6Pipe {
   // landed (the three newer ones stay in flight) and a barrier makes it visible; behind it every wave has
   // issued the MFMAs of this step, which waited for their fragments, so this step's slot may be overwritten
   // by the copies issued during the next step.
-  template <int G = 0>
+  // RS / FS: the slots read and filled during this step when they are known at compile time (six steps in a
+  // row return to the same slots, so `rd` and `fill` stay valid without being touched), -1: `rd` / `fill`
+  template <int RS = -1, int FS = -1, int G = 0>
   __device__ __forceinline__ void step6(const v4i (&ch)[NF], const v2i (&ct)[NF], v4i (&nh)[NF], v2i (&nt)[NF],
                                         v16f (&acc)[MI][NI]) {
     constexpr int MM = MI * NI;
     if constexpr (G < P) {
       constexpr int r_lo = G * NF / P, r_hi = (G + 1) * NF / P, m_lo = G * MM / P, m_hi = (G + 1) * MM / P;
-      chunk_reads6<r_lo, r_hi>(nh, nt);
+      chunk_reads6<RS, r_lo, r_hi>(nh, nt);
       chunk_mfmas6<m_lo, m_hi>(ch, ct, acc);
 #pragma unroll
       for (int i = m_lo; i < m_hi; ++i) {
@@ -235,20 +261,20 @@ struct Fp6Pipe {
         __builtin_amdgcn_sched_group_barrier(0x100, (2 * (r_hi - r_lo) + (m_hi - m_lo) - 1) / (m_hi - m_lo), 0);
       }
       __builtin_amdgcn_sched_barrier(0);
-      issue_one<G>();
+      issue_one<G, FS>();
       __builtin_amdgcn_sched_barrier(0);
-      step6<G + 1>(ch, ct, nh, nt, acc);
+      step6<RS, FS, G + 1>(ch, ct, nh, nt, acc);
     } else {
-      next_read_slot();
+      if constexpr (RS < 0) next_read_slot();
       __builtin_amdgcn_s_waitcnt(vmcnt_imm(3 * P));
       __builtin_amdgcn_s_barrier();
     }
   }
-  template <int LO, int HI>
+  template <int RS, int LO, int HI>
   __device__ __forceinline__ void chunk_reads6(v4i (&nh)[NF], v2i (&nt)[NF]) const {
     if constexpr (LO < HI) {
-      read6_one<LO>(nh, nt);
-      chunk_reads6<LO + 1, HI>(nh, nt);
+      read6_one<LO, RS>(nh, nt);
+      chunk_reads6<RS, LO + 1, HI>(nh, nt);
     }
   }
   template <int LO, int HI>
@@ -300,7 +326,18 @@ struct Fp6Pipe {
     v4i h0[NF], h1[NF];
     v2i t0[NF], t1[NF];
     read6(h0, t0);
-    for (int j = 0; j < steps0; j += 2) {
+    // here: step 0 in h0 / t0, `rd` at slot 1, `fill` at slot 5.  Six steps at a time with the slots as
+    // immediates (no address arithmetic in the loop), then the remaining pairs with `rd` / `fill`
+    int j = 0;
+    for (; j + 6 <= steps0; j += 6) {
+      step6<1, 5>(h0, t0, h1, t1, acc);
+      step6<2, 0>(h1, t1, h0, t0, acc);
+      step6<3, 1>(h0, t0, h1, t1, acc);
+      step6<4, 2>(h1, t1, h0, t0, acc);
+      step6<5, 3>(h0, t0, h1, t1, acc);
+      step6<0, 4>(h1, t1, h0, t0, acc);
+    }
+    for (; j < steps0; j += 2) {
       step6(h0, t0, h1, t1, acc);
       step6(h1, t1, h0, t0, acc);
     }
