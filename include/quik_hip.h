@@ -150,6 +150,30 @@ int quik_mixed_linear_fwd_fp6(const void *x6, const void *w6, const void *meta, 
                               const void *w_reduced, const void *bias, int dtype, int64_t M, int64_t N,
                               int64_t K, int64_t F, void *out, void *stream);
 
+/* ---- W8A8 on tile-ordered operands -------------------------------------------------------------
+ * No counterpart in the reference: the same forward as quik_asym_quantize (bits = 8) +
+ * quik_mixed_linear_fwd (bits = 8, asymmetric), bit for bit, with both int8 operands (and the
+ * outlier columns) stored in the order the GEMM tiles copy them, so that every copy moves whole
+ * cache lines exactly once per tile.  Needs K % 64 == 0, F % 32 == 0, M > 32, a column map that
+ * selects the streaming quantize kernel; operand buffers aligned to 256 bytes. */
+
+/* bytes of an operand buffer for [rows, K] int8 + [rows, F] outliers (0 if the shape is not supported) */
+int64_t quik_tile8_operand_bytes(int64_t rows, int64_t K, int64_t F);
+
+/* weights [N, K] int8 (MixedQLinear.int_weight) and [N, F] fp16/bf16 (fp_weight, may be NULL when
+ * F == 0) -> operand buffer; once per layer */
+int quik_tile8_pack_weight(const int8_t *qw, const void *fp_w, int64_t N, int64_t K, int64_t F, void *out,
+                           void *stream);
+
+/* as quik_asym_quantize with bits = 8, codes and outlier values go to an operand buffer */
+int quik_asym_quantize_tile8(const void *x, int dtype, int64_t rows, int64_t cols, const void *colmap,
+                             int64_t num_int, int64_t num_fp, void *out8, void *meta, void *stream);
+
+/* as quik_mixed_linear_fwd (asymmetric form, bits = 8) on operand buffers */
+int quik_mixed_linear_fwd_tile8(const void *x8, const void *w8, const void *meta, const void *s_col,
+                                const void *w_reduced, const void *bias, int dtype, int64_t M, int64_t N,
+                                int64_t K, int64_t F, void *out, void *stream);
+
 /* quik.matmul.int4Matmul(A, B) -> C int32 [M, N]
  * replaces int4MatmulCUDA, src/matmul/matmul.cu:17-55.
  *   A [M, K/2], B [N, K/2] uint8 nibble-packed, K = number of int4 elements per row.

@@ -93,6 +93,25 @@ def quantize_mapped_fp6(src: torch.Tensor, colmap: torch.Tensor, num_int: int, n
     return x6, meta
 
 
+def quantize_mapped_tile8(src: torch.Tensor, colmap: torch.Tensor, num_int: int, num_fp: int):
+    """quantize_mapped with bits = 8 whose codes and outlier values go to a tile-ordered operand buffer for
+    matmul.mixed_linear_tile8 (internal format, see include/quik_hip.h).  Returns (x8 uint8 buffer, meta)."""
+    L.check_cuda_contiguous("quantize", src=src)
+    dt = L.dtype_id(src, "quantize", allow_bf16=True)
+    rows, cols = src.shape
+    lib = L.load()
+    nbytes = lib.quik_tile8_operand_bytes(max(rows, 1), num_int, num_fp)
+    if nbytes == 0:
+        raise RuntimeError("quantize: the tile-ordered int8 format needs a multiple of 64 integer columns and a "
+                           "multiple of 32 outlier columns")
+    with torch.cuda.device(src.device):
+        x8 = torch.empty((nbytes,), dtype=torch.uint8, device=src.device)
+        meta = torch.empty((2 * rows,), dtype=src.dtype, device=src.device)
+        L.check(lib.quik_asym_quantize_tile8(L.ptr(src), dt, rows, cols, L.ptr(colmap), num_int, num_fp, L.ptr(x8),
+                                             L.ptr(meta), L.stream()), "quantize")
+    return x8, meta
+
+
 def quantize(src: torch.Tensor, int_indices: torch.Tensor, fp_indices: torch.Tensor, bits: int):
     """(dst, meta, fp_x) = quantize(src [M, in], int_indices [K] int64, fp_indices [F] int64, bits).
 

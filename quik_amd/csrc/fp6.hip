@@ -1,5 +1,5 @@
-// int4 GEMM on the 6-bit matrix-core path: weight repacking and the entry points (kernels: gemm_fp6.h,
-// operand format: fp6_format.h; the activation side is produced by the quantize kernel).
+// Weight repacking for the GEMMs that read their operands in tile order (kernels: gemm_fp6.h, gemm_tile8.h;
+// operand formats: fp6_format.h; the activation side is produced by the quantize kernel).
 #include "gemm_fp6.h"
 
 namespace quik {
@@ -49,10 +49,44 @@ __global__ __launch_bounds__(kThreads) void pack_weight_kernel(const uint8_t *__
   if (threadIdx.x == 0) reinterpret_cast<int32_t *>(out + l.sums_off)[row] = total;
 }
 
+// int8 weights [N, K] and outlier weights [N, F] -> int8 operand buffer in tile order; one lane per 16-byte chunk
+__global__ __launch_bounds__(kThreads) void pack_weight8_kernel(const uint8_t *__restrict__ qw,
+                                                                const uint16_t *__restrict__ fp_w, int64_t rows,
+                                                                int64_t K, int64_t F, uint8_t *__restrict__ out) {
+  const Tile8Layout l = tile8_layout(rows, K, F);
+  const int64_t row = blockIdx.x;
+  for (int64_t c = threadIdx.x; c < K / 16; c += kThreads)
+    *reinterpret_cast<uint4 *>(out + tile8_offset(l, row, c >> 1, static_cast<int>(c & 1))) =
+        *reinterpret_cast<const uint4 *>(qw + row * K + c * 16);
+  for (int64_t c = threadIdx.x; c < F / 8; c += kThreads)
+    *reinterpret_cast<uint4 *>(out + tile8_offset(l, row, l.steps + (c >> 1), static_cast<int>(c & 1))) =
+        *reinterpret_cast<const uint4 *>(fp_w + row * F + c * 8);
+}
+
 }  // namespace
 }  // namespace quik
 
 using namespace quik;
+
+extern "C" int64_t quik_tile8_operand_bytes(int64_t rows, int64_t K, int64_t F) {
+  if (rows <= 0 || K <= 0 || K % 64 != 0 || F < 0 || F % 32 != 0) return 0;
+  return tile8_layout(rows, K, F).bytes;
+}
+
+extern "C" int quik_tile8_pack_weight(const int8_t *qw, const void *fp_w, int64_t N, int64_t K, int64_t F, void *out,
+                                      void *stream) {
+  if (N <= 0 || K <= 0 || F < 0) return QUIK_ERR_SHAPE;
+  if (K % 64 != 0 || F % 32 != 0) return QUIK_ERR_ALIGN;
+  if (!qw || !out || (F > 0 && !fp_w)) return QUIK_ERR_NULL;
+  if (reinterpret_cast<uintptr_t>(qw) % 16 != 0 || reinterpret_cast<uintptr_t>(out) % 256 != 0 ||
+      reinterpret_cast<uintptr_t>(fp_w) % 16 != 0)
+    return QUIK_ERR_ALIGN;
+  if (N > (1 << 30)) return QUIK_ERR_RANGE;
+  hipLaunchKernelGGL(pack_weight8_kernel, dim3(static_cast<unsigned>(N)), dim3(kThreads), 0, as_stream(stream),
+                     reinterpret_cast<const uint8_t *>(qw), static_cast<const uint16_t *>(fp_w), N, K, F,
+                     static_cast<uint8_t *>(out));
+  return check_launch();
+}
 
 extern "C" int64_t quik_fp6_operand_bytes(int64_t rows, int64_t K, int64_t F) {
   if (rows <= 0 || K <= 0 || K % 128 != 0 || F < 0 || F % 32 != 0) return 0;

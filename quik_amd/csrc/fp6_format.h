@@ -1,3 +1,5 @@
+// Operand formats of the GEMMs that read their operands in tile order.
+//
 // 6-bit operand format of the int4 GEMM on the E2M3 matrix-core path (consumer: gemm_fp6.h).
 //
 // A level L = code + 8 (0 .. 15) is stored as a 6-bit field holding L: as an E2M3 number that is
@@ -49,6 +51,26 @@ __host__ __device__ inline int64_t fp6_tail_offset(const Fp6Layout &l, int64_t r
 // 16-byte chunk c (8 values) of outlier step t
 __host__ __device__ inline int64_t fp6_outlier_offset(const Fp6Layout &l, int64_t row, int64_t t, int c) {
   return fp6_head_offset(l, row, l.steps + t, c);
+}
+
+// ---- int8 operands in the same order (consumer: gemm_tile8.h): unit (block B, step s) is 2 KB, a step is 32
+// int8 elements (or 16 fp16 / bf16 outlier values) = 32 bytes per row, two 16-byte chunks h per row
+struct Tile8Layout {
+  int64_t blocks, steps, fsteps, block_bytes, bytes;
+};
+__host__ __device__ inline Tile8Layout tile8_layout(int64_t rows, int64_t K, int64_t F) {
+  Tile8Layout l;
+  l.blocks = (rows + 63) / 64;
+  l.steps = K / 32;
+  l.fsteps = F / 16;
+  l.block_bytes = (l.steps + l.fsteps) * 2048;
+  l.bytes = l.blocks * l.block_bytes;
+  return l;
+}
+// 16-byte chunk h of step `step` (integer steps first, then outlier steps) of row `row`
+__host__ __device__ inline int64_t tile8_offset(const Tile8Layout &l, int64_t row, int64_t step, int h) {
+  return (row >> 6) * l.block_bytes + step * 2048 + ((row >> 5) & 1) * 1024 + (row & 31) * 32 +
+         ((h ^ ((row >> 3) & 1)) << 4);
 }
 
 // 4 levels in the bytes of w -> 24 bits, 6 per level

@@ -3,7 +3,7 @@
 #include <cstdint>
 
 #include "gemm_decode.h"
-#include "gemm_fp6.h"
+#include "gemm_tile8.h"
 #include "gemm_kernels.h"
 
 namespace quik {
@@ -316,6 +316,51 @@ int run_fused6(const Fused6Args &p, hipStream_t st) {
   return launch_fused6_split<CfgL, CfgH, BF16>(wide, tail, st);
 }
 
+template <class C, bool BF16>
+int launch_fused8t(const Fused8Args &p, hipStream_t st) {
+  if (p.N <= 0) return QUIK_OK;
+  int tiles_m, tiles_n;
+  const int grid = grid_of<C>(p.M, p.N, tiles_m, tiles_n);
+  auto kern = gemm_fused8t_kernel<C, BF16>;
+  constexpr int smem = fused8t_smem<C>();
+  if (int rc = prepare(kern, smem)) return rc;
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(C::kThreads), smem, st, p, tiles_m, tiles_n);
+  return check_launch();
+}
+
+template <class CW, class CT, bool BF16>
+int launch_fused8t_split(const Fused8Args &wide, const Fused8Args &tail, hipStream_t st) {
+  if (wide.N <= 0) return launch_fused8t<CT, BF16>(tail, st);
+  if (tail.N <= 0) return launch_fused8t<CW, BF16>(wide, st);
+  int tail_blocks;
+  SplitGrid grid = split_grid<CW, CT>(wide.M, wide.N, tail.N, tail_blocks);
+  grid.lead = 0;  // tiles of an XCD that share operand rows stay in step (L2 hits)
+  auto kern = gemm_fused8t_split_kernel<CW, CT, BF16>;
+  constexpr int smem = fused8t_smem<CW>() > fused8t_smem<CT>() ? fused8t_smem<CW>() : fused8t_smem<CT>();
+  if (int rc = prepare(kern, smem)) return rc;
+  hipLaunchKernelGGL(kern, dim3(grid.wide_blocks + tail_blocks), dim3(CW::kThreads), smem, st, wide, tail, grid);
+  return check_launch();
+}
+
+// W8A8 on tile-ordered operands (gemm_tile8.h): same plan and tile shapes as the 6-bit path.
+template <bool BF16>
+int run_fused8t(const Fused8Args &p, hipStream_t st) {
+  const Plan plan = make_plan6(p.M, p.N);
+  if (plan.kind == Plan::kSmall) return QUIK_ERR_SHAPE;  // at most 32 rows: the weight-streaming kernel is the right one
+  if (plan.kind != Plan::kSplit) return launch_fused8t<CfgM, BF16>(p, st);
+  if (plan.n_wide >= p.N) return launch_fused8t<CfgL8, BF16>(p, st);
+  Fused8Args wide = p, tail = p;
+  const int64_t nw = plan.n_wide;
+  wide.N = static_cast<int>(nw);
+  tail.N = static_cast<int>(p.N - nw);
+  tail.n_first = static_cast<int>(nw);
+  tail.s_col = p.s_col + nw;
+  tail.w_red = p.w_red + nw;
+  tail.bias = p.bias ? p.bias + nw : nullptr;
+  tail.out = p.out + nw;
+  return launch_fused8t_split<CfgL, CfgH, BF16>(wide, tail, st);
+}
+
 template <int MODE, bool BF16>
 int run_fused(const FusedArgs &p, hipStream_t st) {
   const Plan plan = make_plan(p.M, p.N, p.kbytes % 64 == 0 && (p.F * 2) % 64 == 0);
@@ -425,4 +470,35 @@ extern "C" int quik_mixed_linear_fwd_fp6(const void *x6, const void *w6, const v
   p.N_total = static_cast<int>(N);
   hipStream_t st = as_stream(stream);
   return dtype == QUIK_F16 ? run_fused6<false>(p, st) : run_fused6<true>(p, st);
+}
+
+extern "C" int quik_mixed_linear_fwd_tile8(const void *x8, const void *w8, const void *meta, const void *s_col,
+                                           const void *w_reduced, const void *bias, int dtype, int64_t M, int64_t N,
+                                           int64_t K, int64_t F, void *out, void *stream) {
+  if (dtype != QUIK_F16 && dtype != QUIK_BF16) return QUIK_ERR_DTYPE;
+  if (M < 0 || N < 0 || K <= 0 || F < 0) return QUIK_ERR_SHAPE;
+  if (M == 0 || N == 0) return QUIK_OK;
+  if (M <= 32) return QUIK_ERR_SHAPE;
+  if (!x8 || !w8 || !meta || !s_col || !w_reduced || !out) return QUIK_ERR_NULL;
+  if (K % 64 != 0 || F % 32 != 0) return QUIK_ERR_ALIGN;
+  auto misaligned = [](const void *p) { return reinterpret_cast<uintptr_t>(p) % 256 != 0; };
+  if (misaligned(x8) || misaligned(w8)) return QUIK_ERR_ALIGN;
+  if (M > (1 << 30) || N > (1 << 30) || K > (1 << 24)) return QUIK_ERR_RANGE;
+  Fused8Args p;
+  p.xbuf = static_cast<const uint8_t *>(x8);
+  p.wbuf = static_cast<const uint8_t *>(w8);
+  p.meta = static_cast<const uint16_t *>(meta);
+  p.s_col = static_cast<const uint16_t *>(s_col);
+  p.w_red = static_cast<const uint16_t *>(w_reduced);
+  p.bias = static_cast<const uint16_t *>(bias);
+  p.out = static_cast<uint16_t *>(out);
+  p.M = static_cast<int>(M);
+  p.N = static_cast<int>(N);
+  p.ldo = static_cast<int>(N);
+  p.K = static_cast<int>(K);
+  p.F = static_cast<int>(F);
+  p.n_first = 0;
+  p.N_total = static_cast<int>(N);
+  hipStream_t st = as_stream(stream);
+  return dtype == QUIK_F16 ? run_fused8t<false>(p, st) : run_fused8t<true>(p, st);
 }

@@ -414,8 +414,10 @@ __device__ __forceinline__ void stream_rows(const uint16_t *__restrict__ x, int6
   // vec_out: 0 byte-wise output, 1 16-byte output, 2 (4 bits only): dst is a 6-bit operand buffer
   // (fp6_format.h) for the matrix-core path of gemm_fp6.h, which also takes the outlier values (fp_x is
   // not written); needs num_int % 128 == 0 and num_fp % 32 == 0
+  // 3 (8 bits only): dst is an int8 operand buffer in tile order for gemm_tile8.h (same conditions)
   const Fp6Layout l6 = fp6_layout(rows, num_int, num_fp);
-  const bool to6 = BITS == 4 && vec_out == 2;
+  const Tile8Layout l8 = tile8_layout(rows, num_int, num_fp);
+  const bool to6 = BITS == 4 && vec_out == 2, to8 = BITS == 8 && vec_out == 3;
   const int tid = threadIdx.x;
   const int nvec = static_cast<int>(cols >> 3);
   const float inf = __builtin_inff();
@@ -513,8 +515,11 @@ __device__ __forceinline__ void stream_rows(const uint16_t *__restrict__ x, int6
     }
     // ---- outliers, in the caller's order
     auto fp_slot = [&](int64_t f) -> uint16_t * {
-      if (!to6) return fp_x + row * num_fp + f;
-      return reinterpret_cast<uint16_t *>(dst + fp6_outlier_offset(l6, row, f >> 4, static_cast<int>((f >> 3) & 1))) + (f & 7);
+      if (to6)
+        return reinterpret_cast<uint16_t *>(dst + fp6_outlier_offset(l6, row, f >> 4, static_cast<int>((f >> 3) & 1))) + (f & 7);
+      if (to8)
+        return reinterpret_cast<uint16_t *>(dst + tile8_offset(l8, row, l8.steps + (f >> 4), static_cast<int>((f >> 3) & 1))) + (f & 7);
+      return fp_x + row * num_fp + f;
     };
 #pragma unroll
     for (int k = 0; k < ND; ++k)
@@ -618,7 +623,7 @@ __device__ __forceinline__ void stream_rows(const uint16_t *__restrict__ x, int6
             drow[b] = static_cast<uint8_t>((b < 4 ? packed.x : packed.y) >> (8 * (b & 3)));
         }
       } else {
-        uint8_t *drow = dst + row * num_int + u * 16;
+        uint8_t *drow = to8 ? dst + tile8_offset(l8, row, u >> 1, u & 1) : dst + row * num_int + u * 16;
         if (valid >= 16 && vec_out) {
           *reinterpret_cast<uint4 *>(drow) = c;
         } else {
@@ -634,14 +639,14 @@ __device__ __forceinline__ void stream_rows(const uint16_t *__restrict__ x, int6
   // No software prefetch: the launch makes one workgroup per row (up to the grid limit), several of
   // them are resident per CU, and their phases drift apart, so loads, arithmetic and stores of
   // different rows overlap.
-  // 6-bit output: a cache line of the operand buffer takes pieces of 4 (heads) or 16 (tails) consecutive rows.
+  // Tile-ordered output: a cache line of the operand buffer takes pieces of 4 (heads) or 16 (tails) consecutive rows.
   // Workgroups are dealt round-robin to the 8 XCDs, so workgroup w takes row (w % 8) * rows / 8 + w / 8: rows
   // that share lines then run at about the same time on the same XCD and meet in its L2.
   const int64_t per_xcd = (rows + 7) >> 3;
-  const int64_t items = to6 ? per_xcd * 8 : rows;
+  const int64_t items = (to6 || to8) ? per_xcd * 8 : rows;
   int parity = 0;
   for (int64_t w = blockIdx.x; w < items; w += gridDim.x) {
-    const int64_t row = to6 ? (w & 7) * per_xcd + (w >> 3) : w;
+    const int64_t row = (to6 || to8) ? (w & 7) * per_xcd + (w >> 3) : w;
     if (row >= rows) continue;
     parity ^= 1;
     uint4 cur[NV], dv[ND];
@@ -830,7 +835,7 @@ constexpr int64_t kMaxLdsRowBytes = 128 * 1024;  // of the 160 KB per CU
 
 template <typename IdxT, int BITS, bool BF16, int NV, int TPR>
 int launch_stream(const void *x, int64_t rows, int64_t cols, const uint8_t *cm, const ColmapLayout &l, int64_t num_int,
-                  int64_t num_fp, void *dst, void *meta, void *fp_x, hipStream_t st, bool fp6) {
+                  int64_t num_fp, void *dst, void *meta, void *fp_x, hipStream_t st, bool tiled) {
   auto kern = asym_quantize_stream_kernel<IdxT, BITS, BF16, NV, TPR>;
   const int64_t lds = align16(cols * 2);  // >= align16(num_int)
   if (lds > 48 * 1024) {
@@ -841,9 +846,10 @@ int launch_stream(const void *x, int64_t rows, int64_t cols, const uint8_t *cm, 
       return QUIK_ERR_LAUNCH;
     }
   }
-  const int64_t items = fp6 ? (rows + 7) / 8 * 8 : rows;
+  const int64_t items = tiled ? (rows + 7) / 8 * 8 : rows;
   const int grid = static_cast<int>(items < (int64_t(1) << 30) ? items : (int64_t(1) << 30));
-  const int vec_out = fp6 ? 2 : (num_int % 16 == 0 && reinterpret_cast<uintptr_t>(dst) % 16 == 0);
+  // tiled: dst is an operand buffer in tile order (6-bit levels for 4 bits, int8 for 8 bits)
+  const int vec_out = tiled ? (BITS == 4 ? 2 : 3) : (num_int % 16 == 0 && reinterpret_cast<uintptr_t>(dst) % 16 == 0);
   hipLaunchKernelGGL(kern, dim3(grid), dim3(TPR), static_cast<size_t>(lds), st,
                      static_cast<const uint16_t *>(x), rows, cols, reinterpret_cast<const IdxT *>(cm),
                      reinterpret_cast<const IdxT *>(cm + l.off_fp), reinterpret_cast<const uint32_t *>(cm + l.off_mask),
@@ -857,7 +863,7 @@ int launch_stream(const void *x, int64_t rows, int64_t cols, const uint8_t *cm, 
 
 template <typename IdxT, int BITS, bool BF16>
 int launch_asym(const void *x, int64_t rows, int64_t cols, const uint8_t *cm, const ColmapLayout &l, int64_t num_int,
-                int64_t num_fp, void *dst, void *meta, void *fp_x, hipStream_t st, bool fp6 = false) {
+                int64_t num_fp, void *dst, void *meta, void *fp_x, hipStream_t st, bool tiled = false) {
   const IdxT *src_col = reinterpret_cast<const IdxT *>(cm);
   const IdxT *fp_col = reinterpret_cast<const IdxT *>(cm + l.off_fp);
   const uint32_t *mask = reinterpret_cast<const uint32_t *>(cm + l.off_mask);
@@ -866,14 +872,14 @@ int launch_asym(const void *x, int64_t rows, int64_t cols, const uint8_t *cm, co
     // better than fewer waves with less per-row fixed work (measured with 64, 128 and 256 threads).
     const int64_t groups = cols / 8;
 #define QUIK_STREAM(NV) \
-  return launch_stream<IdxT, BITS, BF16, NV, kThreads>(x, rows, cols, cm, l, num_int, num_fp, dst, meta, fp_x, st, fp6)
+  return launch_stream<IdxT, BITS, BF16, NV, kThreads>(x, rows, cols, cm, l, num_int, num_fp, dst, meta, fp_x, st, tiled)
     if (groups <= 512) QUIK_STREAM(2);
     if (groups <= 1024) QUIK_STREAM(4);
     if (groups <= 2048) QUIK_STREAM(8);
     QUIK_STREAM(16);
 #undef QUIK_STREAM
   }
-  if (fp6) return QUIK_ERR_SHAPE;  // the 6-bit output exists on the streaming path only
+  if (tiled) return QUIK_ERR_SHAPE;  // tile-ordered output exists on the streaming path only
   const int grid = static_cast<int>(rows < 65535 * 8 ? rows : 65535 * 8);
   const int64_t lds = align16(cols * 2);
   if (lds <= kMaxLdsRowBytes) {
@@ -993,6 +999,22 @@ extern "C" int quik_asym_quantize_fp6(const void *x, int dtype, int64_t rows, in
   return dtype == QUIK_F16
              ? launch_asym<uint16_t, 4, false>(x, rows, cols, cm, l, num_int, num_fp, out6, meta, fp_x, st, true)
              : launch_asym<uint16_t, 4, true>(x, rows, cols, cm, l, num_int, num_fp, out6, meta, fp_x, st, true);
+}
+
+extern "C" int quik_asym_quantize_tile8(const void *x, int dtype, int64_t rows, int64_t cols, const void *colmap,
+                                        int64_t num_int, int64_t num_fp, void *out8, void *meta, void *stream) {
+  if (dtype != QUIK_F16 && dtype != QUIK_BF16) return QUIK_ERR_DTYPE;
+  if (rows < 0 || cols <= 0 || num_int <= 0 || num_fp < 0 || num_int + num_fp != cols) return QUIK_ERR_SHAPE;
+  if (num_int % 64 != 0 || num_fp % 32 != 0 || cols > kStreamMaxCols) return QUIK_ERR_ALIGN;
+  if (rows == 0) return QUIK_OK;
+  if (!x || !colmap || !out8 || !meta) return QUIK_ERR_NULL;
+  if (reinterpret_cast<uintptr_t>(x) % 16 != 0 || reinterpret_cast<uintptr_t>(out8) % 256 != 0) return QUIK_ERR_ALIGN;
+  const ColmapLayout l = colmap_layout(cols, num_int, num_fp);
+  const uint8_t *cm = static_cast<const uint8_t *>(colmap);
+  hipStream_t st = as_stream(stream);
+  return dtype == QUIK_F16
+             ? launch_asym<uint16_t, 8, false>(x, rows, cols, cm, l, num_int, num_fp, out8, meta, nullptr, st, true)
+             : launch_asym<uint16_t, 8, true>(x, rows, cols, cm, l, num_int, num_fp, out8, meta, nullptr, st, true);
 }
 
 extern "C" int quik_asym_find_meta(const void *x, int64_t rows, int64_t cols, int bits, void *meta, void *stream) {

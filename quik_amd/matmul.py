@@ -12,7 +12,8 @@ import torch
 
 from . import _lib as L
 
-__all__ = ["int4Matmul", "int8Matmul", "mixed_linear", "pack_weight_fp6", "mixed_linear_fp6"]
+__all__ = ["int4Matmul", "int8Matmul", "mixed_linear", "pack_weight_fp6", "mixed_linear_fp6", "pack_weight_tile8",
+           "mixed_linear_tile8"]
 
 
 def _matmul(op, A, B, want_dtype, sym, kmul):
@@ -129,4 +130,51 @@ def mixed_linear_fp6(x6, w6, meta, weights_scales, reduced_w, bias, M, N, K, F, 
         L.check(lib.quik_mixed_linear_fwd_fp6(L.ptr(x6), L.ptr(w6), L.ptr(meta), L.ptr(weights_scales),
                                               L.ptr(reduced_w), L.ptr(tensors.get("bias")), dt, M, N, K, F,
                                               L.ptr(out), L.stream()), "mixed_linear_fp6")
+    return out
+
+
+def pack_weight_tile8(int_weight: torch.Tensor, fp_weight: torch.Tensor) -> torch.Tensor:
+    """int8 weights [N, K] and outlier weights [N, F] -> tile-ordered operand buffer for mixed_linear_tile8
+    (once per layer)."""
+    L.check_cuda_contiguous("pack_weight_tile8", int_weight=int_weight, fp_weight=fp_weight)
+    if int_weight.dtype != torch.int8 or int_weight.dim() != 2:
+        raise RuntimeError("pack_weight_tile8: expected an int8 [N, K] int_weight")
+    if fp_weight.dtype not in (torch.float16, torch.bfloat16) or fp_weight.dim() != 2 or \
+            fp_weight.size(0) != int_weight.size(0):
+        raise RuntimeError("pack_weight_tile8: expected an fp16/bf16 [N, F] fp_weight")
+    N, K, F = int_weight.size(0), int_weight.size(1), fp_weight.size(1)
+    lib = L.load()
+    nbytes = lib.quik_tile8_operand_bytes(N, K, F)
+    if nbytes == 0:
+        raise RuntimeError("pack_weight_tile8: K must be a multiple of 64 and F a multiple of 32")
+    with torch.cuda.device(int_weight.device):
+        out = torch.empty((nbytes,), dtype=torch.uint8, device=int_weight.device)
+        L.check(lib.quik_tile8_pack_weight(L.ptr(int_weight), L.ptr(fp_weight) if F else None, N, K, F, L.ptr(out),
+                                           L.stream()), "pack_weight_tile8")
+    return out
+
+
+def mixed_linear_tile8(x8, w8, meta, weights_scales, reduced_w, bias, M, N, K, F, out_dtype):
+    """mixed_linear (asymmetric, 8 bits) on tile-ordered operand buffers (asymmetric.quantize_mapped_tile8,
+    pack_weight_tile8): same result bit for bit, every operand cache line fetched once per tile."""
+    tensors = dict(x8=x8, w8=w8, meta=meta, weights_scales=weights_scales, reduced_w=reduced_w)
+    if bias is not None and bias.numel() > 0:
+        tensors["bias"] = bias
+    L.check_cuda_contiguous("mixed_linear_tile8", **tensors)
+    dt = L.QUIK_F16 if out_dtype == torch.float16 else L.QUIK_BF16 if out_dtype == torch.bfloat16 else None
+    if dt is None:
+        raise RuntimeError(f"mixed_linear_tile8: unsupported dtype {out_dtype}")
+    for name, t in tensors.items():
+        if name not in ("x8", "w8") and t.dtype != out_dtype:
+            raise RuntimeError(f"mixed_linear_tile8: expected {name} of dtype {out_dtype} but got {t.dtype}")
+    lib = L.load()
+    if x8.numel() != lib.quik_tile8_operand_bytes(M, K, F) or w8.numel() != lib.quik_tile8_operand_bytes(N, K, F):
+        raise RuntimeError("mixed_linear_tile8: operand buffers do not match M, N, K, F")
+    if meta.numel() != 2 * M or weights_scales.numel() != N or reduced_w.numel() != N:
+        raise RuntimeError("mixed_linear_tile8: meta / weights_scales / reduced_w sizes are inconsistent with M, N")
+    with torch.cuda.device(x8.device):
+        out = torch.empty((M, N), dtype=out_dtype, device=x8.device)
+        L.check(lib.quik_mixed_linear_fwd_tile8(L.ptr(x8), L.ptr(w8), L.ptr(meta), L.ptr(weights_scales),
+                                                L.ptr(reduced_w), L.ptr(tensors.get("bias")), dt, M, N, K, F,
+                                                L.ptr(out), L.stream()), "mixed_linear_tile8")
     return out
