@@ -45,7 +45,7 @@ class SharedQuantizedInput:
         self.fp_x = None
         self.qscale_x = None
         self.meta = None
-        self.x6 = None  # activation in the 6-bit operand format (codes and outlier values), see MixedQLinear
+        self.x6 = None  # activation as a tile-ordered operand buffer (codes and outlier values), see MixedQLinear
         self.group_size = group_size
         self.cur_group_elem = 0
 
@@ -63,12 +63,14 @@ class SharedQuantizedInput:
 class MixedQLinear(torch.nn.Module):
     """The reference's layer (qlinear.py:40-145) on the HIP kernels.
 
-    W4A4 asymmetric calls with at least `six_bit_min_rows` token rows (everything above decode size) run their int4 products on the
-    6-bit (E2M3) matrix-core path, which has twice the int8 rate: levels code + 8 are exact E2M3 numbers
-    and the integer accumulator is recovered exactly, so the output is bit-identical to the int8-MFMA
-    path.  It needs int_features % 128 == 0, fp_features % 32 == 0 and ascending int_indices, and keeps a
-    second copy of the weights in the operand format of that path (0.75 bytes per int4 weight plus the
-    outlier columns, built on first use); `six_bit_path = False` turns it off."""
+    Asymmetric calls with at least `six_bit_min_rows` token rows (everything above decode size) read both
+    operands in tile order (`tiled_path`; the quantize kernel writes the activation that way, the weights
+    get a second, repacked copy on first use), so every operand cache line is fetched once per tile.
+    W4A4: the int4 products run on the 6-bit (E2M3) matrix-core instructions, which have twice the int8 rate:
+    levels code + 8 are exact E2M3 numbers and the integer accumulator is recovered exactly (needs
+    int_features % 128 == 0; 0.75 bytes per weight).  W8A8: int8 MFMA as before (int_features % 64 == 0;
+    1 byte per weight).  Both need fp_features % 32 == 0 and ascending int_indices and give the output bits
+    of the row-major kernels; `six_bit_path = False` turns them off."""
 
     six_bit_min_rows = 33    # up to 32 rows the weight-streaming decode kernel on the packed int4 weights is the right one
 
@@ -117,9 +119,11 @@ class MixedQLinear(torch.nn.Module):
 
     # -- 6-bit matrix-core path: eligibility and the cached weight operand
     def _six_bit_ok(self, rows):
-        if not (self.six_bit_path and self.fused and not self.symmetric and self.bits == 4):
+        """True if this call takes the tile-ordered path (6-bit matrix-core GEMM for 4 bits, int8 for 8 bits)."""
+        if not (self.six_bit_path and self.fused and not self.symmetric and self.bits in (4, 8)):
             return False
-        if rows < self.six_bit_min_rows or self.int_features_num % 128 != 0 or self.fp_features_num % 32 != 0:
+        k_multiple = 128 if self.bits == 4 else 64
+        if rows < self.six_bit_min_rows or self.int_features_num % k_multiple != 0 or self.fp_features_num % 32 != 0:
             return False
         colmap = self._column_map()
         if self._streams is None:  # one device-to-host word and a stream synchronisation, once per column map
@@ -132,7 +136,8 @@ class MixedQLinear(torch.nn.Module):
         key = (self.int_weight.data_ptr(), self.int_weight._version, fp_w.data_ptr(), fp_w._version,
                self.int_weight.device)
         if self._w6 is None or self._w6_key != key:
-            self._w6 = matmul.pack_weight_fp6(self.int_weight, fp_w)
+            pack = matmul.pack_weight_fp6 if self.bits == 4 else matmul.pack_weight_tile8
+            self._w6 = pack(self.int_weight, fp_w)
             self._w6_key = key
         return self._w6
 
@@ -163,13 +168,14 @@ class MixedQLinear(torch.nn.Module):
         shared_input = self.shared_input if self.shared_input is not None else SharedQuantizedInput(1)
         with torch.cuda.device(x.device):
             if x2.data_ptr() % 16 == 0 and self._six_bit_ok(x2.shape[0]):
+                quantize6 = asymmetric.quantize_mapped_fp6 if self.bits == 4 else asymmetric.quantize_mapped_tile8
+                linear6 = matmul.mixed_linear_fp6 if self.bits == 4 else matmul.mixed_linear_tile8
                 if shared_input.x6 is None:
-                    shared_input.x6, shared_input.meta = asymmetric.quantize_mapped_fp6(
+                    shared_input.x6, shared_input.meta = quantize6(
                         x2, self._column_map(), self.int_features_num, self.fp_features_num)
-                output = matmul.mixed_linear_fp6(shared_input.x6, self._weight6(), shared_input.meta,
-                                                 self.weights_scales, self.reduced_w, self.bias, x2.shape[0],
-                                                 self.out_features, self.int_features_num, self.fp_features_num,
-                                                 self.dtype)
+                output = linear6(shared_input.x6, self._weight6(), shared_input.meta,
+                                 self.weights_scales, self.reduced_w, self.bias, x2.shape[0],
+                                 self.out_features, self.int_features_num, self.fp_features_num, self.dtype)
                 shared_input.finish()
                 return output.reshape(*lead, self.out_features)
             if shared_input.qint_x is None:

@@ -946,6 +946,46 @@ def test_six_bit_operand_buffers_hold_the_int4_codes(rows, K, F, bf16):
     assert np.array_equal(sums, want.sum(1))
 
 
+def test_tile8_operand_buffers_hold_the_int8_codes():
+    """quantize_mapped_tile8 / pack_weight_tile8: the int8 codes of quantize_mapped / int_weight and the outlier
+    values, at the documented places (quik_amd/csrc/gemm_tile8.h)."""
+    from quik_amd import asymmetric, matmul
+    rng = np.random.default_rng(8)
+    rows, K, F = 100, 192, 32
+    n_in = K + F
+    ii, fi = _split(rng, n_in, F)
+    x = _edge_rows(_acts(rng, rows, n_in, fi).astype(np.float16), ii)
+    colmap = asymmetric.build_colmap(_t(ii), _t(fi), n_in)
+    q, meta, fp_x = asymmetric.quantize_mapped(_t(x), colmap, K, F, 8)
+    x8, meta8 = asymmetric.quantize_mapped_tile8(_t(x), colmap, K, F)
+    assert np.array_equal(_bits(meta), _bits(meta8))
+    qw = rng.integers(-128, 128, (rows, K)).astype(np.int8)
+    fpw = (0.02 * rng.standard_normal((rows, F))).astype(np.float16)
+    w8 = matmul.pack_weight_tile8(_t(qw), _t(fpw))
+
+    def decode(buf):
+        steps, fsteps = K // 32, F // 16
+        block_bytes = (steps + fsteps) * 2048
+        assert buf.size == ((rows + 63) // 64) * block_bytes
+        codes, outl = np.zeros((rows, K), np.int8), np.zeros((rows, F), np.uint16)
+        for r in range(rows):
+            base = (r >> 6) * block_bytes + ((r >> 5) & 1) * 1024 + (r & 31) * 32
+            for s_ in range(steps + fsteps):
+                for h in range(2):
+                    chunk = bytes(buf[base + s_ * 2048 + ((h ^ ((r >> 3) & 1)) << 4):][:16])
+                    if s_ < steps:
+                        codes[r, s_ * 32 + h * 16: s_ * 32 + h * 16 + 16] = np.frombuffer(chunk, np.int8)
+                    else:
+                        t = s_ - steps
+                        outl[r, t * 16 + h * 8: t * 16 + h * 8 + 8] = np.frombuffer(chunk, np.uint16)
+        return codes, outl
+
+    codes, outl = decode(x8.cpu().numpy())
+    assert np.array_equal(codes, q.cpu().numpy()) and np.array_equal(outl, _bits(fp_x).reshape(rows, F))
+    codes, outl = decode(w8.cpu().numpy())
+    assert np.array_equal(codes, qw) and np.array_equal(outl, fpw.view(np.uint16))
+
+
 SIX_CASES = [
     # M, N, in, F, bias, kind: K = in - F a multiple of 128, F a multiple of 32, M > 32
     (33, 200, 544, 32, True, "x50"),          # smallest row count of the path
@@ -963,18 +1003,20 @@ SIX_CASES = [
 
 @pytest.mark.parametrize("case", SIX_CASES)
 @pytest.mark.parametrize("bf16", [False, True])
-def test_six_bit_path_is_bit_identical_to_the_int8_path(case, bf16):
-    """MixedQLinear on the 6-bit (E2M3) matrix-core path against the same layer on the int8-MFMA path (which the
-    other tests hold against the oracle): identical output bits, NaN / Inf rows included."""
+@pytest.mark.parametrize("bits", [4, 8])
+def test_six_bit_path_is_bit_identical_to_the_int8_path(case, bf16, bits):
+    """MixedQLinear on the tile-ordered operands (4 bits: 6-bit E2M3 matrix-core GEMM; 8 bits: int8 MFMA) against
+    the same layer on the row-major int8-MFMA kernels (which the other tests hold against the oracle): identical
+    output bits, NaN / Inf rows included."""
     from quik_amd.qlinear import MixedQLinear
     M, N, n_in, F, with_bias, kind = case
-    rng = np.random.default_rng(sum(case[:4]) + bf16)
-    W, s_w, ii, fi = _layer(rng, N, n_in, F, 4)
+    rng = np.random.default_rng(sum(case[:4]) + bf16 + bits)
+    W, s_w, ii, fi = _layer(rng, N, n_in, F, bits)
     bias = rng.standard_normal(N).astype(np.float16) if with_bias else None
     x = _edge_rows(_acts(rng, M, n_in, fi, kind).astype(np.float16), ii)
     mods = []
     for six in (True, False):
-        mod = _module(W, s_w, fi, 4, bias)
+        mod = _module(W, s_w, fi, bits, bias)
         if bf16:
             mod = mod.to(torch.bfloat16)
             mod.dtype = torch.bfloat16
@@ -986,9 +1028,9 @@ def test_six_bit_path_is_bit_identical_to_the_int8_path(case, bf16):
     assert out6.shape == out8.shape == (1, M, N)
     assert np.array_equal(_bits(out6), _bits(out8))
     if not bf16:                                                # and against the oracle, on a slice of the rows
-        omod = qo.from_float(W, s_w, fi, 4)
+        omod = qo.from_float(W, s_w, fi, bits)
         rows = np.r_[0:24, M - 8:M]
-        want, _ = qo.mixed_qlinear_forward(x[rows], omod, 4, bias)
+        want, _ = qo.mixed_qlinear_forward(x[rows], omod, bits, bias)
         got = out6[0].float().cpu().numpy()[rows]
         fin = np.isfinite(want)
         assert np.array_equal(np.isfinite(got), fin)
