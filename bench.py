@@ -121,7 +121,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--unfused", action="store_true", help="run the reference's three-op sequence instead")
     ap.add_argument("--int8-mfma", action="store_true",
-                    help="W4A4: keep the int4 products on the int8 MFMA path (same output bits as the 6-bit path)")
+                    help="row-major operands on the int8 MFMA kernels instead of the tile-ordered paths (same output bits)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run only plain device-to-device copies of a 256 MiB buffer (known traffic: 256 MiB read, "
                          "256 MiB written per launch) to scale the FETCH_SIZE / WRITE_SIZE counters")
@@ -158,23 +158,26 @@ def main():
 
     from quik_amd import asymmetric, matmul
     colmap = mod._column_map()
-    six = mod.fused and not args.int8_mfma and mod._six_bit_ok(M)   # the path MixedQLinear.forward takes
+    # the path MixedQLinear.forward takes: tile-ordered operands (4 bits: 6-bit matrix-core GEMM, 8 bits: int8 MFMA)
+    six = mod.fused and not args.int8_mfma and mod._six_bit_ok(M)
     w6 = mod._weight6() if six else None
+
+    quantize6 = asymmetric.quantize_mapped_fp6 if bits == 4 else asymmetric.quantize_mapped_tile8
+    linear6 = matmul.mixed_linear_fp6 if bits == 4 else matmul.mixed_linear_tile8
 
     def quantize_only():
         if six:
-            return asymmetric.quantize_mapped_fp6(x, colmap, K, F)
+            return quantize6(x, colmap, K, F)
         return asymmetric.quantize_mapped(x, colmap, K, F, bits)
 
     def step(ev=None):
         if ev is not None:
             ev[0].record()
         if six:
-            x6, meta = asymmetric.quantize_mapped_fp6(x, colmap, K, F)
+            x6, meta = quantize6(x, colmap, K, F)
             if ev is not None:
                 ev[1].record()
-            out = matmul.mixed_linear_fp6(x6, w6, meta, mod.weights_scales, mod.reduced_w, mod.bias, M, N, K, F,
-                                          torch.float16)
+            out = linear6(x6, w6, meta, mod.weights_scales, mod.reduced_w, mod.bias, M, N, K, F, torch.float16)
             if ev is not None:
                 ev[2].record()
             return out
@@ -248,12 +251,15 @@ def main():
     gemm_tops = int_ops / (g_avg * 1e-3) / 1e12
     # read the row once; write the codes (6 bits each in the operand format of the 6-bit path, plus a 4-byte
     # level sum per row), the outlier values and the (scale, zero) pair
-    quant_bytes = M * n_in * 2 + (M * K * 6 // 8 + M * 4 if six else M * K * bits // 8) + M * F * 2 + M * 4
+    quant_bytes = M * n_in * 2 + (M * K * 6 // 8 + M * 4 if six and bits == 4 else M * K * bits // 8) + M * F * 2 + M * 4
     quant_gbps = quant_bytes / (q_avg * 1e-3) / 1e9
-    peak = PEAK_FP6_TOPS if six else PEAK_INT8_TOPS
-    if six:
-        gemm_kernel = "gemm_fused6_split_kernel (one launch per step)"
+    peak = PEAK_FP6_TOPS if six and bits == 4 else PEAK_INT8_TOPS
+    if six and bits == 4:
+        gemm_kernel = "gemm_fused6_split_kernel / gemm_fused6_kernel (one launch per step)"
         dtype = "int4 (exact, as E2M3 on the 6-bit MFMA path)"
+    elif six:
+        gemm_kernel = "gemm_fused8t_split_kernel / gemm_fused8t_kernel (tile-ordered int8 operands, one launch per step)"
+        dtype = "int8"
     elif mod.fused:
         gemm_kernel = "gemm_fused_split_kernel (one launch per step)"
         dtype = "int8" if bits == 8 else "int4 (on int8 MFMA)"
@@ -269,7 +275,7 @@ def main():
         "config": {"workload": f"{name}: MixedQLinear fwd, tokens={M}, in={n_in}, out={N}, fp16 outliers={F}, "
                                f"W{bits}A{bits} asymmetric per-token, fp16 activations, "
                                f"{'fused GEMM+dequant' if mod.fused else 'unfused three-op sequence'}"
-                               f"{', 6-bit matrix-core path' if six else ''}",
+                               f"{', 6-bit matrix-core path' if six and bits == 4 else ', tile-ordered operands' if six else ''}",
                    "M": M, "in_features": n_in, "K": K, "N": N, "F": F, "bits": bits},
         "pct_int8_mfma_peak": round(100.0 * tops / PEAK_INT8_TOPS, 2),
         "graph_replay_ms_per_step": None if graph_ms is None else round(graph_ms, 4),
@@ -280,7 +286,7 @@ def main():
                      "traffic": traffic.get("gemm6" if six else "gemm") if mod.fused else None,
                      "avg_ms": round(g_avg, 4), "median_ms": round(g_ms[len(g_ms) // 2], 4),
                      "algorithmic_ops": int_ops},
-        "roofline_quantize": {"kernel": "asym_quantize_stream_kernel" + (" (6-bit operand output)" if six else ""),
+        "roofline_quantize": {"kernel": "asym_quantize_stream_kernel" + (" (tile-ordered operand output)" if six else ""),
                               "bound": "hbm",
                               "achieved": round(quant_gbps, 1),
                               "peak": PEAK_HBM_GBPS, "unit": "GB/s", "frac": round(quant_gbps / PEAK_HBM_GBPS, 4),
