@@ -1064,3 +1064,46 @@ def test_six_bit_path_shared_input_and_fallbacks():
     small = xt[:20].contiguous()                               # decode size: int4 path, weight-streaming kernel
     assert torch.equal(mods[0](small), singles[0](small))
     shared.finish(), shared.finish()
+
+
+def test_tile_ordered_paths_random_shapes():
+    """Op-level sweep of the two tile-ordered paths (quantize + fused GEMM) against the row-major kernels over random
+    shapes, ragged in M and N, both dtypes, with and without bias and outliers: identical bits."""
+    from quik_amd import asymmetric, matmul
+    rng = np.random.default_rng(2024)
+    for it in range(16):
+        bits = int(rng.choice([4, 8]))
+        K = (128 if bits == 4 else 64) * int(rng.integers(1, 24))
+        F = 32 * int(rng.integers(0, 6))
+        M = int(rng.choice([33, 65, 129, 200, 257, 511, 777, 1500, 2049]))
+        N = int(rng.choice([8, 100, 130, 384, 520, 1000, 2048, 4160]))
+        dt = torch.bfloat16 if rng.integers(0, 2) else torch.float16
+        g = torch.Generator().manual_seed(it)
+        n_in = K + F
+        x = torch.randn(M, n_in, generator=g)
+        fi = torch.randperm(n_in, generator=g)[:F]
+        x[:, fi] *= 50
+        x = x.to(dt).to(DEV)
+        keep = torch.ones(n_in, dtype=torch.bool)
+        keep[fi] = False
+        ii = torch.arange(n_in)[keep]
+        cm = asymmetric.build_colmap(ii.to(DEV), fi.to(DEV), n_in)
+        if bits == 4:
+            qw = torch.randint(0, 256, (N, K // 2), dtype=torch.uint8, generator=g).to(DEV)
+        else:
+            qw = torch.randint(-128, 128, (N, K), dtype=torch.int8, generator=g).to(DEV)
+        s_w = (torch.rand(N, 1, generator=g) * 0.009 + 0.001).to(dt).to(DEV)
+        wred = torch.randn(1, N, generator=g).to(dt).to(DEV)
+        fpw = (0.02 * torch.randn(N, F, generator=g)).to(dt).to(DEV)
+        bias = torch.randn(N, generator=g).to(dt).to(DEV) if rng.integers(0, 2) else None
+        q, meta, fp = asymmetric.quantize_mapped(x, cm, K, F, bits)
+        want = matmul.mixed_linear(q, qw, meta, s_w, wred, fp if F else None, fpw if F else None, bias, bits, dt)
+        if bits == 4:
+            xb, meta2 = asymmetric.quantize_mapped_fp6(x, cm, K, F)
+            got = matmul.mixed_linear_fp6(xb, matmul.pack_weight_fp6(qw, fpw), meta2, s_w, wred, bias, M, N, K, F, dt)
+        else:
+            xb, meta2 = asymmetric.quantize_mapped_tile8(x, cm, K, F)
+            got = matmul.mixed_linear_tile8(xb, matmul.pack_weight_tile8(qw, fpw), meta2, s_w, wred, bias, M, N, K, F, dt)
+        case = (it, bits, M, N, K, F, dt)
+        assert np.array_equal(_bits(meta), _bits(meta2)), case
+        assert np.array_equal(_bits(got), _bits(want)), case
