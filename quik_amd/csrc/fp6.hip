@@ -89,7 +89,7 @@ extern "C" int quik_tile8_pack_weight(const int8_t *qw, const void *fp_w, int64_
 }
 
 extern "C" int64_t quik_fp6_operand_bytes(int64_t rows, int64_t K, int64_t F) {
-  if (rows <= 0 || K <= 0 || K % 128 != 0 || F < 0 || F % 32 != 0) return 0;
+  if (rows <= 0 || K <= 0 || K % 128 != 0 || K > 74496 || F < 0 || F % 32 != 0) return 0;
   return fp6_layout(rows, K, F).bytes;
 }
 
@@ -101,7 +101,7 @@ extern "C" int quik_fp6_pack_weight(const uint8_t *qw, const void *fp_w, int64_t
   if (reinterpret_cast<uintptr_t>(qw) % 16 != 0 || reinterpret_cast<uintptr_t>(out) % 256 != 0 ||
       reinterpret_cast<uintptr_t>(fp_w) % 16 != 0)
     return QUIK_ERR_ALIGN;
-  if (N > (1 << 30) || K >= 131072) return QUIK_ERR_RANGE;
+  if (N > (1 << 30) || K > 74496) return QUIK_ERR_RANGE;
   hipLaunchKernelGGL(pack_weight_kernel, dim3(static_cast<unsigned>(N)), dim3(kThreads), 0, as_stream(stream), qw,
                      static_cast<const uint16_t *>(fp_w), N, K, F, static_cast<uint8_t *>(out));
   return check_launch();

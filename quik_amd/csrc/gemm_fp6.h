@@ -3,11 +3,13 @@
 // v_mfma_f32_32x32x64_f8f6f4 with 6-bit E2M3 operands runs at twice the rate of the int8 MFMA.
 // The E2M3 bit patterns 0 .. 15 (sign 0, exponent 00 / 01) are the uniformly spaced values
 // L / 8, so a 4-bit level L = code + 8 IS an E2M3 number, zero-extended to 6 bits.  Products
-// La Lw / 64 are multiples of 1/64 and their sum over K stays below 2^15 for K < 131072, so the
-// fp32 accumulation is exact, and
+// La Lw / 64 are multiples of 1/64 and their sum over K stays below 2^24 / 64 for K <= 74496 (225 K <
+// 2^24), so the fp32 accumulation is exact in any order, and
 //     sum_k a_k w_k = 64 S - 8 sum_k La_k - 8 sum_k Lw_k + 64 K,      S = sum_k (La_k / 8)(Lw_k / 8)
-// recovers the integer accumulator exactly (every term is an integer below 2^24).  From there
-// the epilogue is the one of gemm_kernels.h, so the output is bit-identical to the int8-MFMA path.
+// recovers the integer accumulator exactly (every term is an integer below 2^24).  The accumulators
+// start at -(8 sum_k Lw_k) / 64 (a multiple of 1/8, so still exact), and one fused multiply-add per value,
+// 64 acc - (8 sum_k La_k - 64 K), finishes the job.  From there the epilogue is the one of
+// gemm_kernels.h, so the output is bit-identical to the int8-MFMA path.
 //
 // Operand format: fp6_format.h.  Both operand buffers are stored as the sequence of LDS images the
 // tiles need, so a copy instruction moves one contiguous kilobyte and every cache line is requested
@@ -371,7 +373,7 @@ struct Fused6Args {
 };
 
 // Per-tile vectors in LDS behind the ring: the five of TileVectors plus the two integer corrections
-//   rowc[m] = 8 sum_k Lx - 64 K,  colc[n] = 8 sum_k Lw   (exact in fp32).
+//   rowc[m] = 8 sum_k Lx - 64 K,  colc[n] = -(8 sum_k Lw) / 64 (the accumulators' start value)   (exact in fp32).
 template <class C>
 struct TileVectors6 {
   static constexpr int kBytes = (4 * C::BN + 3 * C::BM) * 4;
@@ -408,7 +410,7 @@ __device__ __forceinline__ void fused6_tile(const Fused6Args &p, int tm, int tn,
       tv.scol[i] = to_f32<BF16>(p.s_col[n]);
       tv.wred[i] = to_f32<BF16>(p.w_red[n]);
       tv.bias[i] = p.bias ? to_f32<BF16>(p.bias[n]) : 0.0f;
-      tv.colc[i] = static_cast<float>(8 * ws[p.n_first + n]);
+      tv.colc[i] = static_cast<float>(ws[p.n_first + n]) * -0.125f;
     }
     for (int i = threadIdx.x; i < C::BM; i += C::kThreads) {
       const int64_t m = m0 + i < p.M ? m0 + i : p.M - 1;
@@ -419,20 +421,23 @@ __device__ __forceinline__ void fused6_tile(const Fused6Args &p, int tm, int tn,
     }
   }  // made visible by the first barrier of the pipeline
 
-  v16f acc[C::MI][C::NI];
-#pragma unroll
-  for (int mi = 0; mi < C::MI; ++mi)
-#pragma unroll
-    for (int ni = 0; ni < C::NI; ++ni)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0.0f;
-
   Pipe pipe;
   pipe.init(smem, p.xbuf, lx, m0 / 64, p.wbuf, lw, (p.n_first + n0) / 64);
-  pipe.start();
+  pipe.start();  // its barrier also makes the vectors visible
+
+  v16f acc[C::MI][C::NI];
+#pragma unroll
+  for (int ni = 0; ni < C::NI; ++ni)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const float4 cc = *reinterpret_cast<const float4 *>(tv.colc + wn * C::WN + ni * 32 + acc_col(g, lane));
+#pragma unroll
+      for (int mi = 0; mi < C::MI; ++mi)
+        acc[mi][ni][4 * g] = cc.x, acc[mi][ni][4 * g + 1] = cc.y, acc[mi][ni][4 * g + 2] = cc.z, acc[mi][ni][4 * g + 3] = cc.w;
+    }
   pipe.run_fp6(acc);
 
-  // acc = 64 S  ->  f32(integer accumulator) * (s_row * s_col), in place, one 32x32 block at a time
+  // acc = S - colc / 64  ->  f32(integer accumulator) * (s_row * s_col), in place, one 32x32 block at a time
   float srow[C::MI], rowc[C::MI];
 #pragma unroll
   for (int mi = 0; mi < C::MI; ++mi) {
@@ -442,20 +447,17 @@ __device__ __forceinline__ void fused6_tile(const Fused6Args &p, int tm, int tn,
   asm volatile("s_nop 15\n\ts_nop 15");  // the last MFMA results are architecturally visible to the reads below
 #pragma unroll
   for (int ni = 0; ni < C::NI; ++ni) {
-    float scv[16], ccv[16];
+    float scv[16];
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
       const float4 sc = *reinterpret_cast<const float4 *>(tv.scol + wn * C::WN + ni * 32 + acc_col(g, lane));
-      const float4 cc = *reinterpret_cast<const float4 *>(tv.colc + wn * C::WN + ni * 32 + acc_col(g, lane));
       scv[4 * g] = sc.x, scv[4 * g + 1] = sc.y, scv[4 * g + 2] = sc.z, scv[4 * g + 3] = sc.w;
-      ccv[4 * g] = cc.x, ccv[4 * g + 1] = cc.y, ccv[4 * g + 2] = cc.z, ccv[4 * g + 3] = cc.w;
     }
 #pragma unroll
     for (int mi = 0; mi < C::MI; ++mi) {
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
-        const float s64 = agpr_read(acc[mi][ni][v]) * 64.0f;
-        const float iacc = (s64 - rowc[mi]) - ccv[v];  // exact: integers below 2^24
+        const float iacc = __builtin_fmaf(agpr_read(acc[mi][ni][v]), 64.0f, -rowc[mi]);  // exact: integers below 2^24
         acc[mi][ni][v] = agpr_write(iacc * (srow[mi] * scv[v]));
       }
     }

@@ -125,6 +125,8 @@ class MixedQLinear(torch.nn.Module):
         k_multiple = 128 if self.bits == 4 else 64
         if rows < self.six_bit_min_rows or self.int_features_num % k_multiple != 0 or self.fp_features_num % 32 != 0:
             return False
+        if self.bits == 4 and self.int_features_num > 74496:   # the 6-bit path's fp32 sums are exact up to here
+            return False
         colmap = self._column_map()
         if self._streams is None:  # one device-to-host word and a stream synchronisation, once per column map
             self._streams = asymmetric.colmap_streams(colmap, self.int_features_num, self.fp_features_num)
