@@ -125,7 +125,8 @@ int quik_sym_fused_dequantize(const void *A, const void *B, const void *scale_ro
  * fp32 sum and the per-row / per-column level sums, so the results are those of
  * quik_mixed_linear_fwd bit for bit.  An operand buffer holds a [rows, K] int4 matrix, its [rows, F]
  * fp16/bf16 outlier columns and the per-row level sums, in the order the GEMM tiles read them.
- * Needs K % 128 == 0, F % 32 == 0, M > 32; operand buffers aligned to 256 bytes. */
+ * Needs K % 128 == 0, K <= 74496 (the fp32 sums are exact up to there), F % 32 == 0, M > 32;
+ * operand buffers aligned to 256 bytes. */
 
 /* bytes of an operand buffer for [rows, K] int4 + [rows, F] outliers (0 if the shape is not supported) */
 int64_t quik_fp6_operand_bytes(int64_t rows, int64_t K, int64_t F);
