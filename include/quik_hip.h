@@ -151,6 +151,21 @@ int quik_mixed_linear_fwd_fp6(const void *x6, const void *w6, const void *meta, 
                               const void *w_reduced, const void *bias, int dtype, int64_t M, int64_t N,
                               int64_t K, int64_t F, void *out, void *stream);
 
+/* ---- symmetric activations in one kernel --------------------------------------------------------
+ * MixedQLinear's symmetric branch (experiments/qlinear.py:97-103) computes, with torch ops and
+ * symmetric.quantize: int_x = x[:, int_indices]; fp_x = x[:, fp_indices];
+ * scale = fp16(max|int_x| / divisor); q = rne(fp16(int_x / scale)) kept modulo 2^bits.  This entry
+ * point does the same in the streaming quantize kernel (fp16 only; the column map must select that
+ * kernel: quik_colmap_streaming(...) == 1, otherwise nothing is written).  tiled == 0: dst is
+ * [rows, num_int/2] uint8 (bits = 4) or [rows, num_int] int8 and fp_x [rows, num_fp]; tiled != 0:
+ * dst is an operand buffer of the tile-ordered GEMMs (quik_fp6_operand_bytes for bits = 4,
+ * quik_tile8_operand_bytes for bits = 8; their shape conditions apply) and fp_x is not used.
+ * scale: [rows] fp16.  A row that holds a NaN gets a NaN scale and all-zero codes, as with torch.
+ * The tile-ordered GEMM entry points take the symmetric form when w_reduced == NULL (meta = scale). */
+int quik_sym_quantize_mapped(const void *x, int64_t rows, int64_t cols, const void *colmap, int64_t num_int,
+                             int64_t num_fp, int bits, float divisor, int tiled, void *dst, void *scale,
+                             void *fp_x, void *stream);
+
 /* ---- W8A8 on tile-ordered operands -------------------------------------------------------------
  * No counterpart in the reference: the same forward as quik_asym_quantize (bits = 8) +
  * quik_mixed_linear_fwd (bits = 8, asymmetric), bit for bit, with both int8 operands (and the

@@ -34,6 +34,8 @@ SIGNATURES = {
     "quik_colmap_streaming": (_int, [_vp, _i64, _i64, _i64, _vp]),
     "quik_asym_quantize_fp6": (_int, [_vp, _int, _i64, _i64, _vp, _i64, _i64, _vp, _vp, _vp]),
     "quik_mixed_linear_fwd_fp6": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _i64, _vp, _vp]),
+    "quik_sym_quantize_mapped": (_int, [_vp, _i64, _i64, _vp, _i64, _i64, _int, ctypes.c_float, _int, _vp, _vp, _vp,
+                                        _vp]),
     "quik_tile8_operand_bytes": (_i64, [_i64, _i64, _i64]),
     "quik_tile8_pack_weight": (_int, [_vp, _vp, _i64, _i64, _i64, _vp, _vp]),
     "quik_asym_quantize_tile8": (_int, [_vp, _int, _i64, _i64, _vp, _i64, _i64, _vp, _vp, _vp]),

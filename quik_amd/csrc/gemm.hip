@@ -310,7 +310,7 @@ int run_fused6(const Fused6Args &p, hipStream_t st) {
   tail.N = static_cast<int>(p.N - nw);
   tail.n_first = static_cast<int>(nw);
   tail.s_col = p.s_col + nw;
-  tail.w_red = p.w_red + nw;
+  tail.w_red = p.w_red ? p.w_red + nw : nullptr;
   tail.bias = p.bias ? p.bias + nw : nullptr;
   tail.out = p.out + nw;
   return launch_fused6_split<CfgL, CfgH, BF16>(wide, tail, st);
@@ -355,7 +355,7 @@ int run_fused8t(const Fused8Args &p, hipStream_t st) {
   tail.N = static_cast<int>(p.N - nw);
   tail.n_first = static_cast<int>(nw);
   tail.s_col = p.s_col + nw;
-  tail.w_red = p.w_red + nw;
+  tail.w_red = p.w_red ? p.w_red + nw : nullptr;
   tail.bias = p.bias ? p.bias + nw : nullptr;
   tail.out = p.out + nw;
   return launch_fused8t_split<CfgL, CfgH, BF16>(wide, tail, st);
@@ -448,7 +448,7 @@ extern "C" int quik_mixed_linear_fwd_fp6(const void *x6, const void *w6, const v
   if (M < 0 || N < 0 || K <= 0 || F < 0) return QUIK_ERR_SHAPE;
   if (M == 0 || N == 0) return QUIK_OK;
   if (M <= 32) return QUIK_ERR_SHAPE;
-  if (!x6 || !w6 || !meta || !s_col || !w_reduced || !out) return QUIK_ERR_NULL;
+  if (!x6 || !w6 || !meta || !s_col || !out) return QUIK_ERR_NULL;  // w_reduced == NULL: symmetric activations
   if (K % 128 != 0 || F % 32 != 0) return QUIK_ERR_ALIGN;
   auto misaligned = [](const void *p) { return reinterpret_cast<uintptr_t>(p) % 256 != 0; };
   if (misaligned(x6) || misaligned(w6)) return QUIK_ERR_ALIGN;
@@ -479,7 +479,7 @@ extern "C" int quik_mixed_linear_fwd_tile8(const void *x8, const void *w8, const
   if (M < 0 || N < 0 || K <= 0 || F < 0) return QUIK_ERR_SHAPE;
   if (M == 0 || N == 0) return QUIK_OK;
   if (M <= 32) return QUIK_ERR_SHAPE;
-  if (!x8 || !w8 || !meta || !s_col || !w_reduced || !out) return QUIK_ERR_NULL;
+  if (!x8 || !w8 || !meta || !s_col || !out) return QUIK_ERR_NULL;  // w_reduced == NULL: symmetric activations
   if (K % 64 != 0 || F % 32 != 0) return QUIK_ERR_ALIGN;
   auto misaligned = [](const void *p) { return reinterpret_cast<uintptr_t>(p) % 256 != 0; };
   if (misaligned(x8) || misaligned(w8)) return QUIK_ERR_ALIGN;

@@ -408,15 +408,16 @@ __device__ __forceinline__ void fused6_tile(const Fused6Args &p, int tm, int tn,
     for (int i = threadIdx.x; i < C::BN; i += C::kThreads) {
       const int n = n0 + i < p.N ? n0 + i : p.N - 1;
       tv.scol[i] = to_f32<BF16>(p.s_col[n]);
-      tv.wred[i] = to_f32<BF16>(p.w_red[n]);
+      tv.wred[i] = p.w_red ? to_f32<BF16>(p.w_red[n]) : 0.0f;
       tv.bias[i] = p.bias ? to_f32<BF16>(p.bias[n]) : 0.0f;
       tv.colc[i] = static_cast<float>(ws[p.n_first + n]) * -0.125f;
     }
     for (int i = threadIdx.x; i < C::BM; i += C::kThreads) {
       const int64_t m = m0 + i < p.M ? m0 + i : p.M - 1;
-      const float s = to_f32<BF16>(p.meta[2 * m]);
+      // asymmetric: meta holds (scale, zero) pairs; symmetric (no w_red): one scale per row and no zero term
+      const float s = to_f32<BF16>(p.meta[p.w_red ? 2 * m : m]);
       tv.srow[i] = s;
-      tv.zs[i] = to_f32<BF16>(p.meta[2 * m + 1]) + 8.0f * s;
+      tv.zs[i] = p.w_red ? to_f32<BF16>(p.meta[2 * m + 1]) + 8.0f * s : 0.0f;
       tv.rowc[i] = static_cast<float>(8 * xs[m] - 64 * p.K);
     }
   }  // made visible by the first barrier of the pipeline

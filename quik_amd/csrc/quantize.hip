@@ -199,6 +199,19 @@ struct RowQuant {
     slow = !(range <= max_finite) || !(scale >= 1e-20f);
   }
 
+  // Symmetric activations (reference: experiments/qlinear.py:97-103): scale = fp16(max |x| / divisor), zero = 0.
+  // `absmax_bits` is the largest |x| as an fp16 bit pattern (NaN patterns count as larger than infinity, so a NaN
+  // in the row makes the scale NaN, as torch.max does).
+  __device__ __forceinline__ void init_sym(uint32_t absmax_bits, float divisor) {
+    const float absmax = to_f32<false>(static_cast<uint16_t>(absmax_bits));
+    scale_bits = from_f32<false>(absmax / divisor);
+    zero_bits = 0;
+    scale = to_f32<false>(scale_bits);
+    zero = 0.0f;
+    rcp = 1.0f / scale;
+    slow = !(scale >= 1e-6f) || !(absmax <= 65504.0f);
+  }
+
   // same with the path chosen at compile time (callers branch once per row on `slow`)
   template <bool SLOW>
   __device__ __forceinline__ float quotient_t(uint16_t xbits) const {
@@ -343,6 +356,7 @@ __device__ __forceinline__ void gather_rows(
 // code bytes per lane, packs them to nibbles (int4) and writes 8 or 16 contiguous bytes per lane.
 typedef _Float16 h2 __attribute__((ext_vector_type(2)));
 typedef float f2 __attribute__((ext_vector_type(2)));
+typedef uint16_t u2 __attribute__((ext_vector_type(2)));
 
 struct __attribute__((packed, aligned(1))) Bytes8 {
   uint32_t a, b;
@@ -350,11 +364,36 @@ struct __attribute__((packed, aligned(1))) Bytes8 {
 
 // Codes of the two halves of word w in bytes 0 and 2 of the result (other bytes: don't care).
 // The code is (level - 2^(BITS-1)) mod 256; for BITS == 4 only its low nibble is meaningful.
-template <int BITS, bool BF16, bool SLOW>
+// SYM (fp16 only): symmetric codes, rne(fp16(x / scale)) kept modulo 256 without a clamp (reference:
+// src/symmetric/symmetric.cu:6-61; NaN -> 0, +-infinity saturate as __half2int_rn does before the low bits are cut).
+template <int BITS, bool BF16, bool SLOW, bool SYM = false>
 __device__ __forceinline__ uint32_t code_pair(uint32_t w, const RowQuant<BF16> &rq) {
   constexpr float kMaxQ = static_cast<float>((1 << BITS) - 1);
   constexpr uint32_t kBias = 1u << (BITS - 1);
-  if constexpr (BF16) {
+  if constexpr (SYM) {
+    static_assert(!BF16, "symmetric activations are fp16");
+    const h2 d = __builtin_bit_cast(h2, w);
+    h2 t;
+    if constexpr (SLOW) {
+      const f2 q = f2{static_cast<float>(d.x) / rq.scale, static_cast<float>(d.y) / rq.scale};
+      t = __builtin_convertvector(q, h2);
+    } else {
+      uint32_t tb;
+      asm("v_fma_mixlo_f16 %0, %1, %2, 0 op_sel_hi:[1,0,0]\n\t"
+          "v_fma_mixhi_f16 %0, %1, %2, 0 op_sel:[1,0,0] op_sel_hi:[1,0,0]"
+          : "=&v"(tb)
+          : "v"(w), "v"(rq.rcp));
+      t = __builtin_bit_cast(h2, tb);
+    }
+    // [-512, 511] holds every legitimate quotient (|q| <= divisor) unchanged, maps NaN to -512 and the infinities to
+    // the ends; + 1536 lands in [1024, 2048), where one fp16 ulp is 1: the sum is rne(t) + 1536 and its low byte is
+    // rne(t) mod 256 (0 for NaN and -infinity, 255 for +infinity: the low bits of the saturated integers)
+    const _Float16 lo = static_cast<_Float16>(-512.0f), hi = static_cast<_Float16>(511.0f);
+    t = __builtin_elementwise_min(__builtin_elementwise_max(t, h2{lo, lo}), h2{hi, hi});
+    constexpr _Float16 magic = static_cast<_Float16>(1536);
+    t = t + h2{magic, magic};
+    return __builtin_bit_cast(uint32_t, t);
+  } else if constexpr (BF16) {
     const uint32_t a = RowQuant<true>::to_level(rq.template quotient_t<SLOW>(static_cast<uint16_t>(w & 0xFFFFu)), kMaxQ);
     const uint32_t b = RowQuant<true>::to_level(rq.template quotient_t<SLOW>(static_cast<uint16_t>(w >> 16)), kMaxQ);
     return (a + kBias) | ((b + kBias) << 16);
@@ -387,10 +426,10 @@ __device__ __forceinline__ uint32_t code_pair(uint32_t w, const RowQuant<BF16> &
 }
 
 // 8 codes of one group as 8 bytes
-template <int BITS, bool BF16, bool SLOW>
+template <int BITS, bool BF16, bool SLOW, bool SYM = false>
 __device__ __forceinline__ uint2 group_codes(const uint4 &v, const RowQuant<BF16> &rq) {
-  const uint32_t p0 = code_pair<BITS, BF16, SLOW>(v.x, rq), p1 = code_pair<BITS, BF16, SLOW>(v.y, rq);
-  const uint32_t p2 = code_pair<BITS, BF16, SLOW>(v.z, rq), p3 = code_pair<BITS, BF16, SLOW>(v.w, rq);
+  const uint32_t p0 = code_pair<BITS, BF16, SLOW, SYM>(v.x, rq), p1 = code_pair<BITS, BF16, SLOW, SYM>(v.y, rq);
+  const uint32_t p2 = code_pair<BITS, BF16, SLOW, SYM>(v.z, rq), p3 = code_pair<BITS, BF16, SLOW, SYM>(v.w, rq);
   uint2 c;
   c.x = __builtin_amdgcn_perm(p1, p0, 0x06040200u);  // bytes 0, 2 of p0 then bytes 0, 2 of p1
   c.y = __builtin_amdgcn_perm(p3, p2, 0x06040200u);
@@ -403,14 +442,15 @@ __device__ __forceinline__ uint2 group_codes(const uint4 &v, const RowQuant<BF16
 
 // One row is handled by the TPR threads of one workgroup (a multiple of 64, at most 256; the
 // launches use 256), which walks over rows blockIdx.x, blockIdx.x + gridDim.x, ...
-template <int BITS, bool BF16, int NV, int TPR>
+// SYM: symmetric activations (scale = fp16(max |x| / sym_divisor), one scale per row in meta[row]); fp16 only.
+template <int BITS, bool BF16, int NV, int TPR, bool SYM = false>
 __device__ __forceinline__ void stream_rows(const uint16_t *__restrict__ x, int64_t rows, int64_t cols,
                                             const uint32_t *__restrict__ grp, const uint32_t *__restrict__ dirty,
                                             const uint16_t *__restrict__ dirty_grp, int ndirty,
                                             const uint16_t *__restrict__ fp_col, int64_t num_int, int64_t num_fp,
                                             uint8_t *__restrict__ dst, uint16_t *__restrict__ meta,
                                             uint16_t *__restrict__ fp_x, uint8_t *codes_s, float *red, int vec_out,
-                                            int *rowsum_s) {
+                                            int *rowsum_s, float sym_divisor = 1.0f) {
   // vec_out: 0 byte-wise output, 1 16-byte output, 2 (4 bits only): dst is a 6-bit operand buffer
   // (fp6_format.h) for the matrix-core path of gemm_fp6.h, which also takes the outlier values (fp_x is
   // not written); needs num_int % 128 == 0 and num_fp % 32 == 0
@@ -465,11 +505,22 @@ __device__ __forceinline__ void stream_rows(const uint16_t *__restrict__ x, int6
       }
     }
   };
+  // SYM: largest |x| pattern of one dirty group, outlier halves zeroed
+  auto dirty_absmax = [&](const uint4 &v, uint32_t mb, u2 &amax) {
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const uint32_t lo = static_cast<uint32_t>(__builtin_amdgcn_sbfe(static_cast<int>(mb), 2 * k, 1));
+      const uint32_t hi = static_cast<uint32_t>(__builtin_amdgcn_sbfe(static_cast<int>(mb), 2 * k + 1, 1));
+      const uint32_t outl = __builtin_amdgcn_perm(hi, lo, 0x07060100u);  // 0xFFFF in the outlier halves
+      amax = __builtin_elementwise_max(amax, __builtin_bit_cast(u2, w[k] & 0x7FFF7FFFu & ~outl));
+    }
+  };
   // codes of one dirty group, outliers squeezed out
   auto dirty_codes = [&](const uint4 &v, uint32_t info, const RowQuant<BF16> &rq, auto slow_c) {
     constexpr bool SLOW = decltype(slow_c)::value;
     const uint32_t mb = info & 0xFFu;
-    const uint2 c = group_codes<BITS, BF16, SLOW>(v, rq);
+    const uint2 c = group_codes<BITS, BF16, SLOW, SYM>(v, rq);
     uint8_t *out = codes_s + (info >> 8);
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
@@ -486,7 +537,17 @@ __device__ __forceinline__ void stream_rows(const uint16_t *__restrict__ x, int6
     float mn = inf, mx = -inf;
     const h2 pinf = h2{static_cast<_Float16>(inf), static_cast<_Float16>(inf)};
     h2 pmn = pinf, pmx = -pinf;
-    if constexpr (!BF16) {
+    u2 amax = u2{0, 0};  // SYM: largest |x| bit pattern per half (non-negative fp16 patterns order like unsigned integers)
+    if constexpr (SYM) {
+#pragma unroll
+      for (int i = 0; i < NV; ++i) {
+        const u2 a = __builtin_bit_cast(u2, cur[i].x & 0x7FFF7FFFu), b = __builtin_bit_cast(u2, cur[i].y & 0x7FFF7FFFu);
+        const u2 c = __builtin_bit_cast(u2, cur[i].z & 0x7FFF7FFFu), d = __builtin_bit_cast(u2, cur[i].w & 0x7FFF7FFFu);
+        const u2 hi = __builtin_elementwise_max(__builtin_elementwise_max(a, b), __builtin_elementwise_max(c, d));
+        const bool clean = (g[i] & 0xFFu) == 0u;
+        amax = __builtin_elementwise_max(amax, clean ? hi : u2{0, 0});
+      }
+    } else if constexpr (!BF16) {
 #pragma unroll
       for (int i = 0; i < NV; ++i) {
         const h2 a = __builtin_bit_cast(h2, cur[i].x), b = __builtin_bit_cast(h2, cur[i].y);
@@ -526,14 +587,23 @@ __device__ __forceinline__ void stream_rows(const uint16_t *__restrict__ x, int6
       if (tid + k * TPR < num_fp) *fp_slot(tid + k * TPR) = fpv[k];
     for (int64_t f = tid + ND * TPR; f < num_fp; f += TPR) *fp_slot(f) = x[row * cols + fp_col[f]];
     // ---- lanes 0 .. ndirty-1: one dirty group each (more when there are more than ND * TPR of them)
+    if constexpr (SYM) {
 #pragma unroll
-    for (int k = 0; k < ND; ++k)
-      if (tid + k * TPR < ndirty) dirty_minmax(dv[k], my_dirty[k] & 0xFFu, pmn, pmx, mn, mx);
-    for (int j = tid + ND * TPR; j < ndirty; j += TPR)
-      dirty_minmax(xv[dirty_grp[j]], dirty[j] & 0xFFu, pmn, pmx, mn, mx);
-    if constexpr (!BF16) {
-      mn = fminf(static_cast<float>(pmn.x), static_cast<float>(pmn.y));
-      mx = fmaxf(static_cast<float>(pmx.x), static_cast<float>(pmx.y));
+      for (int k = 0; k < ND; ++k)
+        if (tid + k * TPR < ndirty) dirty_absmax(dv[k], my_dirty[k] & 0xFFu, amax);
+      for (int j = tid + ND * TPR; j < ndirty; j += TPR) dirty_absmax(xv[dirty_grp[j]], dirty[j] & 0xFFu, amax);
+      mn = 0.0f;
+      mx = static_cast<float>(amax.x > amax.y ? amax.x : amax.y);  // a 15-bit integer: exact, ordered like the patterns
+    } else {
+#pragma unroll
+      for (int k = 0; k < ND; ++k)
+        if (tid + k * TPR < ndirty) dirty_minmax(dv[k], my_dirty[k] & 0xFFu, pmn, pmx, mn, mx);
+      for (int j = tid + ND * TPR; j < ndirty; j += TPR)
+        dirty_minmax(xv[dirty_grp[j]], dirty[j] & 0xFFu, pmn, pmx, mn, mx);
+      if constexpr (!BF16) {
+        mn = fminf(static_cast<float>(pmn.x), static_cast<float>(pmn.y));
+        mx = fmaxf(static_cast<float>(pmx.x), static_cast<float>(pmx.y));
+      }
     }
     mn = wave_min(mn);
     mx = wave_max(mx);
@@ -554,17 +624,22 @@ __device__ __forceinline__ void stream_rows(const uint16_t *__restrict__ x, int6
     }
 
     RowQuant<BF16> rq;
-    rq.init(mn, mx, BITS);
-    if (tid == 0) {
-      meta[2 * row] = rq.scale_bits;
-      meta[2 * row + 1] = rq.zero_bits;
+    if constexpr (SYM) {
+      rq.init_sym(static_cast<uint32_t>(mx), sym_divisor);
+      if (tid == 0) meta[row] = rq.scale_bits;
+    } else {
+      rq.init(mn, mx, BITS);
+      if (tid == 0) {
+        meta[2 * row] = rq.scale_bits;
+        meta[2 * row + 1] = rq.zero_bits;
+      }
     }
     // ---- quantise in source order, 8 code bytes per clean group to their destination position
     auto quantise = [&](auto slow_c) {
       constexpr bool SLOW = decltype(slow_c)::value;
 #pragma unroll
       for (int i = 0; i < NV; ++i) {
-        const uint2 c = group_codes<BITS, BF16, SLOW>(cur[i], rq);
+        const uint2 c = group_codes<BITS, BF16, SLOW, SYM>(cur[i], rq);
         if ((g[i] & 0xFFu) == 0u) *reinterpret_cast<Bytes8 *>(codes_s + (g[i] >> 8)) = Bytes8{c.x, c.y};
       }
 #pragma unroll
@@ -677,13 +752,14 @@ __global__ __launch_bounds__(kThreads) void asym_quantize_kernel(
 
 // Shapes that may stream: the column map's flag (known only on the device) picks the path.
 // Dynamic LDS: the row (gather path) or one byte per code (streaming path), whichever is larger.
-template <typename IdxT, int BITS, bool BF16, int NV, int TPR>
+// SYM: symmetric activations; exists on the streaming path only (the host checks the column map's flag first).
+template <typename IdxT, int BITS, bool BF16, int NV, int TPR, bool SYM = false>
 __global__ __launch_bounds__(TPR) void asym_quantize_stream_kernel(
     const uint16_t *__restrict__ x, int64_t rows, int64_t cols, const IdxT *__restrict__ src_col,
     const IdxT *__restrict__ fp_col, const uint32_t *__restrict__ mask, const uint32_t *__restrict__ grp,
     const uint32_t *__restrict__ dirty, const uint16_t *__restrict__ dirty_grp, const uint32_t *__restrict__ flags,
     int64_t num_int, int64_t num_fp, uint8_t *__restrict__ dst, uint16_t *__restrict__ meta,
-    uint16_t *__restrict__ fp_x, int vec_out) {
+    uint16_t *__restrict__ fp_x, int vec_out, float sym_divisor) {
   static_assert(sizeof(IdxT) == 2, "streaming needs cols <= 32768");
   extern __shared__ __align__(16) uint16_t row_s[];
   __shared__ float red[16];
@@ -691,10 +767,10 @@ __global__ __launch_bounds__(TPR) void asym_quantize_stream_kernel(
   if (threadIdx.x == 0) rowsum_s = 0;
   if (flags[0] & 1u) {
     uint8_t *codes_s = reinterpret_cast<uint8_t *>(row_s);
-    stream_rows<BITS, BF16, NV, TPR>(x, rows, cols, grp, dirty, dirty_grp, static_cast<int>(flags[1]),
-                                     reinterpret_cast<const uint16_t *>(fp_col), num_int, num_fp, dst, meta, fp_x,
-                                     codes_s, red, vec_out, &rowsum_s);
-  } else {
+    stream_rows<BITS, BF16, NV, TPR, SYM>(x, rows, cols, grp, dirty, dirty_grp, static_cast<int>(flags[1]),
+                                          reinterpret_cast<const uint16_t *>(fp_col), num_int, num_fp, dst, meta, fp_x,
+                                          codes_s, red, vec_out, &rowsum_s, sym_divisor);
+  } else if constexpr (!SYM) {
     gather_rows<IdxT, BITS, BF16, TPR>(x, rows, cols, src_col, fp_col, mask, num_int, num_fp, dst, meta, fp_x, 1,
                                        row_s, red);
   }
@@ -833,10 +909,11 @@ int grid_for(int64_t work_items, int64_t per_block) {
 
 constexpr int64_t kMaxLdsRowBytes = 128 * 1024;  // of the 160 KB per CU
 
-template <typename IdxT, int BITS, bool BF16, int NV, int TPR>
+template <typename IdxT, int BITS, bool BF16, int NV, int TPR, bool SYM = false>
 int launch_stream(const void *x, int64_t rows, int64_t cols, const uint8_t *cm, const ColmapLayout &l, int64_t num_int,
-                  int64_t num_fp, void *dst, void *meta, void *fp_x, hipStream_t st, bool tiled) {
-  auto kern = asym_quantize_stream_kernel<IdxT, BITS, BF16, NV, TPR>;
+                  int64_t num_fp, void *dst, void *meta, void *fp_x, hipStream_t st, bool tiled,
+                  float sym_divisor = 1.0f) {
+  auto kern = asym_quantize_stream_kernel<IdxT, BITS, BF16, NV, TPR, SYM>;
   const int64_t lds = align16(cols * 2);  // >= align16(num_int)
   if (lds > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -857,8 +934,25 @@ int launch_stream(const void *x, int64_t rows, int64_t cols, const uint8_t *cm, 
                      reinterpret_cast<const uint32_t *>(cm + l.off_dirty),
                      reinterpret_cast<const uint16_t *>(cm + l.off_slot),
                      reinterpret_cast<const uint32_t *>(cm + l.off_flags), num_int, num_fp,
-                     static_cast<uint8_t *>(dst), static_cast<uint16_t *>(meta), static_cast<uint16_t *>(fp_x), vec_out);
+                     static_cast<uint8_t *>(dst), static_cast<uint16_t *>(meta), static_cast<uint16_t *>(fp_x), vec_out,
+                     sym_divisor);
   return check_launch();
+}
+
+// symmetric activations through the streaming kernel (fp16; the caller has checked that the column map streams)
+template <int BITS>
+int launch_sym_stream(const void *x, int64_t rows, int64_t cols, const uint8_t *cm, const ColmapLayout &l,
+                      int64_t num_int, int64_t num_fp, void *dst, void *scale, void *fp_x, hipStream_t st, bool tiled,
+                      float divisor) {
+  const int64_t groups = cols / 8;
+#define QUIK_SYM_STREAM(NV)                                                                                       \
+  return launch_stream<uint16_t, BITS, false, NV, kThreads, true>(x, rows, cols, cm, l, num_int, num_fp, dst, scale, \
+                                                                  fp_x, st, tiled, divisor)
+  if (groups <= 512) QUIK_SYM_STREAM(2);
+  if (groups <= 1024) QUIK_SYM_STREAM(4);
+  if (groups <= 2048) QUIK_SYM_STREAM(8);
+  QUIK_SYM_STREAM(16);
+#undef QUIK_SYM_STREAM
 }
 
 template <typename IdxT, int BITS, bool BF16>
@@ -1015,6 +1109,25 @@ extern "C" int quik_asym_quantize_tile8(const void *x, int dtype, int64_t rows, 
   return dtype == QUIK_F16
              ? launch_asym<uint16_t, 8, false>(x, rows, cols, cm, l, num_int, num_fp, out8, meta, nullptr, st, true)
              : launch_asym<uint16_t, 8, true>(x, rows, cols, cm, l, num_int, num_fp, out8, meta, nullptr, st, true);
+}
+
+extern "C" int quik_sym_quantize_mapped(const void *x, int64_t rows, int64_t cols, const void *colmap, int64_t num_int,
+                                        int64_t num_fp, int bits, float divisor, int tiled, void *dst, void *scale,
+                                        void *fp_x, void *stream) {
+  if (bits != 4 && bits != 8) return QUIK_ERR_BITS;
+  if (rows < 0 || cols <= 0 || num_int <= 0 || num_fp < 0 || num_int + num_fp != cols) return QUIK_ERR_SHAPE;
+  if (cols % 8 != 0 || cols > kStreamMaxCols || !(divisor > 0.0f)) return QUIK_ERR_SHAPE;
+  if (tiled && (num_int % (bits == 4 ? 128 : 64) != 0 || num_fp % 32 != 0)) return QUIK_ERR_ALIGN;
+  if (bits == 4 && num_int % 2 != 0) return QUIK_ERR_ALIGN;
+  if (rows == 0) return QUIK_OK;
+  if (!x || !colmap || !dst || !scale || (!tiled && num_fp > 0 && !fp_x)) return QUIK_ERR_NULL;
+  if (reinterpret_cast<uintptr_t>(x) % 16 != 0 || reinterpret_cast<uintptr_t>(dst) % (tiled ? 256 : 1) != 0)
+    return QUIK_ERR_ALIGN;
+  const ColmapLayout l = colmap_layout(cols, num_int, num_fp);
+  const uint8_t *cm = static_cast<const uint8_t *>(colmap);
+  hipStream_t st = as_stream(stream);
+  return bits == 4 ? launch_sym_stream<4>(x, rows, cols, cm, l, num_int, num_fp, dst, scale, fp_x, st, tiled != 0, divisor)
+                   : launch_sym_stream<8>(x, rows, cols, cm, l, num_int, num_fp, dst, scale, fp_x, st, tiled != 0, divisor);
 }
 
 extern "C" int quik_asym_find_meta(const void *x, int64_t rows, int64_t cols, int bits, void *meta, void *stream) {

@@ -110,7 +110,10 @@ def pack_weight_fp6(int_weight: torch.Tensor, fp_weight: torch.Tensor) -> torch.
 def mixed_linear_fp6(x6, w6, meta, weights_scales, reduced_w, bias, M, N, K, F, out_dtype):
     """mixed_linear (asymmetric, 4 bits) on operand buffers (asymmetric.quantize_mapped_fp6, pack_weight_fp6):
     the int4 products run on the E2M3 matrix-core path at twice the int8 rate; same result bit for bit."""
-    tensors = dict(x6=x6, w6=w6, meta=meta, weights_scales=weights_scales, reduced_w=reduced_w)
+    tensors = dict(x6=x6, w6=w6, meta=meta, weights_scales=weights_scales)
+    symmetric = reduced_w is None      # meta then holds one scale per row and there is no zero-point term
+    if not symmetric:
+        tensors["reduced_w"] = reduced_w
     if bias is not None and bias.numel() > 0:
         tensors["bias"] = bias
     L.check_cuda_contiguous("mixed_linear_fp6", **tensors)
@@ -123,12 +126,13 @@ def mixed_linear_fp6(x6, w6, meta, weights_scales, reduced_w, bias, M, N, K, F, 
     lib = L.load()
     if x6.numel() != lib.quik_fp6_operand_bytes(M, K, F) or w6.numel() != lib.quik_fp6_operand_bytes(N, K, F):
         raise RuntimeError("mixed_linear_fp6: operand buffers do not match M, N, K, F")
-    if meta.numel() != 2 * M or weights_scales.numel() != N or reduced_w.numel() != N:
+    if meta.numel() != (M if symmetric else 2 * M) or weights_scales.numel() != N or \
+            (not symmetric and reduced_w.numel() != N):
         raise RuntimeError("mixed_linear_fp6: meta / weights_scales / reduced_w sizes are inconsistent with M, N")
     with torch.cuda.device(x6.device):
         out = torch.empty((M, N), dtype=out_dtype, device=x6.device)
         L.check(lib.quik_mixed_linear_fwd_fp6(L.ptr(x6), L.ptr(w6), L.ptr(meta), L.ptr(weights_scales),
-                                              L.ptr(reduced_w), L.ptr(tensors.get("bias")), dt, M, N, K, F,
+                                              L.ptr(tensors.get("reduced_w")), L.ptr(tensors.get("bias")), dt, M, N, K, F,
                                               L.ptr(out), L.stream()), "mixed_linear_fp6")
     return out
 
@@ -157,7 +161,10 @@ def pack_weight_tile8(int_weight: torch.Tensor, fp_weight: torch.Tensor) -> torc
 def mixed_linear_tile8(x8, w8, meta, weights_scales, reduced_w, bias, M, N, K, F, out_dtype):
     """mixed_linear (asymmetric, 8 bits) on tile-ordered operand buffers (asymmetric.quantize_mapped_tile8,
     pack_weight_tile8): same result bit for bit, every operand cache line fetched once per tile."""
-    tensors = dict(x8=x8, w8=w8, meta=meta, weights_scales=weights_scales, reduced_w=reduced_w)
+    tensors = dict(x8=x8, w8=w8, meta=meta, weights_scales=weights_scales)
+    symmetric = reduced_w is None      # meta then holds one scale per row and there is no zero-point term
+    if not symmetric:
+        tensors["reduced_w"] = reduced_w
     if bias is not None and bias.numel() > 0:
         tensors["bias"] = bias
     L.check_cuda_contiguous("mixed_linear_tile8", **tensors)
@@ -170,11 +177,12 @@ def mixed_linear_tile8(x8, w8, meta, weights_scales, reduced_w, bias, M, N, K, F
     lib = L.load()
     if x8.numel() != lib.quik_tile8_operand_bytes(M, K, F) or w8.numel() != lib.quik_tile8_operand_bytes(N, K, F):
         raise RuntimeError("mixed_linear_tile8: operand buffers do not match M, N, K, F")
-    if meta.numel() != 2 * M or weights_scales.numel() != N or reduced_w.numel() != N:
+    if meta.numel() != (M if symmetric else 2 * M) or weights_scales.numel() != N or \
+            (not symmetric and reduced_w.numel() != N):
         raise RuntimeError("mixed_linear_tile8: meta / weights_scales / reduced_w sizes are inconsistent with M, N")
     with torch.cuda.device(x8.device):
         out = torch.empty((M, N), dtype=out_dtype, device=x8.device)
         L.check(lib.quik_mixed_linear_fwd_tile8(L.ptr(x8), L.ptr(w8), L.ptr(meta), L.ptr(weights_scales),
-                                                L.ptr(reduced_w), L.ptr(tensors.get("bias")), dt, M, N, K, F,
+                                                L.ptr(tensors.get("reduced_w")), L.ptr(tensors.get("bias")), dt, M, N, K, F,
                                                 L.ptr(out), L.stream()), "mixed_linear_tile8")
     return out

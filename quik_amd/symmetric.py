@@ -11,7 +11,7 @@ import torch
 
 from . import _lib as L
 
-__all__ = ["quantize", "dequantize", "int4FusedDequantize", "int8FusedDequantize"]
+__all__ = ["quantize", "dequantize", "int4FusedDequantize", "int8FusedDequantize", "quantize_mapped"]
 
 
 def quantize(src: torch.Tensor, scale: torch.Tensor, bits: int = 4) -> torch.Tensor:
@@ -95,3 +95,36 @@ def int4FusedDequantize(A, B, scale_row, scale_col, y):
 def int8FusedDequantize(A, B, scale_row, scale_col, y):
     """int8 operands [M, K] / [N, K]; otherwise as int4FusedDequantize (src/symmetric/symmetric.cpp:59-72)."""
     return _fused_dequantize("int8FusedDequantize", 8, A, B, scale_row, scale_col, y)
+
+
+def quantize_mapped(src: torch.Tensor, colmap: torch.Tensor, num_int: int, num_fp: int, bits: int, divisor: float,
+                    tiled: bool):
+    """MixedQLinear's symmetric activation branch (experiments/qlinear.py:97-103) in one kernel: outlier gather,
+    scale = fp16(max|x[:, int]| / divisor) and rne(fp16(x / scale)) codes.  fp16 only; the column map must select
+    the streaming kernel (asymmetric.colmap_streams).  Returns (q, scale [rows, 1], fp_x) with q / fp_x as
+    symmetric.quantize would give them, or, with tiled=True, (operand buffer, scale, None) for
+    matmul.mixed_linear_fp6 (bits=4) / matmul.mixed_linear_tile8 (bits=8)."""
+    L.check_cuda_contiguous("quantize", src=src)
+    if bits not in (4, 8):
+        raise RuntimeError("Unsupported data type")
+    L.dtype_id(src, "quantize", allow_bf16=False)
+    rows, cols = src.shape
+    lib = L.load()
+    with torch.cuda.device(src.device):
+        if tiled:
+            nbytes = (lib.quik_fp6_operand_bytes if bits == 4 else lib.quik_tile8_operand_bytes)(max(rows, 1), num_int,
+                                                                                                  num_fp)
+            if nbytes == 0:
+                raise RuntimeError("quantize: shape not supported by the tile-ordered operand format")
+            dst = torch.empty((nbytes,), dtype=torch.uint8, device=src.device)
+            fp_x = None
+        else:
+            dst = torch.empty((rows, num_int // 2) if bits == 4 else (rows, num_int),
+                              dtype=torch.uint8 if bits == 4 else torch.int8, device=src.device)
+            fp_x = torch.empty((rows, num_fp), dtype=src.dtype, device=src.device)
+        scale = torch.empty((rows, 1), dtype=torch.float16, device=src.device)
+        L.check(lib.quik_sym_quantize_mapped(L.ptr(src), rows, cols, L.ptr(colmap), num_int, num_fp, bits,
+                                             float(divisor), 1 if tiled else 0, L.ptr(dst), L.ptr(scale),
+                                             L.ptr(fp_x) if fp_x is not None and num_fp else None, L.stream()),
+                "quantize")
+    return dst, scale, fp_x
