@@ -120,17 +120,16 @@ class MixedQLinear(torch.nn.Module):
     # -- 6-bit matrix-core path: eligibility and the cached weight operand
     def _six_bit_ok(self, rows):
         """True if this call takes the tile-ordered path (6-bit matrix-core GEMM for 4 bits, int8 for 8 bits)."""
-        if not (self.six_bit_path and self.fused and not self.symmetric and self.bits in (4, 8)):
+        if not (self.six_bit_path and self.fused and self.bits in (4, 8)):
+            return False
+        if self.symmetric and self.dtype != torch.float16:      # symmetric activations are fp16 (as in the reference)
             return False
         k_multiple = 128 if self.bits == 4 else 64
         if rows < self.six_bit_min_rows or self.int_features_num % k_multiple != 0 or self.fp_features_num % 32 != 0:
             return False
         if self.bits == 4 and self.int_features_num > 74496:   # the 6-bit path's fp32 sums are exact up to here
             return False
-        colmap = self._column_map()
-        if self._streams is None:  # one device-to-host word and a stream synchronisation, once per column map
-            self._streams = asymmetric.colmap_streams(colmap, self.int_features_num, self.fp_features_num)
-        return self._streams
+        return self._streams_flag()
 
     def _weight6(self):
         fp_w = self.fp_weight if self.fp_features_num > 0 else \
@@ -143,8 +142,21 @@ class MixedQLinear(torch.nn.Module):
             self._w6_key = key
         return self._w6
 
+    def _streams_flag(self):
+        """True if the column map selects the streaming quantize kernel (cached; one synchronisation per map)."""
+        colmap = self._column_map()
+        if self._streams is None:
+            self._streams = asymmetric.colmap_streams(colmap, self.int_features_num, self.fp_features_num)
+        return self._streams
+
     def _quantize_input(self, x, shared_input):
-        if self.symmetric:
+        if self.symmetric and x.dtype == torch.float16 and x.data_ptr() % 16 == 0 and self._streams_flag():
+            # the op sequence of the next branch in one kernel, same bits
+            shared_input.qint_x, shared_input.qscale_x, shared_input.fp_x = symmetric.quantize_mapped(
+                x, self._column_map(), self.int_features_num, self.fp_features_num, self.bits, self.sym_divisor, False)
+            if self.fp_features_num == 0:
+                shared_input.fp_x = None
+        elif self.symmetric:
             if self.fp_features_num > 0:
                 int_x = x[:, self.int_indices].contiguous()
                 shared_input.fp_x = x[:, self.fp_indices].contiguous()
@@ -169,15 +181,23 @@ class MixedQLinear(torch.nn.Module):
             x2 = x2.contiguous()
         shared_input = self.shared_input if self.shared_input is not None else SharedQuantizedInput(1)
         with torch.cuda.device(x.device):
-            if x2.data_ptr() % 16 == 0 and self._six_bit_ok(x2.shape[0]):
+            if x2.data_ptr() % 16 == 0 and (not self.symmetric or x2.dtype == torch.float16) \
+                    and self._six_bit_ok(x2.shape[0]):
                 quantize6 = asymmetric.quantize_mapped_fp6 if self.bits == 4 else asymmetric.quantize_mapped_tile8
                 linear6 = matmul.mixed_linear_fp6 if self.bits == 4 else matmul.mixed_linear_tile8
                 if shared_input.x6 is None:
-                    shared_input.x6, shared_input.meta = quantize6(
-                        x2, self._column_map(), self.int_features_num, self.fp_features_num)
-                output = linear6(shared_input.x6, self._weight6(), shared_input.meta,
-                                 self.weights_scales, self.reduced_w, self.bias, x2.shape[0],
-                                 self.out_features, self.int_features_num, self.fp_features_num, self.dtype)
+                    if self.symmetric:
+                        shared_input.x6, shared_input.qscale_x, _ = symmetric.quantize_mapped(
+                            x2, self._column_map(), self.int_features_num, self.fp_features_num, self.bits,
+                            self.sym_divisor, True)
+                    else:
+                        shared_input.x6, shared_input.meta = quantize6(
+                            x2, self._column_map(), self.int_features_num, self.fp_features_num)
+                output = linear6(shared_input.x6, self._weight6(),
+                                 shared_input.qscale_x if self.symmetric else shared_input.meta,
+                                 self.weights_scales, None if self.symmetric else self.reduced_w, self.bias,
+                                 x2.shape[0], self.out_features, self.int_features_num, self.fp_features_num,
+                                 self.dtype)
                 shared_input.finish()
                 return output.reshape(*lead, self.out_features)
             if shared_input.qint_x is None:

@@ -1038,6 +1038,82 @@ def test_six_bit_path_is_bit_identical_to_the_int8_path(case, bf16, bits):
         assert np.abs(got[fin].astype(np.float64) - want[fin]).max() <= 1e-2 * rms
 
 
+SYM_QUANT_CASES = [(40, 160, 32), (300, 1088, 64), (77, 512, 0), (1000, 4096, 256), (64, 8192 + 1024, 1024)]
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("case", SYM_QUANT_CASES)
+def test_sym_quantize_mapped_is_the_op_sequence_in_one_kernel(case, bits):
+    """symmetric.quantize_mapped against the module's op sequence (experiments/qlinear.py:97-103: gather, max|x| /
+    divisor in fp16, symmetric.quantize) and against the oracle's symmetric quantizer on the scale it produced:
+    scale, codes and outlier values bit-equal, zero / subnormal / overflowing / Inf / NaN rows included."""
+    import quik
+    from quik_amd import asymmetric, symmetric
+    M, n_in, F = case
+    K = n_in - F
+    rng = np.random.default_rng(M + n_in + F + bits)
+    ii, fi = _split(rng, n_in, F)
+    x = _edge_rows(_acts(rng, M, n_in, fi).astype(np.float16), ii)
+    x[8, :] = 6e-8                                   # scale underflows to zero
+    x[9, :] = -3.0
+    xt, iit, fit = _t(x), _t(ii), _t(fi)
+    divisor = 1 << ((bits - 1) - 1)
+    colmap = asymmetric.build_colmap(iit, fit, n_in)
+    assert asymmetric.colmap_streams(colmap, K, F)
+    int_x = xt[:, iit].contiguous()
+    scale = (torch.max(torch.abs(int_x), dim=1)[0].unsqueeze(1) / divisor).to(torch.float16)
+    q = quik.symmetric.quantize(int_x, scale, bits)
+    q2, scale2, fp2 = symmetric.quantize_mapped(xt, colmap, K, F, bits, divisor, False)
+    nan_rows = torch.isnan(scale.float()).flatten().cpu().numpy()
+    assert np.array_equal(_bits(scale)[~nan_rows], _bits(scale2)[~nan_rows])
+    assert torch.isnan(scale2.float()).flatten().cpu().numpy()[nan_rows].all()
+    assert np.array_equal(q.cpu().numpy(), q2.cpu().numpy())
+    assert np.array_equal(_bits(fp2), x[:, fi].view(np.uint16))
+    want = qo.sym_quantize(x[:, ii], scale2.cpu().numpy(), bits)
+    assert np.array_equal(q2.cpu().numpy(), want)
+
+
+SYM_SIX_CASES = [
+    # M, N, in, F, bias
+    (33, 200, 544, 32, True),
+    (300, 520, 1088, 64, False),
+    (512, 1024, 1024, 0, True),
+    (1000, 4160, 4096, 256, True),
+    (2048, 8192, 1024 + 128, 128, False),
+]
+
+
+@pytest.mark.parametrize("case", SYM_SIX_CASES)
+def test_symmetric_module_on_tile_ordered_operands(case):
+    """A symmetric MixedQLinear (4 bits, the only width from_float accepts) on the tile-ordered path (one quantize
+    kernel into the 6-bit operand buffer, E2M3 matrix-core GEMM with the symmetric epilogue) against the same
+    layer on the row-major kernels: identical output bits; and against the oracle within the fp16 tolerance."""
+    M, N, n_in, F, with_bias = case
+    bits = 4
+    rng = np.random.default_rng(sum(case[:4]) + 5)
+    W, s_w, ii, fi = _layer(rng, N, n_in, F, bits)
+    bias = rng.standard_normal(N).astype(np.float16) if with_bias else None
+    x = _edge_rows(_acts(rng, M, n_in, fi).astype(np.float16), ii)
+    mods = []
+    for six in (True, False):
+        mod = _module(W, s_w, fi, bits, bias, symm=True)
+        mod.six_bit_path = six
+        mods.append(mod)
+    out6, out8 = mods[0](_t(x)), mods[1](_t(x))
+    assert mods[0]._w6 is not None and mods[1]._w6 is None
+    assert out6.shape == out8.shape == (1, M, N)
+    got6, got8 = _bits(out6).reshape(M, N), _bits(out8).reshape(M, N)
+    nan_rows = np.isnan(x[:, ii].astype(np.float32)).any(1)
+    assert np.array_equal(got6[~nan_rows], got8[~nan_rows])
+    assert torch.isnan(out6[0].float()).cpu().numpy()[nan_rows].all()
+    rows = np.r_[8:32, M - 1:M]                       # finite rows
+    omod = qo.from_float(W, s_w, fi, bits, symm=True)
+    want, _ = qo.mixed_qlinear_forward(x[rows], omod, bits, bias, symm=True)
+    got = out6[0].float().cpu().numpy()[rows]
+    rms = np.sqrt((want.astype(np.float64) ** 2).mean())
+    assert np.abs(got.astype(np.float64) - want).max() <= 1e-2 * rms
+
+
 def test_six_bit_path_shared_input_and_fallbacks():
     """A q/k/v-style group on the 6-bit path quantizes once into the operand format; a member with the path
     switched off, or a call with fewer rows than the threshold, takes the int4 path, with the same results."""
