@@ -76,11 +76,32 @@ def check(status: int, op: str):
 
 
 def ptr(t):
-    return None if t is None else ctypes.c_void_p(t.data_ptr())
+    """Device address of a tensor as ctypes takes it for a void* argument (None -> NULL)."""
+    return None if t is None else t.data_ptr()
 
 
 def stream():
-    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    """torch's current stream on the current device, as a raw hipStream_t value."""
+    return torch._C._cuda_getCurrentRawStream(torch._C._cuda_getDevice())
+
+
+class _NoGuard:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_GUARD = _NoGuard()
+
+
+def device_guard(device: torch.device):
+    """`with device_guard(t.device):` makes the tensor's GPU current for the launch, as the reference's CUDAGuard
+    does (asymmetric.cu:179,322,495); free when it already is (the usual case: this sits on every forward)."""
+    if device.index is None or device.index == torch._C._cuda_getDevice():
+        return _NO_GUARD
+    return torch.cuda.device(device)
 
 
 def dtype_id(t: torch.Tensor, op: str, allow_bf16: bool) -> int:

@@ -31,7 +31,7 @@ def build_colmap(int_indices: torch.Tensor, fp_indices: torch.Tensor, cols: int)
     if num_fp + num_int != cols:
         raise RuntimeError("Quantize: number of fp and int columns is not equal to total number of columns")
     nbytes = lib.quik_colmap_bytes(cols, num_int, num_fp)
-    with torch.cuda.device(int_indices.device):
+    with L.device_guard(int_indices.device):
         cm = torch.empty(nbytes, dtype=torch.uint8, device=int_indices.device)
         L.check(lib.quik_colmap_build(L.ptr(int_indices), num_int, L.ptr(fp_indices) if num_fp else None, num_fp,
                                       cols, L.ptr(cm), L.stream()), "quantize")
@@ -51,7 +51,7 @@ def quantize_mapped(src: torch.Tensor, colmap: torch.Tensor, num_int: int, num_f
     if num_int % 2 != 0:
         raise RuntimeError("Quantize: number of int columns has to be even (implementation detail)")
     lib = L.load()
-    with torch.cuda.device(src.device):
+    with L.device_guard(src.device):
         if bits == 4:
             dst = torch.empty((rows, num_int // 2), dtype=torch.uint8, device=src.device)
         else:
@@ -67,7 +67,7 @@ def colmap_streams(colmap: torch.Tensor, num_int: int, num_fp: int) -> bool:
     """True if the column map selects the streaming kernel (ascending int_indices that partition the
     columns with fp_indices, cols % 8 == 0, cols <= 32768).  Synchronises once: call per layer, not per step."""
     lib = L.load()
-    with torch.cuda.device(colmap.device):
+    with L.device_guard(colmap.device):
         rc = lib.quik_colmap_streaming(L.ptr(colmap), num_int + num_fp, num_int, num_fp, L.stream())
     if rc < 0:
         L.check(rc, "colmap_streams")
@@ -85,7 +85,7 @@ def quantize_mapped_fp6(src: torch.Tensor, colmap: torch.Tensor, num_int: int, n
     if nbytes == 0:
         raise RuntimeError("quantize: the 6-bit operand format needs a multiple of 128 integer columns and a "
                            "multiple of 32 outlier columns")
-    with torch.cuda.device(src.device):
+    with L.device_guard(src.device):
         x6 = torch.empty((nbytes,), dtype=torch.uint8, device=src.device)
         meta = torch.empty((2 * rows,), dtype=src.dtype, device=src.device)
         L.check(lib.quik_asym_quantize_fp6(L.ptr(src), dt, rows, cols, L.ptr(colmap), num_int, num_fp, L.ptr(x6),
@@ -104,7 +104,7 @@ def quantize_mapped_tile8(src: torch.Tensor, colmap: torch.Tensor, num_int: int,
     if nbytes == 0:
         raise RuntimeError("quantize: the tile-ordered int8 format needs a multiple of 64 integer columns and a "
                            "multiple of 32 outlier columns")
-    with torch.cuda.device(src.device):
+    with L.device_guard(src.device):
         x8 = torch.empty((nbytes,), dtype=torch.uint8, device=src.device)
         meta = torch.empty((2 * rows,), dtype=src.dtype, device=src.device)
         L.check(lib.quik_asym_quantize_tile8(L.ptr(src), dt, rows, cols, L.ptr(colmap), num_int, num_fp, L.ptr(x8),
@@ -153,7 +153,7 @@ def dequantize(x: torch.Tensor, meta: torch.Tensor, scale_col: torch.Tensor, wRe
         if t.dtype != y.dtype:
             raise RuntimeError(f"dequantize: expected {name} to have dtype {y.dtype} but got {t.dtype}")
     lib = L.load()
-    with torch.cuda.device(x.device):
+    with L.device_guard(x.device):
         out = torch.empty_like(y)
         L.check(lib.quik_asym_dequantize(L.ptr(x), L.ptr(meta), L.ptr(scale_col), L.ptr(wReduced.contiguous()),
                                          L.ptr(y), dt, rows, cols, bits, L.ptr(out), L.stream()), "dequantize")
@@ -167,7 +167,7 @@ def find_meta(src: torch.Tensor, bits: int) -> torch.Tensor:
     L.dtype_id(src, "find_meta", allow_bf16=False)
     rows, cols = src.shape
     lib = L.load()
-    with torch.cuda.device(src.device):
+    with L.device_guard(src.device):
         meta = torch.empty((2 * rows,), dtype=torch.float16, device=src.device)
         L.check(lib.quik_asym_find_meta(L.ptr(src), rows, cols, bits, L.ptr(meta), L.stream()), "find_meta")
     return meta
@@ -183,7 +183,7 @@ def quantizeOld(src: torch.Tensor, meta: torch.Tensor, bits: int) -> torch.Tenso
     if meta.size(0) != 2 * rows:
         raise RuntimeError(f"quantize: expected meta to have size {2 * rows} at dimension 0, got {meta.size(0)}")
     lib = L.load()
-    with torch.cuda.device(src.device):
+    with L.device_guard(src.device):
         if bits == 4:
             dst = torch.empty((rows, (cols + 1) // 2), dtype=torch.uint8, device=src.device)
         else:
@@ -212,7 +212,7 @@ def _fused_dequantize(op, bits, A, B, scale_row, scale_col, shift_value, zero_ro
         if t.numel() != n:
             raise RuntimeError(f"{op}: expected {name} to have {n} elements but got {t.numel()}")
     lib = L.load()
-    with torch.cuda.device(A.device):
+    with L.device_guard(A.device):
         acc = torch.empty((M, N), dtype=torch.int32, device=A.device)
         out = torch.empty((M, N), dtype=torch.float16, device=A.device)
         L.check(lib.quik_asym_fused_dequantize(L.ptr(A), L.ptr(B), L.ptr(scale_row), L.ptr(scale_col),

@@ -24,7 +24,7 @@ def _matmul(op, A, B, want_dtype, sym, kmul):
         raise RuntimeError(f"{op}: A [M, K] and B [N, K] must agree in K, got {tuple(A.shape)} and {tuple(B.shape)}")
     M, N, K = A.size(0), B.size(0), A.size(1) * kmul
     lib = L.load()
-    with torch.cuda.device(A.device):
+    with L.device_guard(A.device):
         C = torch.empty((M, N), dtype=torch.int32, device=A.device)
         L.check(getattr(lib, sym)(L.ptr(A), L.ptr(B), L.ptr(C), M, N, K, L.stream()), op)
     return C
@@ -77,7 +77,7 @@ def mixed_linear(qx, int_weight, meta, weights_scales, reduced_w, fp_x, fp_weigh
     if "bias" in tensors and bias.numel() != N:
         raise RuntimeError("mixed_linear: bias must have N elements")
     lib = L.load()
-    with torch.cuda.device(qx.device):
+    with L.device_guard(qx.device):
         out = torch.empty((M, N), dtype=out_dtype, device=qx.device)
         L.check(lib.quik_mixed_linear_fwd(L.ptr(qx), L.ptr(int_weight), L.ptr(meta), L.ptr(weights_scales),
                                           L.ptr(reduced_w), L.ptr(fp_x) if F else None,
@@ -100,7 +100,7 @@ def pack_weight_fp6(int_weight: torch.Tensor, fp_weight: torch.Tensor) -> torch.
     nbytes = lib.quik_fp6_operand_bytes(N, K, F)
     if nbytes == 0:
         raise RuntimeError("pack_weight_fp6: K must be a multiple of 128 and F a multiple of 32")
-    with torch.cuda.device(int_weight.device):
+    with L.device_guard(int_weight.device):
         out = torch.empty((nbytes,), dtype=torch.uint8, device=int_weight.device)
         L.check(lib.quik_fp6_pack_weight(L.ptr(int_weight), L.ptr(fp_weight) if F else None, N, K, F, L.ptr(out),
                                          L.stream()), "pack_weight_fp6")
@@ -129,7 +129,7 @@ def mixed_linear_fp6(x6, w6, meta, weights_scales, reduced_w, bias, M, N, K, F, 
     if meta.numel() != (M if symmetric else 2 * M) or weights_scales.numel() != N or \
             (not symmetric and reduced_w.numel() != N):
         raise RuntimeError("mixed_linear_fp6: meta / weights_scales / reduced_w sizes are inconsistent with M, N")
-    with torch.cuda.device(x6.device):
+    with L.device_guard(x6.device):
         out = torch.empty((M, N), dtype=out_dtype, device=x6.device)
         L.check(lib.quik_mixed_linear_fwd_fp6(L.ptr(x6), L.ptr(w6), L.ptr(meta), L.ptr(weights_scales),
                                               L.ptr(tensors.get("reduced_w")), L.ptr(tensors.get("bias")), dt, M, N, K, F,
@@ -151,7 +151,7 @@ def pack_weight_tile8(int_weight: torch.Tensor, fp_weight: torch.Tensor) -> torc
     nbytes = lib.quik_tile8_operand_bytes(N, K, F)
     if nbytes == 0:
         raise RuntimeError("pack_weight_tile8: K must be a multiple of 64 and F a multiple of 32")
-    with torch.cuda.device(int_weight.device):
+    with L.device_guard(int_weight.device):
         out = torch.empty((nbytes,), dtype=torch.uint8, device=int_weight.device)
         L.check(lib.quik_tile8_pack_weight(L.ptr(int_weight), L.ptr(fp_weight) if F else None, N, K, F, L.ptr(out),
                                            L.stream()), "pack_weight_tile8")
@@ -180,7 +180,7 @@ def mixed_linear_tile8(x8, w8, meta, weights_scales, reduced_w, bias, M, N, K, F
     if meta.numel() != (M if symmetric else 2 * M) or weights_scales.numel() != N or \
             (not symmetric and reduced_w.numel() != N):
         raise RuntimeError("mixed_linear_tile8: meta / weights_scales / reduced_w sizes are inconsistent with M, N")
-    with torch.cuda.device(x8.device):
+    with L.device_guard(x8.device):
         out = torch.empty((M, N), dtype=out_dtype, device=x8.device)
         L.check(lib.quik_mixed_linear_fwd_tile8(L.ptr(x8), L.ptr(w8), L.ptr(meta), L.ptr(weights_scales),
                                                 L.ptr(tensors.get("reduced_w")), L.ptr(tensors.get("bias")), dt, M, N, K, F,

@@ -21,6 +21,7 @@ import torch
 from torch import Tensor
 
 from . import asymmetric, matmul, symmetric
+from ._lib import device_guard
 
 __all__ = ["MixedQLinear", "SharedQuantizedInput", "FusedMixedQLinearGroup", "Linear4bit", "Linear8bit", "pack_to_i4",
            "two_compl"]
@@ -180,7 +181,7 @@ class MixedQLinear(torch.nn.Module):
         if not x2.is_contiguous():
             x2 = x2.contiguous()
         shared_input = self.shared_input if self.shared_input is not None else SharedQuantizedInput(1)
-        with torch.cuda.device(x.device):
+        with device_guard(x.device):
             if x2.data_ptr() % 16 == 0 and (not self.symmetric or x2.dtype == torch.float16) \
                     and self._six_bit_ok(x2.shape[0]):
                 quantize6 = asymmetric.quantize_mapped_fp6 if self.bits == 4 else asymmetric.quantize_mapped_tile8

@@ -26,7 +26,7 @@ def quantize(src: torch.Tensor, scale: torch.Tensor, bits: int = 4) -> torch.Ten
     if scale.size(0) != rows:
         raise RuntimeError(f"quantize: expected scale to have size {rows} at dimension 0, got {scale.size(0)}")
     lib = L.load()
-    with torch.cuda.device(src.device):
+    with L.device_guard(src.device):
         if bits == 4:
             dst = torch.empty((rows, (cols + 1) // 2), dtype=torch.uint8, device=src.device)
         else:
@@ -58,7 +58,7 @@ def dequantize(x: torch.Tensor, scale_row: torch.Tensor, scale_col: torch.Tensor
     for name, t in (("scale_row", scale_row), ("scale_col", scale_col), ("y", y)):
         L.dtype_id(t, "dequantize", allow_bf16=False)
     lib = L.load()
-    with torch.cuda.device(x.device):
+    with L.device_guard(x.device):
         out = torch.empty_like(y)
         L.check(lib.quik_sym_dequantize(L.ptr(x), bits, L.ptr(scale_row), L.ptr(scale_col), L.ptr(y), rows, cols,
                                         L.ptr(out), L.stream()), "dequantize")
@@ -78,7 +78,7 @@ def _fused_dequantize(op, bits, A, B, scale_row, scale_col, y):
         if t.numel() != n:
             raise RuntimeError(f"{op}: expected {name} to have {n} elements but got {t.numel()}")
     lib = L.load()
-    with torch.cuda.device(A.device):
+    with L.device_guard(A.device):
         acc = torch.empty((M, N), dtype=torch.int32, device=A.device)
         out = torch.empty((M, N), dtype=torch.float16, device=A.device)
         L.check(lib.quik_sym_fused_dequantize(L.ptr(A), L.ptr(B), L.ptr(scale_row), L.ptr(scale_col), L.ptr(y), M, N, K,
@@ -110,7 +110,7 @@ def quantize_mapped(src: torch.Tensor, colmap: torch.Tensor, num_int: int, num_f
     L.dtype_id(src, "quantize", allow_bf16=False)
     rows, cols = src.shape
     lib = L.load()
-    with torch.cuda.device(src.device):
+    with L.device_guard(src.device):
         if tiled:
             nbytes = (lib.quik_fp6_operand_bytes if bits == 4 else lib.quik_tile8_operand_bytes)(max(rows, 1), num_int,
                                                                                                   num_fp)
