@@ -112,12 +112,171 @@ def cpu_baseline(name, x, W, int_idx, fp_idx, budget_s=25.0):
             "ms_per_step": med * 1e3}
 
 
+# ---------------------------------------------------------------------------------------------------
+# Full decoder block at Llama-2-70B dims (hidden 8192, 64 heads, 8 KV heads, MLP 28672): the seven
+# linears are MixedQLinear (q/k/v/o/gate/up W4A4, down_proj W8A8, 256 fp16 outlier columns each, q/k/v and
+# gate/up sharing their quantized input as experiments/llama.py:394-440 sets them up); RMSNorm, rotary-free
+# attention (torch SDPA, causal for prefill) and SiLU stay in PyTorch.  Random-init weights made on the device.
+BLOCK_WORKLOADS = {
+    # name: (batch, new tokens per sequence, tokens already in the KV cache)
+    "llama2-70b.decoder_block.prefill": (16, 512, 0),
+    "llama2-70b.decoder_block.decode": (64, 1, 512),
+}
+BLOCK_DIMS = dict(hidden=8192, heads=64, kv_heads=8, head_dim=128, mlp=28672, F=256)
+
+
+def make_device_layer(n_in, N, F, bits, fp_idx, shared, gen, device):
+    """A MixedQLinear with random codes and scales written straight into its buffers on the device (what
+    from_float would store for W = codes * scale; the distributions of make_layer)."""
+    import torch
+
+    from quik_amd.qlinear import MixedQLinear, pack_to_i4
+    K = n_in - F
+    mod = MixedQLinear(n_in, N, shared, fp_features_num=F, symm=False, bits=bits, dtype=torch.float16).to(device)
+    lo, hi = (-8, 8) if bits == 4 else (-127, 128)
+    s_w = (torch.rand(N, 1, generator=gen, device=device) * 0.009 + 0.001).half()
+    int_idx = torch.arange(n_in, device=device)
+    int_idx = int_idx[~torch.isin(int_idx, fp_idx)]
+    red = torch.empty(N, dtype=torch.float32, device=device)
+    for s in range(0, N, 4096):
+        e = min(N, s + 4096)
+        codes = torch.randint(lo, hi, (e - s, K), generator=gen, device=device, dtype=torch.int8)
+        mod.int_weight[s:e] = pack_to_i4(codes) if bits == 4 else codes
+        red[s:e] = (codes.float() * s_w[s:e].float()).half().float().sum(1)
+    mod.weights_scales.copy_(s_w)
+    mod.reduced_w.copy_(red.half().reshape(1, N))
+    mod.fp_weight.copy_((0.02 * torch.randn(N, F, generator=gen, device=device)).half())
+    mod.int_indices.copy_(int_idx)
+    mod.fp_indices.copy_(fp_idx)
+    mod.bias = None
+    return mod
+
+
+def bench_block(args):
+    import torch
+    import torch.nn.functional as Fn
+
+    from quik_amd.qlinear import FusedMixedQLinearGroup, SharedQuantizedInput
+    dev = torch.device("cuda:0")
+    B, S, past = BLOCK_WORKLOADS[args.workload]
+    d = BLOCK_DIMS
+    H, heads, kvh, hd, mlp, F = d["hidden"], d["heads"], d["kv_heads"], d["head_dim"], d["mlp"], d["F"]
+    gen = torch.Generator(device=dev).manual_seed(0)
+    fp_h = torch.randperm(H, generator=gen, device=dev)[:F]
+    fp_m = torch.randperm(mlp, generator=gen, device=dev)[:F]
+    sh_qkv, sh_mlp = SharedQuantizedInput(3), SharedQuantizedInput(2)
+    L = {
+        "q": make_device_layer(H, heads * hd, F, 4, fp_h, sh_qkv, gen, dev),
+        "k": make_device_layer(H, kvh * hd, F, 4, fp_h, sh_qkv, gen, dev),
+        "v": make_device_layer(H, kvh * hd, F, 4, fp_h, sh_qkv, gen, dev),
+        "o": make_device_layer(heads * hd, H, F, 4, fp_h, None, gen, dev),
+        "gate": make_device_layer(H, mlp, F, 4, fp_h, sh_mlp, gen, dev),
+        "up": make_device_layer(H, mlp, F, 4, fp_h, sh_mlp, gen, dev),
+        "down": make_device_layer(mlp, H, F, 8, fp_m, None, gen, dev),
+    }
+    # the same weights as two fused groups: one quantize and ONE GEMM for q/k/v and for gate/up
+    import copy
+    members = {n: copy.copy(L[n]) for n in ("q", "k", "v", "gate", "up")}
+    for m in members.values():
+        m.shared_input = None
+    g_qkv = FusedMixedQLinearGroup([members["q"], members["k"], members["v"]])
+    g_mlp = FusedMixedQLinearGroup([members["gate"], members["up"]])
+    norm1 = torch.ones(H, dtype=torch.float16, device=dev)
+    norm2 = torch.ones(H, dtype=torch.float16, device=dev)
+    x = torch.randn(B, S, H, generator=gen, device=dev)
+    x[..., fp_h] *= 50
+    x = x.half()
+    k_cache = torch.randn(B, kvh, past, hd, generator=gen, device=dev).half() if past else None
+    v_cache = torch.randn(B, kvh, past, hd, generator=gen, device=dev).half() if past else None
+
+    def rmsnorm(t, w):
+        v = t.float()
+        return (v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + 1e-5)).half() * w
+
+    def attention(q, k, v):
+        q = q.view(B, S, heads, hd).transpose(1, 2)
+        k = k.view(B, S, kvh, hd).transpose(1, 2)
+        v = v.view(B, S, kvh, hd).transpose(1, 2)
+        if past:
+            k, v = torch.cat([k_cache, k], 2), torch.cat([v_cache, v], 2)
+        k = k.repeat_interleave(heads // kvh, 1)
+        v = v.repeat_interleave(heads // kvh, 1)
+        o = Fn.scaled_dot_product_attention(q, k, v, is_causal=(past == 0 and S > 1))
+        return o.transpose(1, 2).reshape(B, S, heads * hd)
+
+    def block(t, fused_groups):
+        h = rmsnorm(t, norm1)
+        if fused_groups:
+            q, k, v = g_qkv(h)
+        else:
+            q, k, v = L["q"](h), L["k"](h), L["v"](h)
+        t = t + L["o"](attention(q, k, v))
+        h = rmsnorm(t, norm2)
+        if fused_groups:
+            g, u = g_mlp(h)
+        else:
+            g, u = L["gate"](h), L["up"](h)
+        return t + L["down"](Fn.silu(g) * u)
+
+    # inputs of realistic scale for timing the seven linears alone
+    h_in = rmsnorm(x, norm1)
+    a_in = torch.randn(B, S, heads * hd, generator=gen, device=dev).half()
+    m_in = torch.randn(B, S, mlp, generator=gen, device=dev)
+    m_in[..., fp_m] *= 50
+    m_in = m_in.half()
+
+    def linears(fused_groups):
+        if fused_groups:
+            g_qkv(h_in)
+        else:
+            L["q"](h_in), L["k"](h_in), L["v"](h_in)
+        L["o"](a_in)
+        if fused_groups:
+            g_mlp(h_in)
+        else:
+            L["gate"](h_in), L["up"](h_in)
+        L["down"](m_in)
+
+    def timed(fn):
+        for _ in range(args.warmup):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / args.steps
+
+    out = block(x, False)
+    out_f = block(x, True)
+    assert torch.isfinite(out).all() and torch.equal(out, out_f)       # the fused groups give the same bits
+    block_ms = timed(lambda: block(x, False))
+    block_f_ms = timed(lambda: block(x, True))
+    lin_ms = timed(lambda: linears(False))
+    lin_f_ms = timed(lambda: linears(True))
+    M = B * S
+    ops = sum(2.0 * M * m.out_features * m.int_features_num for m in L.values())
+    res = {
+        "metric": "decoder block latency, Llama-2-70B dims, 7 MixedQLinear + PyTorch norm/attention, 1 GPU",
+        "value": round(block_f_ms, 4), "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(block_f_ms, 4), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int4 / int8 (down_proj) codes, fp16 activations", "data": "synthetic",
+        "config": {"workload": f"{args.workload}: batch {B} x {S} new tokens, {past} cached; q/k/v and gate/up as "
+                               f"one GEMM each (FusedMixedQLinearGroup)", "tokens": M, **d},
+        "block_ms_seven_modules_shared_input": round(block_ms, 4),
+        "linears_only_ms": {"seven_modules_shared_input": round(lin_ms, 4), "fused_groups": round(lin_f_ms, 4)},
+        "linears_int_tops": round(ops / (lin_f_ms * 1e-3) / 1e12, 1),
+        "linears_pct_int8_mfma_peak": round(100.0 * ops / (lin_f_ms * 1e-3) / 1e12 / PEAK_INT8_TOPS, 2),
+    }
+    print(json.dumps(res))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="llama2-70b.gate_proj", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="llama2-70b.gate_proj", choices=sorted(WORKLOADS) + sorted(BLOCK_WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--unfused", action="store_true", help="run the reference's three-op sequence instead")
     ap.add_argument("--int8-mfma", action="store_true",
@@ -147,6 +306,10 @@ def main():
         torch.cuda.synchronize()
         print(json.dumps({"copy_calibration": True, "bytes_read_per_launch": src.numel() * 2,
                           "bytes_written_per_launch": src.numel() * 2, "launches": max(args.steps, 1)}))
+        return
+
+    if args.workload in BLOCK_WORKLOADS:
+        bench_block(args)
         return
 
     name = args.workload

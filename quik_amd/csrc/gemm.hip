@@ -20,6 +20,7 @@ using CfgLp = Cfg<256, 256, 2, 2, 0>;  // plain fallbacks
 using CfgMp = Cfg<128, 128, 2, 2, 0>;
 
 constexpr int kCUs = 256;
+constexpr int kLdsBytes = 160 * 1024;  // per CU, and the most one workgroup may ask for
 
 template <typename K>
 int prepare(K kern, int smem) {
@@ -110,22 +111,32 @@ int decode_waves(int64_t N, int64_t kbytes) {
   return (chunks >= 16 && slabs <= kCUs) ? 8 : 4;
 }
 
-template <int MODE, bool BF16, bool FUSED, int WAVES>
+template <int MODE, bool BF16, bool FUSED, int WAVES, bool XLDS>
 int launch_decode_w(const FusedArgs &p, int32_t *C, int ldc, hipStream_t st) {
-  auto kern = gemm_decode_kernel<MODE, BF16, FUSED, WAVES>;
-  constexpr int smem = decode_smem<WAVES, FUSED>();
+  auto kern = gemm_decode_kernel<MODE, BF16, FUSED, WAVES, XLDS>;
+  const int smem = decode_smem<WAVES, FUSED, XLDS>() + (XLDS ? static_cast<int>(decode_x_lds_bytes(p.M, p.kbytes)) : 0);
   if (int rc = prepare(kern, smem)) return rc;
-  // persistent workgroups: as many as are resident at once (8 waves per CU at this register count)
-  const int64_t slabs = (p.N + 31) / 32, resident = int64_t(kCUs) * (8 / WAVES);
+  // persistent workgroups: as many as are resident at once (8 waves per CU at this register count; the LDS copy
+  // of the token rows leaves room for one workgroup)
+  const int64_t slabs = (p.N + 31) / 32, resident = int64_t(kCUs) * (XLDS ? 1 : 8 / WAVES);
   hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(slabs < resident ? slabs : resident)), dim3(WAVES * 64), smem, st,
                      p, C, ldc);
   return check_launch();
 }
 
+// The token rows stay in LDS when they fit beside the reduction area and there is more than one slab per
+// workgroup to reuse them for (with fewer than 4 rows the L2 reads they replace cost less than the copy).
+template <int WAVES, bool FUSED>
+bool decode_x_fits(const FusedArgs &p) {
+  return p.M >= 4 && decode_smem<WAVES, FUSED, true>() + decode_x_lds_bytes(p.M, p.kbytes) <= kLdsBytes &&
+         (p.N + 31) / 32 > kCUs;
+}
+
 template <int MODE, bool BF16, bool FUSED>
 int launch_decode(const FusedArgs &p, int32_t *C, int ldc, hipStream_t st) {
-  if (decode_waves(p.N, p.kbytes) == 8) return launch_decode_w<MODE, BF16, FUSED, 8>(p, C, ldc, st);
-  return launch_decode_w<MODE, BF16, FUSED, 4>(p, C, ldc, st);
+  if (decode_x_fits<8, FUSED>(p)) return launch_decode_w<MODE, BF16, FUSED, 8, true>(p, C, ldc, st);
+  if (decode_waves(p.N, p.kbytes) == 8) return launch_decode_w<MODE, BF16, FUSED, 8, false>(p, C, ldc, st);
+  return launch_decode_w<MODE, BF16, FUSED, 4, false>(p, C, ldc, st);
 }
 
 // How a problem is cut into tiles.  Columns [0, n_wide) go to 256x256 tiles, [n_wide, N) to

@@ -15,6 +15,12 @@
 // slab the waves' partial accumulators (int32, exact in any order; fp32 outlier sums, added in
 // wave order) meet in LDS, and every wave finalises 16 / WAVES of the 16 values a lane owns with
 // the same epilogue formula as the large tiles.
+//
+// XLDS: the token operand lives in LDS.  Without it every slab re-reads all token rows from L2, as many bytes
+// as the slab's weights when there are 32 rows, and that traffic, not the weight stream, sets the time (a
+// 28672 x 7936 int4 layer: 34 us with one token row, 57 us with 32).  When the rows fit (rows x K bytes beside
+// the reduction area), each persistent workgroup copies them once, in the order the lanes read them
+// ([chunk][step][K half][row], 16 bytes each: conflict-free), and only the weights are streamed.
 #pragma once
 #include "gemm_kernels.h"
 
@@ -23,13 +29,20 @@ namespace quik {
 constexpr int kDecodeChunk = 128;  // K bytes per row and wave turn
 constexpr int kDecodeSteps = kDecodeChunk / 32;
 
-template <int WAVES, bool FUSED>
+// reduction area: int32 partial sums and, for the fused form, fp32 outlier sums; with XLDS the two share one
+// area (one after the other) to leave room for the token rows
+template <int WAVES, bool FUSED, bool XLDS = false>
 constexpr int decode_smem() {
-  return WAVES * 4096 * (FUSED ? 2 : 1);
+  return WAVES * 4096 * (FUSED && !XLDS ? 2 : 1);
+}
+// bytes of the LDS copy of `rows` token rows of `kbytes` bytes (whole 1 KB copies)
+inline int64_t decode_x_lds_bytes(int64_t rows, int64_t kbytes) {
+  const int64_t units = (kbytes + kDecodeChunk - 1) / kDecodeChunk * kDecodeSteps * 2 * rows;
+  return (units + 63) / 64 * 1024;
 }
 
 // FUSED: p.out receives the MixedQLinear output.  !FUSED: Cm receives the int32 product.
-template <int MODE, bool BF16, bool FUSED, int WAVES>
+template <int MODE, bool BF16, bool FUSED, int WAVES, bool XLDS = false>
 __global__ __launch_bounds__(WAVES * 64) void gemm_decode_kernel(FusedArgs args, int32_t *__restrict__ Cm, int ldc) {
   static_assert(WAVES == 4 || WAVES == 8, "16 values per lane are split over the waves");
   // plain locals: the lambdas below capture by reference, and a captured argument struct ends up in scratch
@@ -58,8 +71,24 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_decode_kernel(FusedArgs args,
   using FpOps = FragOps<BF16 ? kBF16 : kF16>;
 
   struct Buf {
-    v4i w[kDecodeSteps], x[kDecodeSteps];
+    v4i w[kDecodeSteps], x[XLDS ? 1 : kDecodeSteps];
   };
+  // ---- XLDS: copy the token rows into LDS, 16-byte unit u = ((chunk step) * 2 + K half) * M + row
+  const uint8_t *x_lds = smem + decode_smem<WAVES, FUSED, XLDS>();
+  if constexpr (XLDS) {
+    const int units = nchunks * kDecodeSteps * 2 * p.M;
+    const uint32_t lds_base = lds_address(x_lds);
+    for (int u0 = __builtin_amdgcn_readfirstlane(wave) * 64; u0 < units; u0 += WAVES * 64) {
+      const int u = u0 + lane < units ? u0 + lane : units - 1;  // the last copy is padded with a valid unit
+      const int cs = u / (2 * p.M), rem = u - cs * 2 * p.M;
+      const int hh = rem >= p.M ? 1 : 0, row = rem - hh * p.M;
+      int off = cs * 32 + hh * 16;
+      off = off < kbytes ? off : 0;  // past the row's end: the weights of these positions are zeroed below
+      dma_load16(p.qx, static_cast<uint32_t>(row * kbytes + off), lds_base + u0 * 16);
+    }
+    x_lds += (h * p.M + mrow) * 16;  // this lane's unit inside a step
+  }
+  const int x_step = 2 * p.M * 16;
   // ---- loader: item (ld_slab, ld_c) -> b, then advance to this wave's next item
   int ld_slab = blockIdx.x, ld_c = wave;
   auto issue = [&](Buf &b) __attribute__((always_inline)) {
@@ -72,10 +101,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_decode_kernel(FusedArgs args,
       const int off = base + s * 32;
       if (live && off + h * 16 < kbytes) {
         b.w[s] = *reinterpret_cast<const v4i *>(wp + off);
-        b.x[s] = *reinterpret_cast<const v4i *>(xp + off);
+        if constexpr (!XLDS) b.x[s] = *reinterpret_cast<const v4i *>(xp + off);
       } else {
         b.w[s] = v4i{0, 0, 0, 0};
-        b.x[s] = v4i{0, 0, 0, 0};
+        if constexpr (!XLDS) b.x[s] = v4i{0, 0, 0, 0};
       }
     }
     ld_c += WAVES;
@@ -129,19 +158,25 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_decode_kernel(FusedArgs args,
   v16i acc;
 #pragma unroll
   for (int v = 0; v < 16; ++v) acc[v] = 0;
-  auto multiply = [&](const Buf &b) __attribute__((always_inline)) {
+  auto multiply = [&](const Buf &b, int chunk) __attribute__((always_inline)) {
+    const uint8_t *xs = x_lds + (chunk < nchunks ? chunk : 0) * kDecodeSteps * x_step;  // (empty items: zero weights)
 #pragma unroll
     for (int s = 0; s < kDecodeSteps; ++s) {
       v4i wu[FragOps<MODE>::H], xu[FragOps<MODE>::H];
       FragOps<MODE>::unpack(b.w[s], wu);
-      FragOps<MODE>::unpack(b.x[s], xu);
+      if constexpr (XLDS) {
+        FragOps<MODE>::unpack(*reinterpret_cast<const v4i *>(xs + s * x_step), xu);
+      } else {
+        FragOps<MODE>::unpack(b.x[s], xu);
+      }
 #pragma unroll
       for (int k = 0; k < FragOps<MODE>::H; ++k) FragOps<MODE>::mma(xu[k], wu[k], acc);
     }
   };
 
   int32_t *red_i = reinterpret_cast<int32_t *>(smem);
-  float *red_f = reinterpret_cast<float *>(smem + WAVES * 4096);
+  constexpr bool kTwoPhase = XLDS && FUSED;  // fp32 sums go through the int32 area after it has been read
+  float *red_f = reinterpret_cast<float *>(smem + (kTwoPhase ? 0 : WAVES * 4096));
   // ---- end of a slab: outlier product, cross-wave reduction, epilogue, stores
   auto slab_end = [&](int slab) __attribute__((always_inline)) {
     v16f accf;
@@ -164,21 +199,40 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_decode_kernel(FusedArgs args,
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
       red_i[(wave * 16 + v) * 64 + lane] = acc[v];
-      if constexpr (FUSED) red_f[(wave * 16 + v) * 64 + lane] = accf[v];
+      if constexpr (FUSED && !kTwoPhase) red_f[(wave * 16 + v) * 64 + lane] = accf[v];
       acc[v] = 0;
     }
     __syncthreads();
     // wave w finalises values [w * VPW, (w + 1) * VPW) of every lane
+    int32_t tis[VPW];
+    float tfs[VPW];
 #pragma unroll
     for (int j = 0; j < VPW; ++j) {
       const int v = wave * VPW + j;
-      int32_t ti = 0;
-      float tf = 0.0f;
+      tis[j] = 0;
+      tfs[j] = 0.0f;
 #pragma unroll
       for (int q = 0; q < WAVES; ++q) {
-        ti += red_i[(q * 16 + v) * 64 + lane];
-        if constexpr (FUSED) tf += red_f[(q * 16 + v) * 64 + lane];
+        tis[j] += red_i[(q * 16 + v) * 64 + lane];
+        if constexpr (FUSED && !kTwoPhase) tfs[j] += red_f[(q * 16 + v) * 64 + lane];
       }
+    }
+    if constexpr (kTwoPhase) {
+      __syncthreads();
+#pragma unroll
+      for (int v = 0; v < 16; ++v) red_f[(wave * 16 + v) * 64 + lane] = accf[v];
+      __syncthreads();
+#pragma unroll
+      for (int j = 0; j < VPW; ++j) {
+#pragma unroll
+        for (int q = 0; q < WAVES; ++q) tfs[j] += red_f[(q * 16 + wave * VPW + j) * 64 + lane];
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < VPW; ++j) {
+      const int v = wave * VPW + j;
+      const int32_t ti = tis[j];
+      const float tf = tfs[j];
       const int n = slab * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
       if (r >= p.M || n >= p.N) continue;
       if constexpr (FUSED) {
@@ -197,12 +251,16 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_decode_kernel(FusedArgs args,
   int slab = blockIdx.x, c = wave;  // the item being multiplied
   slab_begin(slab);
   static_for<NB - 1>([&](auto I) __attribute__((always_inline)) { issue(buf[I.value]); });
+  if constexpr (XLDS) {  // every wave's share of the token rows has landed (with the first weight chunks)
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+    __syncthreads();
+  }
   while (slab < slabs) {  // uniform over the workgroup: all waves see the same slab sequence
     static_for<NB>([&](auto I) __attribute__((always_inline)) {
       if (slab >= slabs) return;
       constexpr int i = I.value;
       issue(buf[(i + NB - 1) % NB]);
-      multiply(buf[i]);
+      multiply(buf[i], c);
       c += WAVES;
       if (c >= nchunks) {
         slab_end(slab);

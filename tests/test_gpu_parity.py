@@ -753,12 +753,47 @@ FULL_SIZE = [
     (128, 13824, 5120, 256, 8, "student"),   # Llama-2-13B down_proj, int8, 128 tokens
     (16, 5120, 5120, 256, 4, "student"),     # Llama-2-13B q/k/v/o, 16 tokens
     (1, 5120, 13824, 256, 4, "student"),     # Llama-2-13B gate/up, single-token decode
+    (16, 5120, 13824, 256, 4, "student"),    # Llama-2-13B gate/up, 16 tokens: token rows resident in LDS
+    (32, 8192, 10240, 256, 4, "x50"),        # Llama-2-70B q+k+v, 32 tokens: the largest resident token operand
 ]
 
 
 @pytest.mark.parametrize("case", FULL_SIZE)
 def test_full_size_properties(case):
     _full_size_check(*case)
+
+
+DECODE_RESIDENT = [
+    # M, N, in, F, bits: N > 8192, so a workgroup of the weight-streaming kernel walks over several slabs
+    (16, 8192 + 4128, 1024 + 64, 64, 4),
+    (32, 8192 + 167, 2048 + 32, 32, 8),
+    (7, 9000, 512, 0, 4),
+    (32, 8320, 8192, 256, 4),
+    (4, 8224, 28672, 256, 8),      # int8 rows of a down_proj: four of them still fit
+]
+
+
+@pytest.mark.parametrize("case", DECODE_RESIDENT)
+def test_decode_kernel_with_token_rows_resident_in_lds(case):
+    """At most 32 token rows and more than 8192 output columns: the weight-streaming kernel keeps the token rows in
+    LDS.  Its output must have the bits of the same layer cut into column halves of at most 8192 columns (which
+    stream the token rows from L2), and agree with the oracle."""
+    M, N, n_in, F, bits = case
+    rng = np.random.default_rng(sum(case))
+    W, s_w, ii, fi = _layer(rng, N, n_in, F, bits)
+    bias = rng.standard_normal(N).astype(np.float16)
+    x = _acts(rng, M, n_in, fi).astype(np.float16)
+    out = _module(W, s_w, fi, bits, bias)(_t(x))[0]
+    half = N // 2
+    lo = _module(W[:half], s_w[:half], fi, bits, bias[:half])(_t(x))[0]
+    hi = _module(W[half:], s_w[half:], fi, bits, bias[half:])(_t(x))[0]
+    assert np.array_equal(_bits(out), np.concatenate([_bits(lo), _bits(hi)], axis=1))
+    cols = np.r_[0:64, N - 64:N]
+    omod = qo.from_float(W[cols], s_w[cols], fi, bits)
+    want, _ = qo.mixed_qlinear_forward(x, omod, bits, bias[cols])
+    got = out.float().cpu().numpy()[:, cols]
+    rms = np.sqrt((want.astype(np.float64) ** 2).mean())
+    assert np.abs(got.astype(np.float64) - want).max() <= 1e-2 * rms
 
 
 # ------------------------------------------------------------------------------ decoder block chain
