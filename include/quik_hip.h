@@ -170,7 +170,7 @@ int quik_sym_quantize_mapped(const void *x, int64_t rows, int64_t cols, const vo
  * No counterpart in the reference: the same forward as quik_asym_quantize (bits = 8) +
  * quik_mixed_linear_fwd (bits = 8, asymmetric), bit for bit, with both int8 operands (and the
  * outlier columns) stored in the order the GEMM tiles copy them, so that every copy moves whole
- * cache lines exactly once per tile.  Needs K % 64 == 0, F % 32 == 0, M > 32, a column map that
+ * cache lines exactly once per tile.  Needs K % 64 == 0, F % 32 == 0, a column map that
  * selects the streaming quantize kernel; operand buffers aligned to 256 bytes. */
 
 /* bytes of an operand buffer for [rows, K] int8 + [rows, F] outliers (0 if the shape is not supported) */
@@ -189,6 +189,27 @@ int quik_asym_quantize_tile8(const void *x, int dtype, int64_t rows, int64_t col
 int quik_mixed_linear_fwd_tile8(const void *x8, const void *w8, const void *meta, const void *s_col,
                                 const void *w_reduced, const void *bias, int dtype, int64_t M, int64_t N,
                                 int64_t K, int64_t F, void *out, void *stream);
+
+/* ---- K split for the tile-ordered GEMMs ----------------------------------------------------------
+ * No counterpart in the reference.  With few token rows and few output columns the 128x128 tiles of
+ * the tile-ordered GEMMs are fewer than the CUs and each walks the whole K (70B down_proj, 64 tokens:
+ * 64 tiles, K = 28416).  Given a workspace, several workgroups per tile take a K range each, add
+ * their exact accumulators through it, and the one that finishes last does the outlier product and
+ * the epilogue: same output bits, the weights stream through all CUs.
+ * quik_splitk_workspace_bytes: bytes with which the _ws entry points split this shape (0: they do
+ * not; bits = 4: the 6-bit path, bits = 8: the int8 path).  The workspace must be zero before its
+ * first use (its head holds arrival counters, which every launch leaves at zero again), 16-byte
+ * aligned, and must not be shared by launches that may overlap (other streams).  workspace == NULL
+ * or too small: no split, as the entry points without _ws. */
+int64_t quik_splitk_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits);
+int quik_mixed_linear_fwd_fp6_ws(const void *x6, const void *w6, const void *meta, const void *s_col,
+                                 const void *w_reduced, const void *bias, int dtype, int64_t M, int64_t N,
+                                 int64_t K, int64_t F, void *out, void *workspace, int64_t workspace_bytes,
+                                 void *stream);
+int quik_mixed_linear_fwd_tile8_ws(const void *x8, const void *w8, const void *meta, const void *s_col,
+                                   const void *w_reduced, const void *bias, int dtype, int64_t M, int64_t N,
+                                   int64_t K, int64_t F, void *out, void *workspace, int64_t workspace_bytes,
+                                   void *stream);
 
 /* quik.matmul.int4Matmul(A, B) -> C int32 [M, N]
  * replaces int4MatmulCUDA, src/matmul/matmul.cu:17-55.

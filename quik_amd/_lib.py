@@ -40,6 +40,11 @@ SIGNATURES = {
     "quik_tile8_pack_weight": (_int, [_vp, _vp, _i64, _i64, _i64, _vp, _vp]),
     "quik_asym_quantize_tile8": (_int, [_vp, _int, _i64, _i64, _vp, _i64, _i64, _vp, _vp, _vp]),
     "quik_mixed_linear_fwd_tile8": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _i64, _vp, _vp]),
+    "quik_splitk_workspace_bytes": (_i64, [_i64, _i64, _i64, _int]),
+    "quik_mixed_linear_fwd_fp6_ws": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _i64, _vp, _vp, _i64,
+                                            _vp]),
+    "quik_mixed_linear_fwd_tile8_ws": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _i64, _vp, _vp, _i64,
+                                              _vp]),
     "quik_int4_matmul": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "quik_int8_matmul": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "quik_mixed_linear_fwd": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _i64, _int,

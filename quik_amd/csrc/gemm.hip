@@ -262,8 +262,8 @@ int run_i32(const uint8_t *X, const uint8_t *W, int32_t *C, int64_t M, int64_t N
 
 // Tile plan of the 6-bit path (gemm_fp6.h).  Costs in percent of a 256x256 tile, measured at K = 7936, F = 256:
 // a 256x128 tile 59; 128x128 tiles run two to a CU, 66 for a pair, 36 for one that has the CU to itself.
-Plan make_plan6(int64_t M, int64_t N) {
-  if (M <= 32) return {Plan::kSmall, 0};
+Plan make_plan6(int64_t M, int64_t N, int64_t min_rows = 33) {
+  if (M < min_rows) return {Plan::kSmall, 0};
   const int64_t tiles_m = (M + 255) / 256;
   const int64_t mid_tiles = ((M + 127) / 128) * ((N + 127) / 128);
   const int64_t pairs = mid_tiles / (2 * kCUs), left = mid_tiles % (2 * kCUs);
@@ -279,6 +279,54 @@ Plan make_plan6(int64_t M, int64_t N) {
   }
   if (mid < best) return {Plan::kMid, 0};
   return {Plan::kSplit, best_n};
+}
+
+// Split over K for the tile-ordered kernels: few 128x128 tiles (at most half the CUs) and a long K.  Each of
+// `splits` workgroups per tile takes `per` steps (even); workspace = counters (one per tile, zero between launches)
+// followed by the partial accumulators.
+constexpr int64_t kSplitCounterBytes = 4096;
+constexpr int64_t kSplitMinSteps8 = 32, kSplitMinSteps6 = 32;  // at least 1024 (int8) / 2048 (6-bit) elements of K per workgroup
+struct SplitPlan {
+  int splits, per;
+  int64_t bytes;
+};
+SplitPlan plan_splitk(int64_t M, int64_t N, int64_t steps, int64_t min_steps, int64_t min_rows) {
+  SplitPlan none{1, 0, 0};
+  if (make_plan6(M, N, min_rows).kind != Plan::kMid) return none;
+  const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
+  if (tiles > kCUs / 2 || tiles * 4 > kSplitCounterBytes) return none;
+  for (int64_t splits = kCUs / tiles < 8 ? kCUs / tiles : 8; splits > 1; --splits) {
+    const int64_t per = ((steps + splits - 1) / splits + 1) / 2 * 2;
+    if (per >= min_steps && (splits - 1) * per < steps)
+      return {static_cast<int>(splits), static_cast<int>(per), kSplitCounterBytes + tiles * splits * 128 * 128 * 4};
+  }
+  return none;
+}
+
+template <bool BF16>
+int launch_fused6_splitk(const Fused6Args &p, const SplitPlan &sp, void *workspace, hipStream_t st) {
+  int tiles_m, tiles_n;
+  const int grid_tiles = grid_of<CfgM>(p.M, p.N, tiles_m, tiles_n);
+  SplitK sk{sp.splits, sp.per, grid_tiles, static_cast<uint32_t *>(workspace),
+            reinterpret_cast<int32_t *>(static_cast<uint8_t *>(workspace) + kSplitCounterBytes)};
+  auto kern = gemm_fused6_splitk_kernel<CfgM, BF16>;
+  constexpr int smem = fused6_smem<CfgM>();
+  if (int rc = prepare(kern, smem)) return rc;
+  hipLaunchKernelGGL(kern, dim3(grid_tiles * sp.splits), dim3(CfgM::kThreads), smem, st, p, tiles_m, tiles_n, sk);
+  return check_launch();
+}
+
+template <bool BF16>
+int launch_fused8t_splitk(const Fused8Args &p, const SplitPlan &sp, void *workspace, hipStream_t st) {
+  int tiles_m, tiles_n;
+  const int grid_tiles = grid_of<CfgM>(p.M, p.N, tiles_m, tiles_n);
+  SplitK sk{sp.splits, sp.per, grid_tiles, static_cast<uint32_t *>(workspace),
+            reinterpret_cast<int32_t *>(static_cast<uint8_t *>(workspace) + kSplitCounterBytes)};
+  auto kern = gemm_fused8t_splitk_kernel<CfgM, BF16>;
+  constexpr int smem = fused8t_smem<CfgM>();
+  if (int rc = prepare(kern, smem)) return rc;
+  hipLaunchKernelGGL(kern, dim3(grid_tiles * sp.splits), dim3(CfgM::kThreads), smem, st, p, tiles_m, tiles_n, sk);
+  return check_launch();
 }
 
 template <class C, bool BF16>
@@ -310,11 +358,15 @@ int launch_fused6_split(const Fused6Args &wide, const Fused6Args &tail, hipStrea
 // The 6-bit matrix-core path (gemm_fp6.h): 256x256 tiles alone (eight waves), 256x256 + 256x128 tiles in one
 // launch (four waves), or 128x128 tiles.
 template <bool BF16>
-int run_fused6(const Fused6Args &p, hipStream_t st) {
+int run_fused6(const Fused6Args &p, hipStream_t st, void *workspace, int64_t workspace_bytes) {
   const Plan plan = make_plan6(p.M, p.N);
   if (plan.kind == Plan::kSmall) return QUIK_ERR_SHAPE;  // at most 32 rows: the weight-streaming kernel is the right one
   if (plan.kind == Plan::kSplit && plan.n_wide >= p.N) return launch_fused6<CfgL8, BF16>(p, st);
-  if (plan.kind != Plan::kSplit) return launch_fused6<CfgM, BF16>(p, st);
+  if (plan.kind != Plan::kSplit) {
+    const SplitPlan sp = plan_splitk(p.M, p.N, p.K / 64, kSplitMinSteps6, 33);
+    if (sp.splits > 1 && workspace && workspace_bytes >= sp.bytes) return launch_fused6_splitk<BF16>(p, sp, workspace, st);
+    return launch_fused6<CfgM, BF16>(p, st);
+  }
   Fused6Args wide = p, tail = p;
   const int64_t nw = plan.n_wide;
   wide.N = static_cast<int>(nw);
@@ -355,10 +407,13 @@ int launch_fused8t_split(const Fused8Args &wide, const Fused8Args &tail, hipStre
 
 // W8A8 on tile-ordered operands (gemm_tile8.h): same plan and tile shapes as the 6-bit path.
 template <bool BF16>
-int run_fused8t(const Fused8Args &p, hipStream_t st) {
-  const Plan plan = make_plan6(p.M, p.N);
-  if (plan.kind == Plan::kSmall) return QUIK_ERR_SHAPE;  // at most 32 rows: the weight-streaming kernel is the right one
-  if (plan.kind != Plan::kSplit) return launch_fused8t<CfgM, BF16>(p, st);
+int run_fused8t(const Fused8Args &p, hipStream_t st, void *workspace, int64_t workspace_bytes) {
+  const Plan plan = make_plan6(p.M, p.N, 1);  // any row count: with few rows this path competes with the weight-streaming kernel
+  if (plan.kind != Plan::kSplit) {
+    const SplitPlan sp = plan_splitk(p.M, p.N, p.K / 32, kSplitMinSteps8, 1);
+    if (sp.splits > 1 && workspace && workspace_bytes >= sp.bytes) return launch_fused8t_splitk<BF16>(p, sp, workspace, st);
+    return launch_fused8t<CfgM, BF16>(p, st);
+  }
   if (plan.n_wide >= p.N) return launch_fused8t<CfgL8, BF16>(p, st);
   Fused8Args wide = p, tail = p;
   const int64_t nw = plan.n_wide;
@@ -452,9 +507,22 @@ extern "C" int quik_mixed_linear_fwd(const void *qx, const void *qw, const void 
   return dtype == QUIK_F16 ? run_fused<kInt8, false>(p, st) : run_fused<kInt8, true>(p, st);
 }
 
+extern "C" int64_t quik_splitk_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits) {
+  if (M <= 0 || N <= 0 || K <= 0 || (bits != 4 && bits != 8)) return 0;
+  if (bits == 4 ? K % 128 != 0 : K % 64 != 0) return 0;
+  return (bits == 4 ? plan_splitk(M, N, K / 64, kSplitMinSteps6, 33) : plan_splitk(M, N, K / 32, kSplitMinSteps8, 1)).bytes;
+}
+
 extern "C" int quik_mixed_linear_fwd_fp6(const void *x6, const void *w6, const void *meta, const void *s_col,
                                          const void *w_reduced, const void *bias, int dtype, int64_t M, int64_t N,
                                          int64_t K, int64_t F, void *out, void *stream) {
+  return quik_mixed_linear_fwd_fp6_ws(x6, w6, meta, s_col, w_reduced, bias, dtype, M, N, K, F, out, nullptr, 0, stream);
+}
+
+extern "C" int quik_mixed_linear_fwd_fp6_ws(const void *x6, const void *w6, const void *meta, const void *s_col,
+                                            const void *w_reduced, const void *bias, int dtype, int64_t M, int64_t N,
+                                            int64_t K, int64_t F, void *out, void *workspace,
+                                            int64_t workspace_bytes, void *stream) {
   if (dtype != QUIK_F16 && dtype != QUIK_BF16) return QUIK_ERR_DTYPE;
   if (M < 0 || N < 0 || K <= 0 || F < 0) return QUIK_ERR_SHAPE;
   if (M == 0 || N == 0) return QUIK_OK;
@@ -480,16 +548,24 @@ extern "C" int quik_mixed_linear_fwd_fp6(const void *x6, const void *w6, const v
   p.n_first = 0;
   p.N_total = static_cast<int>(N);
   hipStream_t st = as_stream(stream);
-  return dtype == QUIK_F16 ? run_fused6<false>(p, st) : run_fused6<true>(p, st);
+  if (workspace && reinterpret_cast<uintptr_t>(workspace) % 16 != 0) return QUIK_ERR_ALIGN;
+  return dtype == QUIK_F16 ? run_fused6<false>(p, st, workspace, workspace_bytes)
+                           : run_fused6<true>(p, st, workspace, workspace_bytes);
 }
 
 extern "C" int quik_mixed_linear_fwd_tile8(const void *x8, const void *w8, const void *meta, const void *s_col,
                                            const void *w_reduced, const void *bias, int dtype, int64_t M, int64_t N,
                                            int64_t K, int64_t F, void *out, void *stream) {
+  return quik_mixed_linear_fwd_tile8_ws(x8, w8, meta, s_col, w_reduced, bias, dtype, M, N, K, F, out, nullptr, 0, stream);
+}
+
+extern "C" int quik_mixed_linear_fwd_tile8_ws(const void *x8, const void *w8, const void *meta, const void *s_col,
+                                              const void *w_reduced, const void *bias, int dtype, int64_t M, int64_t N,
+                                              int64_t K, int64_t F, void *out, void *workspace,
+                                              int64_t workspace_bytes, void *stream) {
   if (dtype != QUIK_F16 && dtype != QUIK_BF16) return QUIK_ERR_DTYPE;
   if (M < 0 || N < 0 || K <= 0 || F < 0) return QUIK_ERR_SHAPE;
   if (M == 0 || N == 0) return QUIK_OK;
-  if (M <= 32) return QUIK_ERR_SHAPE;
   if (!x8 || !w8 || !meta || !s_col || !out) return QUIK_ERR_NULL;  // w_reduced == NULL: symmetric activations
   if (K % 64 != 0 || F % 32 != 0) return QUIK_ERR_ALIGN;
   auto misaligned = [](const void *p) { return reinterpret_cast<uintptr_t>(p) % 256 != 0; };
@@ -511,5 +587,7 @@ extern "C" int quik_mixed_linear_fwd_tile8(const void *x8, const void *w8, const
   p.n_first = 0;
   p.N_total = static_cast<int>(N);
   hipStream_t st = as_stream(stream);
-  return dtype == QUIK_F16 ? run_fused8t<false>(p, st) : run_fused8t<true>(p, st);
+  if (workspace && reinterpret_cast<uintptr_t>(workspace) % 16 != 0) return QUIK_ERR_ALIGN;
+  return dtype == QUIK_F16 ? run_fused8t<false>(p, st, workspace, workspace_bytes)
+                           : run_fused8t<true>(p, st, workspace, workspace_bytes);
 }

@@ -79,8 +79,11 @@ struct Fp6Pipe {
                             // then have to be copied into the operand tuples behind an exposed LDS round trip
 
   // xb0 / wb0: first 64-row block of the tile in each operand buffer
+  // unit0: first unit (step) of every block to copy; n_int / n_f: integer and outlier steps from there on
+  // (-1: all of the block's, from its first unit)
   __device__ __forceinline__ void init(uint8_t *smem_, const uint8_t *xbuf, const Fp6Layout &lx, int64_t xb0,
-                                       const uint8_t *wbuf, const Fp6Layout &lw, int64_t wb0) {
+                                       const uint8_t *wbuf, const Fp6Layout &lw, int64_t wb0, int unit0 = 0,
+                                       int n_int = -1, int n_f = -1) {
     smem = smem_;
     lds0 = lds_address(smem_);
     const int lane = threadIdx.x & 63;
@@ -90,7 +93,7 @@ struct Fp6Pipe {
       const Fp6Layout &l = is_x ? lx : lw;
       int64_t B = (is_x ? xb0 : wb0) + blk;
       B = B < l.blocks ? B : l.blocks - 1;  // blocks past the matrix: any valid block, results never stored
-      return (is_x ? xbuf : wbuf) + B * l.block_bytes;
+      return (is_x ? xbuf : wbuf) + B * l.block_bytes + int64_t(unit0) * 3072;
     };
     {
       const bool is_x = wave < XB;
@@ -110,8 +113,8 @@ struct Fp6Pipe {
     lane16 = lane * 16;
     fill = lds0;
     rd = 0;
-    steps0 = static_cast<int>(lx.steps);
-    steps = steps0 + static_cast<int>(lx.fsteps);
+    steps0 = n_int < 0 ? static_cast<int>(lx.steps) : n_int;
+    steps = steps0 + (n_f < 0 ? static_cast<int>(lx.fsteps) : n_f);
     left = steps;
     const int r = lane & 31, h = lane >> 5;
     const int slot16 = (h ^ ((r >> 3) & 1)) << 4;
@@ -394,8 +397,99 @@ constexpr int fused6_smem() {
   return Fp6Pipe<C>::SMEM + TileVectors6<C>::kBytes;
 }
 
-template <class C, bool BF16>
-__device__ __forceinline__ void fused6_tile(const Fused6Args &p, int tm, int tn, uint8_t *smem) {
+// Split over K (few tiles, long K): `splits` workgroups per tile take `per` integer steps each and add their raw
+// accumulators (int32, or the exact fp32 sums of the 6-bit path) through `partials`; the one that arrives last (counted in `counters`, which are zero between
+// launches) sums them, exactly, and goes on with the outlier steps and the epilogue as a whole-K tile would: the
+// result has the same bits.  partials: [tile][split][register][thread], 4 bytes each.
+struct SplitK {
+  int splits, per, grid_tiles;
+  uint32_t *counters;
+  int32_t *partials;
+};
+// The partial sums cross from one XCD's L2 to another's.  A device-wide fence would do that by writing back and
+// invalidating the whole L2 of the XCD, once per wave, under the operand streams of the other tiles (measured: the
+// launch takes three times as long), and device-scope atomic loads are issued one at a time.  Instead the partial
+// sums are moved by ordinary 16-byte stores and loads that carry the device-scope cache policy (sc1: past the L2,
+// one access at a time); the stores are complete (vmcnt) before the workgroup's barrier and the arrival count
+// behind it, and the loads are issued only after the count has been seen.
+// partials: [tile][split][group of 4 registers][thread][4].
+// (the wait states: a store of more than 8 bytes reads its data registers over several cycles, and the instruction
+// after this statement may be one that overwrites them; between the compiler's own instructions the compiler
+// keeps that distance, around inline assembly it does not)
+__device__ __forceinline__ void splitk_store4(int32_t *p, v4i v) {
+  asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 2" : : "v"(p), "v"(v) : "memory");
+}
+__device__ __forceinline__ void splitk_stores_done() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+// eight 16-byte loads, STRIDE int32 apart, and the wait for them in one statement: the compiler sees the
+// registers only once they hold the data
+template <int STRIDE>
+__device__ __forceinline__ void splitk_load8(const int32_t *p, v4i *r) {
+  asm volatile(
+      "global_load_dwordx4 %0, %8, off sc1\n\tglobal_load_dwordx4 %1, %9, off sc1\n\t"
+      "global_load_dwordx4 %2, %10, off sc1\n\tglobal_load_dwordx4 %3, %11, off sc1\n\t"
+      "global_load_dwordx4 %4, %12, off sc1\n\tglobal_load_dwordx4 %5, %13, off sc1\n\t"
+      "global_load_dwordx4 %6, %14, off sc1\n\tglobal_load_dwordx4 %7, %15, off sc1\n\t"
+      "s_waitcnt vmcnt(0)"
+      : "=&v"(r[0]), "=&v"(r[1]), "=&v"(r[2]), "=&v"(r[3]), "=&v"(r[4]), "=&v"(r[5]), "=&v"(r[6]), "=&v"(r[7])
+      : "v"(p), "v"(p + STRIDE), "v"(p + 2 * STRIDE), "v"(p + 3 * STRIDE), "v"(p + 4 * STRIDE), "v"(p + 5 * STRIDE),
+        "v"(p + 6 * STRIDE), "v"(p + 7 * STRIDE)
+      : "memory");
+}
+
+// Adds a tile's raw accumulators over the splits (see SplitK).  Returns false in every workgroup but the one that
+// arrived last; there `acc` holds the whole-K sums (INT: int32 bit patterns, else fp32) and the ring is idle.
+template <class C, bool INT>
+__device__ __forceinline__ bool splitk_combine(v16f (&acc)[C::MI][C::NI], const SplitK &sk, int tile_id, int split,
+                                               uint8_t *smem) {
+  static_assert(C::MI * C::NI == 4, "16 groups of 4 registers");
+  constexpr int STRIDE = C::kThreads * 4;
+  asm volatile("s_nop 15\n\ts_nop 15");  // the last MFMA results are architecturally visible
+  int32_t *mine = sk.partials + (int64_t(tile_id) * sk.splits + split) * 16 * STRIDE + threadIdx.x * 4;
+#pragma unroll
+  for (int b = 0; b < C::MI * C::NI; ++b)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const v16f &a = acc[b / C::NI][b % C::NI];
+      splitk_store4(mine + (b * 4 + g) * STRIDE,
+                    v4i{__float_as_int(agpr_read(a[4 * g])), __float_as_int(agpr_read(a[4 * g + 1])),
+                        __float_as_int(agpr_read(a[4 * g + 2])), __float_as_int(agpr_read(a[4 * g + 3]))});
+    }
+  splitk_stores_done();
+  __syncthreads();
+  int *last_s = reinterpret_cast<int *>(smem);
+  if (threadIdx.x == 0) {
+    const uint32_t before = __hip_atomic_fetch_add(sk.counters + tile_id, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    *last_s = before == static_cast<uint32_t>(sk.splits - 1);
+  }
+  __syncthreads();
+  const bool last = *last_s != 0;
+  __syncthreads();
+  if (!last) return false;
+  for (int q = 0; q < sk.splits; ++q) {  // exact sums: the order does not matter
+    if (q == split) continue;
+    const int32_t *theirs = sk.partials + (int64_t(tile_id) * sk.splits + q) * 16 * STRIDE + threadIdx.x * 4;
+    v4i t[16];
+    splitk_load8<STRIDE>(theirs, t);
+    splitk_load8<STRIDE>(theirs + 8 * STRIDE, t + 8);
+#pragma unroll
+    for (int b = 0; b < C::MI * C::NI; ++b)
+#pragma unroll
+      for (int g = 0; g < 4; ++g)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          v16f &a = acc[b / C::NI][b % C::NI];
+          const float mine_v = agpr_read(a[4 * g + e]);
+          a[4 * g + e] = agpr_write(INT ? __int_as_float(__float_as_int(mine_v) + t[b * 4 + g][e])
+                                        : mine_v + __int_as_float(t[b * 4 + g][e]));
+        }
+  }
+  if (threadIdx.x == 0) __hip_atomic_store(sk.counters + tile_id, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return true;
+}
+
+template <class C, bool BF16, bool SPLITK = false>
+__device__ __forceinline__ void fused6_tile(const Fused6Args &p, int tm, int tn, uint8_t *smem, int split = 0,
+                                            int tile_id = 0, const SplitK *sk = nullptr) {
   using Pipe = Fp6Pipe<C>;
   const int m0 = tm * C::BM, n0 = tn * C::BN;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -423,7 +517,15 @@ __device__ __forceinline__ void fused6_tile(const Fused6Args &p, int tm, int tn,
   }  // made visible by the first barrier of the pipeline
 
   Pipe pipe;
-  pipe.init(smem, p.xbuf, lx, m0 / 64, p.wbuf, lw, (p.n_first + n0) / 64);
+  const int total = static_cast<int>(lx.steps);
+  int k0 = 0, k1 = total;
+  if constexpr (SPLITK) {
+    k0 = split * sk->per;
+    k1 = k0 + sk->per < total ? k0 + sk->per : total;
+    pipe.init(smem, p.xbuf, lx, m0 / 64, p.wbuf, lw, (p.n_first + n0) / 64, k0, k1 - k0, 0);
+  } else {
+    pipe.init(smem, p.xbuf, lx, m0 / 64, p.wbuf, lw, (p.n_first + n0) / 64);
+  }
   pipe.start();  // its barrier also makes the vectors visible
 
   v16f acc[C::MI][C::NI];
@@ -431,12 +533,23 @@ __device__ __forceinline__ void fused6_tile(const Fused6Args &p, int tm, int tn,
   for (int ni = 0; ni < C::NI; ++ni)
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
-      const float4 cc = *reinterpret_cast<const float4 *>(tv.colc + wn * C::WN + ni * 32 + acc_col(g, lane));
+      float4 cc = *reinterpret_cast<const float4 *>(tv.colc + wn * C::WN + ni * 32 + acc_col(g, lane));
+      if (SPLITK && split != 0) cc = make_float4(0.0f, 0.0f, 0.0f, 0.0f);  // the column term enters once
 #pragma unroll
       for (int mi = 0; mi < C::MI; ++mi)
         acc[mi][ni][4 * g] = cc.x, acc[mi][ni][4 * g + 1] = cc.y, acc[mi][ni][4 * g + 2] = cc.z, acc[mi][ni][4 * g + 3] = cc.w;
     }
   pipe.run_fp6(acc);
+  if constexpr (SPLITK) {
+    pipe.drain();  // the copies past the last step have landed too: the ring is free
+    if (!splitk_combine<C, false>(acc, *sk, tile_id, split, smem)) return;
+    if (lx.fsteps > 0) {
+      pipe.init(smem, p.xbuf, lx, m0 / 64, p.wbuf, lw, (p.n_first + n0) / 64, total, 0, static_cast<int>(lx.fsteps));
+      pipe.start();
+    } else {
+      pipe.steps0 = pipe.steps = 0;
+    }
+  }
 
   // acc = S - colc / 64  ->  f32(integer accumulator) * (s_row * s_col), in place, one 32x32 block at a time
   float srow[C::MI], rowc[C::MI];
@@ -523,6 +636,17 @@ __global__ __launch_bounds__(C::kThreads) void gemm_fused6_kernel(Fused6Args p, 
   int tm, tn;
   if (!tile_of_block(blockIdx.x, tiles_m, tiles_n, tm, tn)) return;
   fused6_tile<C, BF16>(p, tm, tn, smem);
+}
+
+// K split over sk.splits workgroups per tile: block b works on tile b % grid_tiles, split b / grid_tiles.
+template <class C, bool BF16>
+__global__ __launch_bounds__(C::kThreads) void gemm_fused6_splitk_kernel(Fused6Args p, int tiles_m, int tiles_n,
+                                                                          SplitK sk) {
+  extern __shared__ __align__(16) uint8_t smem[];
+  int tm, tn;
+  const int split = blockIdx.x / sk.grid_tiles;
+  if (!tile_of_block(blockIdx.x - split * sk.grid_tiles, tiles_m, tiles_n, tm, tn)) return;
+  fused6_tile<C, BF16, true>(p, tm, tn, smem, split, tm * tiles_n + tn, &sk);
 }
 
 // One launch, two tile shapes (see gemm_i32_split_kernel).

@@ -52,8 +52,11 @@ struct Tile8Pipe {
   uint32_t x_head, w_head;  // this lane's fragment offsets inside a slot (fragment j: + 2048 (j / 2) + 1024 (j % 2))
   uint32_t x_head3[3], w_head3[3];  // the same inside slots 0, 2, 4
 
+  // unit0: first unit (step) of every block to copy; n_int / n_f: integer and outlier steps from there on
+  // (-1: all of the block's, from its first unit)
   __device__ __forceinline__ void init(uint8_t *smem_, const uint8_t *xbuf, const Tile8Layout &lx, int64_t xb0,
-                                       const uint8_t *wbuf, const Tile8Layout &lw, int64_t wb0) {
+                                       const uint8_t *wbuf, const Tile8Layout &lw, int64_t wb0, int unit0 = 0,
+                                       int n_int = -1, int n_f = -1) {
     smem = smem_;
     lds0 = lds_address(smem_);
     const int lane = threadIdx.x & 63;
@@ -63,7 +66,7 @@ struct Tile8Pipe {
       const Tile8Layout &l = is_x ? lx : lw;
       int64_t B = (is_x ? xb0 : wb0) + blk;
       B = B < l.blocks ? B : l.blocks - 1;  // blocks past the matrix: any valid block, results never stored
-      return (is_x ? xbuf : wbuf) + B * l.block_bytes;
+      return (is_x ? xbuf : wbuf) + B * l.block_bytes + int64_t(unit0) * 2048;
     };
     {
       const bool is_x = wave < XB;
@@ -83,8 +86,8 @@ struct Tile8Pipe {
     lane16 = lane * 16;
     fill = lds0;
     rd = 0;
-    steps0 = static_cast<int>(lx.steps);
-    steps = steps0 + static_cast<int>(lx.fsteps);
+    steps0 = n_int < 0 ? static_cast<int>(lx.steps) : n_int;
+    steps = steps0 + (n_f < 0 ? static_cast<int>(lx.fsteps) : n_f);
     left = steps;
     const int r = lane & 31, h = lane >> 5;
     const int slot16 = (h ^ ((r >> 3) & 1)) << 4;
@@ -251,8 +254,9 @@ constexpr int fused8t_smem() {
   return tile8_vectors_offset<C>() + TileVectors<C>::kBytes;
 }
 
-template <class C, bool BF16>
-__device__ __forceinline__ void fused8t_tile(const Fused8Args &p, int tm, int tn, uint8_t *smem) {
+template <class C, bool BF16, bool SPLITK = false>
+__device__ __forceinline__ void fused8t_tile(const Fused8Args &p, int tm, int tn, uint8_t *smem, int split = 0,
+                                             int tile_id = 0, const SplitK *sk = nullptr) {
   using Pipe = Tile8Pipe<C>;
   const int m0 = tm * C::BM, n0 = tn * C::BN;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -282,11 +286,29 @@ __device__ __forceinline__ void fused8t_tile(const Fused8Args &p, int tm, int tn
       for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0.0f;
 
   Pipe pipe;
-  pipe.init(smem, p.xbuf, lx, m0 / 64, p.wbuf, lw, (p.n_first + n0) / 64);
-  pipe.start();
   v4i f0[Pipe::NF], f1[Pipe::NF];
-  pipe.read_all(f0);
-  pipe.template run<kInt8, true>(0, pipe.steps0, f0, f1, acc);
+  if constexpr (!SPLITK) {
+    pipe.init(smem, p.xbuf, lx, m0 / 64, p.wbuf, lw, (p.n_first + n0) / 64);
+    pipe.start();
+    pipe.read_all(f0);
+    pipe.template run<kInt8, true>(0, pipe.steps0, f0, f1, acc);
+  } else {
+    const int total = static_cast<int>(lx.steps), k0 = split * sk->per;
+    const int k1 = k0 + sk->per < total ? k0 + sk->per : total;
+    pipe.init(smem, p.xbuf, lx, m0 / 64, p.wbuf, lw, (p.n_first + n0) / 64, k0, k1 - k0, 0);
+    pipe.start();
+    pipe.read_all(f0);
+    pipe.template run<kInt8, true>(0, pipe.steps0, f0, f1, acc);
+    pipe.drain();  // the copies past the last step have landed too: the ring is free
+    if (!splitk_combine<C, true>(acc, *sk, tile_id, split, smem)) return;
+    if (lx.fsteps > 0) {
+      pipe.init(smem, p.xbuf, lx, m0 / 64, p.wbuf, lw, (p.n_first + n0) / 64, total, 0, static_cast<int>(lx.fsteps));
+      pipe.start();
+      pipe.read_all(f0);
+    } else {
+      pipe.steps0 = pipe.steps = 0;
+    }
+  }
 
   // acc -> f32(acc) * (s_row * s_col), in place, one 32x32 block at a time
   float srow[C::MI];
@@ -369,6 +391,18 @@ __global__ __launch_bounds__(C::kThreads) void gemm_fused8t_kernel(Fused8Args p,
   int tm, tn;
   if (!tile_of_block(blockIdx.x, tiles_m, tiles_n, tm, tn)) return;
   fused8t_tile<C, BF16>(p, tm, tn, smem);
+}
+
+// K split over sk.splits workgroups per tile: block b works on tile b % grid_tiles (same XCD for all splits of a
+// tile's neighbourhood), split b / grid_tiles.
+template <class C, bool BF16>
+__global__ __launch_bounds__(C::kThreads) void gemm_fused8t_splitk_kernel(Fused8Args p, int tiles_m, int tiles_n,
+                                                                           SplitK sk) {
+  extern __shared__ __align__(16) uint8_t smem[];
+  int tm, tn;
+  const int split = blockIdx.x / sk.grid_tiles;
+  if (!tile_of_block(blockIdx.x - split * sk.grid_tiles, tiles_m, tiles_n, tm, tn)) return;
+  fused8t_tile<C, BF16, true>(p, tm, tn, smem, split, tm * tiles_n + tn, &sk);
 }
 
 // One launch, two tile shapes (see gemm_i32_split_kernel).

@@ -86,6 +86,32 @@ def mixed_linear(qx, int_weight, meta, weights_scales, reduced_w, fp_x, fp_weigh
     return out
 
 
+# K split of the tile-ordered GEMMs (few token rows, few output columns, long K): one zeroed workspace per GPU,
+# shared by all layers (arrival counters, which every launch leaves at zero, and partial sums).  Launches that may
+# overlap on one GPU (several streams) must not share it: set split_k = False there.
+split_k = True
+_SPLITK_BYTES = 4096 + 256 * 128 * 128 * 4   # the largest request: 256 workgroups of one 128x128 tile each
+_splitk_workspaces = {}
+_splitk_needed = {}
+
+
+def _splitk_workspace(device, M, N, K, bits):
+    if not split_k:
+        return None, 0
+    key = (M, N, K, bits)
+    need = _splitk_needed.get(key)
+    if need is None:
+        need = _splitk_needed[key] = L.load().quik_splitk_workspace_bytes(M, N, K, bits)
+    if need == 0:
+        return None, 0
+    ws = _splitk_workspaces.get(device.index)
+    if ws is None:
+        if torch.cuda.is_current_stream_capturing():   # no allocation that a graph's pool would own
+            return None, 0
+        ws = _splitk_workspaces[device.index] = torch.zeros(_SPLITK_BYTES, dtype=torch.uint8, device=device)
+    return ws, ws.numel()
+
+
 def pack_weight_fp6(int_weight: torch.Tensor, fp_weight: torch.Tensor) -> torch.Tensor:
     """Nibble-packed int4 weights [N, K/2] and outlier weights [N, F] -> operand buffer for mixed_linear_fp6
     (once per layer)."""
@@ -131,9 +157,10 @@ def mixed_linear_fp6(x6, w6, meta, weights_scales, reduced_w, bias, M, N, K, F, 
         raise RuntimeError("mixed_linear_fp6: meta / weights_scales / reduced_w sizes are inconsistent with M, N")
     with L.device_guard(x6.device):
         out = torch.empty((M, N), dtype=out_dtype, device=x6.device)
-        L.check(lib.quik_mixed_linear_fwd_fp6(L.ptr(x6), L.ptr(w6), L.ptr(meta), L.ptr(weights_scales),
-                                              L.ptr(tensors.get("reduced_w")), L.ptr(tensors.get("bias")), dt, M, N, K, F,
-                                              L.ptr(out), L.stream()), "mixed_linear_fp6")
+        ws, ws_bytes = _splitk_workspace(x6.device, M, N, K, 4)
+        L.check(lib.quik_mixed_linear_fwd_fp6_ws(L.ptr(x6), L.ptr(w6), L.ptr(meta), L.ptr(weights_scales),
+                                                 L.ptr(tensors.get("reduced_w")), L.ptr(tensors.get("bias")), dt, M, N, K,
+                                                 F, L.ptr(out), L.ptr(ws), ws_bytes, L.stream()), "mixed_linear_fp6")
     return out
 
 
@@ -182,7 +209,9 @@ def mixed_linear_tile8(x8, w8, meta, weights_scales, reduced_w, bias, M, N, K, F
         raise RuntimeError("mixed_linear_tile8: meta / weights_scales / reduced_w sizes are inconsistent with M, N")
     with L.device_guard(x8.device):
         out = torch.empty((M, N), dtype=out_dtype, device=x8.device)
-        L.check(lib.quik_mixed_linear_fwd_tile8(L.ptr(x8), L.ptr(w8), L.ptr(meta), L.ptr(weights_scales),
-                                                L.ptr(tensors.get("reduced_w")), L.ptr(tensors.get("bias")), dt, M, N, K, F,
-                                                L.ptr(out), L.stream()), "mixed_linear_tile8")
+        ws, ws_bytes = _splitk_workspace(x8.device, M, N, K, 8)
+        L.check(lib.quik_mixed_linear_fwd_tile8_ws(L.ptr(x8), L.ptr(w8), L.ptr(meta), L.ptr(weights_scales),
+                                                   L.ptr(tensors.get("reduced_w")), L.ptr(tensors.get("bias")), dt, M, N,
+                                                   K, F, L.ptr(out), L.ptr(ws), ws_bytes, L.stream()),
+                "mixed_linear_tile8")
     return out

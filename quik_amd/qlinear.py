@@ -74,6 +74,7 @@ class MixedQLinear(torch.nn.Module):
     of the row-major kernels; `six_bit_path = False` turns them off."""
 
     six_bit_min_rows = 33    # up to 32 rows the weight-streaming decode kernel on the packed int4 weights is the right one
+    tile8_min_rows = 17      # 8 bits: with its K split the tile-ordered path passes the weight-streaming kernel at 8 to 18 rows (70B to 7B down_proj)
 
     def __init__(self, in_features, out_features, shared_input=None,
                  fp_features_num=0, symm=False, bits=4, dtype=torch.float16, fused=True):
@@ -126,7 +127,8 @@ class MixedQLinear(torch.nn.Module):
         if self.symmetric and self.dtype != torch.float16:      # symmetric activations are fp16 (as in the reference)
             return False
         k_multiple = 128 if self.bits == 4 else 64
-        if rows < self.six_bit_min_rows or self.int_features_num % k_multiple != 0 or self.fp_features_num % 32 != 0:
+        min_rows = self.six_bit_min_rows if self.bits == 4 else self.tile8_min_rows
+        if rows < min_rows or self.int_features_num % k_multiple != 0 or self.fp_features_num % 32 != 0:
             return False
         if self.bits == 4 and self.int_features_num > 74496:   # the 6-bit path's fp32 sums are exact up to here
             return False

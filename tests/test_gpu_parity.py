@@ -1149,6 +1149,69 @@ def test_symmetric_module_on_tile_ordered_operands(case):
     assert np.abs(got.astype(np.float64) - want).max() <= 1e-2 * rms
 
 
+SPLIT_K_CASES = [
+    # M, N, in, F, bits, symm, bf16: few 128x128 tiles and a long K
+    (64, 512, 4096 + 64, 64, 4, False, False),
+    (64, 1024, 8192, 256, 4, False, True),
+    (100, 640, 4096 + 32, 32, 8, False, False),
+    (256, 520, 2048 + 64, 64, 8, False, True),      # ragged N
+    (64, 384, 8192, 0, 4, False, False),            # no outlier columns
+    (33, 130, 4096 + 64, 64, 4, True, False),       # symmetric activations, ragged M and N
+    (200, 8192, 28672, 256, 8, False, False),       # Llama-2-70B down_proj at 200 tokens
+]
+
+
+@pytest.mark.parametrize("case", SPLIT_K_CASES)
+def test_split_k_gives_the_same_bits(case):
+    """Tile-ordered GEMMs with K split over several workgroups per tile (partial sums through a workspace, the last
+    workgroup to arrive finishes the tile) against the same layer without the split: identical output bits, on
+    repeated calls (the arrival counters return to zero) and with edge-case rows."""
+    from quik_amd import _lib, matmul
+    M, N, n_in, F, bits, symm, bf16 = case
+    K = n_in - F
+    assert _lib.load().quik_splitk_workspace_bytes(M, N, K, bits) > 0       # the shape does split
+    rng = np.random.default_rng(sum(case[:5]))
+    W, s_w, ii, fi = _layer(rng, N, n_in, F, bits)
+    bias = rng.standard_normal(N).astype(np.float16)
+    x = _edge_rows(_acts(rng, M, n_in, fi).astype(np.float16), ii)
+    mod = _module(W, s_w, fi, bits, bias, symm=symm)
+    if bf16:
+        mod = mod.to(torch.bfloat16)
+        mod.dtype = torch.bfloat16
+    xt = _bf16_t(x.astype(np.float32)) if bf16 else _t(x)
+    assert matmul.split_k
+    try:
+        got = [_bits(mod(xt)) for _ in range(3)]
+        matmul.split_k = False
+        want = _bits(mod(xt))
+    finally:
+        matmul.split_k = True
+    nan_rows = np.isnan(x[:, ii].astype(np.float32)).any(1) if symm else np.zeros(M, bool)
+    for g in got:
+        assert np.array_equal(g[0][~nan_rows], want[0][~nan_rows])
+    ws = matmul._splitk_workspaces[torch.cuda.current_device()]
+    assert int(ws[:4096].view(torch.int32).abs().sum()) == 0               # counters are back at zero
+
+
+@pytest.mark.parametrize("M", [16, 17, 24, 32])
+def test_int8_layers_switch_to_tile_ordered_operands_at_17_rows(M):
+    """W8A8: from 17 token rows the tile-ordered path (with its K split) is faster than the weight-streaming
+    kernel; below, that kernel runs.  Both against the oracle (their fp32 sums differ in order, so not bit for bit
+    against each other)."""
+    N, n_in, F, bits = 520, 4096 + 64, 64, 8
+    rng = np.random.default_rng(M)
+    W, s_w, ii, fi = _layer(rng, N, n_in, F, bits)
+    bias = rng.standard_normal(N).astype(np.float16)
+    x = _acts(rng, M, n_in, fi).astype(np.float16)
+    mod = _module(W, s_w, fi, bits, bias)
+    out = mod(_t(x))[0].float().cpu().numpy()
+    assert (mod._w6 is not None) == (M >= 17)
+    omod = qo.from_float(W, s_w, fi, bits)
+    want, _ = qo.mixed_qlinear_forward(x, omod, bits, bias)
+    rms = np.sqrt((want.astype(np.float64) ** 2).mean())
+    assert np.abs(out.astype(np.float64) - want).max() <= 1e-2 * rms
+
+
 def test_six_bit_path_shared_input_and_fallbacks():
     """A q/k/v-style group on the 6-bit path quantizes once into the operand format; a member with the path
     switched off, or a call with fewer rows than the threshold, takes the int4 path, with the same results."""
