@@ -46,6 +46,8 @@ WORKLOADS = {
     "llama2-13b.gate_proj.t1": (1, 5120, 13824, 256, 4),
     "llama2-13b.down_proj.int8.t16": (16, 13824, 5120, 256, 8),
     "llama2-70b.gate_proj.t64": (64, 8192, 28672, 256, 4),
+    "llama2-70b.gate_proj.t32": (32, 8192, 28672, 256, 4),          # weight-streaming kernel, token rows in LDS
+    "llama2-70b.down_proj.int8.t64": (64, 28672, 8192, 256, 8),     # 64 tiles, K = 28416: split over K
 }
 
 PEAK_INT8_TOPS = 5000.0   # MI355X dense int8 MFMA, published
@@ -417,14 +419,19 @@ def main():
     quant_bytes = M * n_in * 2 + (M * K * 6 // 8 + M * 4 if six and bits == 4 else M * K * bits // 8) + M * F * 2 + M * 4
     quant_gbps = quant_bytes / (q_avg * 1e-3) / 1e9
     peak = PEAK_FP6_TOPS if six and bits == 4 else PEAK_INT8_TOPS
+    split_k = six and matmul.split_k and _lib.load().quik_splitk_workspace_bytes(M, N, K, bits) > 0
     if six and bits == 4:
-        gemm_kernel = "gemm_fused6_split_kernel / gemm_fused6_kernel (one launch per step)"
+        gemm_kernel = "gemm_fused6_splitk_kernel (K split over several workgroups per tile)" if split_k else \
+            "gemm_fused6_split_kernel / gemm_fused6_kernel (one launch per step)"
         dtype = "int4 (exact, as E2M3 on the 6-bit MFMA path)"
     elif six:
-        gemm_kernel = "gemm_fused8t_split_kernel / gemm_fused8t_kernel (tile-ordered int8 operands, one launch per step)"
+        gemm_kernel = "gemm_fused8t_splitk_kernel (tile-ordered int8 operands, K split over several workgroups per " \
+            "tile)" if split_k else \
+            "gemm_fused8t_split_kernel / gemm_fused8t_kernel (tile-ordered int8 operands, one launch per step)"
         dtype = "int8"
     elif mod.fused:
-        gemm_kernel = "gemm_fused_split_kernel (one launch per step)"
+        gemm_kernel = "gemm_decode_kernel (weight streaming, one launch per step)" if M <= 32 else \
+            "gemm_fused_split_kernel / gemm_fused_kernel (one launch per step)"
         dtype = "int8" if bits == 8 else "int4 (on int8 MFMA)"
     else:
         gemm_kernel = "gemm_i32_split_kernel + dequantize + F.linear"

@@ -168,7 +168,9 @@ int quik_sym_quantize_mapped(const void *x, int64_t rows, int64_t cols, const vo
 
 /* ---- W8A8 on tile-ordered operands -------------------------------------------------------------
  * No counterpart in the reference: the same forward as quik_asym_quantize (bits = 8) +
- * quik_mixed_linear_fwd (bits = 8, asymmetric), bit for bit, with both int8 operands (and the
+ * quik_mixed_linear_fwd (bits = 8, asymmetric), bit for bit for more than 32 rows (up to 32 rows
+ * that entry point runs a weight-streaming kernel, which adds the fp32 terms in another order:
+ * equal within rounding), with both int8 operands (and the
  * outlier columns) stored in the order the GEMM tiles copy them, so that every copy moves whole
  * cache lines exactly once per tile.  Needs K % 64 == 0, F % 32 == 0, a column map that
  * selects the streaming quantize kernel; operand buffers aligned to 256 bytes. */
