@@ -290,12 +290,14 @@ struct SplitPlan {
   int splits, per;
   int64_t bytes;
 };
-SplitPlan plan_splitk(int64_t M, int64_t N, int64_t steps, int64_t min_steps, int64_t min_rows) {
+// min_splits: with two workgroups per tile the exchange and the restart for the outlier steps cost the 6-bit path
+// (K <= 8192 in every Llama layer it serves) what the halved K loop saves; measured gains start at three.
+SplitPlan plan_splitk(int64_t M, int64_t N, int64_t steps, int64_t min_steps, int64_t min_rows, int64_t min_splits) {
   SplitPlan none{1, 0, 0};
   if (make_plan6(M, N, min_rows).kind != Plan::kMid) return none;
   const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
   if (tiles > kCUs / 2 || tiles * 4 > kSplitCounterBytes) return none;
-  for (int64_t splits = kCUs / tiles < 8 ? kCUs / tiles : 8; splits > 1; --splits) {
+  for (int64_t splits = kCUs / tiles < 8 ? kCUs / tiles : 8; splits >= min_splits; --splits) {
     const int64_t per = ((steps + splits - 1) / splits + 1) / 2 * 2;
     if (per >= min_steps && (splits - 1) * per < steps)
       return {static_cast<int>(splits), static_cast<int>(per), kSplitCounterBytes + tiles * splits * 128 * 128 * 4};
@@ -363,7 +365,7 @@ int run_fused6(const Fused6Args &p, hipStream_t st, void *workspace, int64_t wor
   if (plan.kind == Plan::kSmall) return QUIK_ERR_SHAPE;  // at most 32 rows: the weight-streaming kernel is the right one
   if (plan.kind == Plan::kSplit && plan.n_wide >= p.N) return launch_fused6<CfgL8, BF16>(p, st);
   if (plan.kind != Plan::kSplit) {
-    const SplitPlan sp = plan_splitk(p.M, p.N, p.K / 64, kSplitMinSteps6, 33);
+    const SplitPlan sp = plan_splitk(p.M, p.N, p.K / 64, kSplitMinSteps6, 33, 3);
     if (sp.splits > 1 && workspace && workspace_bytes >= sp.bytes) return launch_fused6_splitk<BF16>(p, sp, workspace, st);
     return launch_fused6<CfgM, BF16>(p, st);
   }
@@ -410,7 +412,7 @@ template <bool BF16>
 int run_fused8t(const Fused8Args &p, hipStream_t st, void *workspace, int64_t workspace_bytes) {
   const Plan plan = make_plan6(p.M, p.N, 1);  // any row count: with few rows this path competes with the weight-streaming kernel
   if (plan.kind != Plan::kSplit) {
-    const SplitPlan sp = plan_splitk(p.M, p.N, p.K / 32, kSplitMinSteps8, 1);
+    const SplitPlan sp = plan_splitk(p.M, p.N, p.K / 32, kSplitMinSteps8, 1, 2);
     if (sp.splits > 1 && workspace && workspace_bytes >= sp.bytes) return launch_fused8t_splitk<BF16>(p, sp, workspace, st);
     return launch_fused8t<CfgM, BF16>(p, st);
   }
@@ -510,7 +512,7 @@ extern "C" int quik_mixed_linear_fwd(const void *qx, const void *qw, const void 
 extern "C" int64_t quik_splitk_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits) {
   if (M <= 0 || N <= 0 || K <= 0 || (bits != 4 && bits != 8)) return 0;
   if (bits == 4 ? K % 128 != 0 : K % 64 != 0) return 0;
-  return (bits == 4 ? plan_splitk(M, N, K / 64, kSplitMinSteps6, 33) : plan_splitk(M, N, K / 32, kSplitMinSteps8, 1)).bytes;
+  return (bits == 4 ? plan_splitk(M, N, K / 64, kSplitMinSteps6, 33, 3) : plan_splitk(M, N, K / 32, kSplitMinSteps8, 1, 2)).bytes;
 }
 
 extern "C" int quik_mixed_linear_fwd_fp6(const void *x6, const void *w6, const void *meta, const void *s_col,

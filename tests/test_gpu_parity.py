@@ -1151,12 +1151,12 @@ def test_symmetric_module_on_tile_ordered_operands(case):
 
 SPLIT_K_CASES = [
     # M, N, in, F, bits, symm, bf16: few 128x128 tiles and a long K
-    (64, 512, 4096 + 64, 64, 4, False, False),
+    (64, 512, 8192 + 64, 64, 4, False, False),
     (64, 1024, 8192, 256, 4, False, True),
     (100, 640, 4096 + 32, 32, 8, False, False),
     (256, 520, 2048 + 64, 64, 8, False, True),      # ragged N
     (64, 384, 8192, 0, 4, False, False),            # no outlier columns
-    (33, 130, 4096 + 64, 64, 4, True, False),       # symmetric activations, ragged M and N
+    (33, 130, 8192 + 64, 64, 4, True, False),       # symmetric activations, ragged M and N
     (200, 8192, 28672, 256, 8, False, False),       # Llama-2-70B down_proj at 200 tokens
 ]
 
