@@ -7,10 +7,16 @@
 // continuous stream of (slab, chunk) items with NB register sets in rotation, so NB - 1 chunks
 // are always in flight ahead of the one being multiplied, across slab boundaries too: the memory
 // latency is paid once per wave, not once per slab.
-// Lane l loads 16 bytes of weight row l % 32 at K half l / 32 of each 32-byte step and the
-// matching 16 bytes of token row l % 32: exactly the operand layout of v_mfma_i32_32x32x32_i8, so
-// there is no LDS stage and no shuffle (int4: the same in-register nibble split as the large
-// tiles).  The fp16/bf16 outlier columns are split over the waves the same way; those loads and
+// The MFMA wants lane l to hold 16 bytes of weight row l % 32 at K half l / 32 of a 32-byte step.  Loading them
+// that way asks for 32 bytes of 32 different rows per instruction, and the memory path then delivers 13-24 % less
+// than when an instruction covers whole 128-byte lines (measured with the loads rearranged and the results
+// ignored).  So load i of a chunk has lane l fetch 16-byte piece l % 8 of row 8 i + l / 8 (eight whole lines), and
+// at multiply time the wave passes the chunk through 4 KB of LDS of its own, written as a row-major 32 x 128 byte
+// tile (pieces XOR-swizzled by (row / 2) % 8, so that the writes and the reads below are conflict-free) and read
+// back in the operand layout.  The LDS of a wave executes in order: no waits beyond the data dependences.
+// The token rows take the same route in the fused form (rows past M repeat the last one), are loaded in the operand
+// layout directly in the plain integer form, or are read from their LDS copy (XLDS); int4: the same in-register
+// nibble split as the large tiles.  The fp16/bf16 outlier columns are split over the waves the same way; those loads and
 // the epilogue's per-row / per-column scalars are requested when a slab starts.  At the end of a
 // slab the waves' partial accumulators (int32, exact in any order; fp32 outlier sums, added in
 // wave order) meet in LDS, and every wave finalises 16 / WAVES of the 16 values a lane owns with
@@ -93,18 +99,24 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_decode_kernel(FusedArgs args,
   int ld_slab = blockIdx.x, ld_c = wave;
   auto issue = [&](Buf &b) __attribute__((always_inline)) {
     const bool live = ld_slab < slabs && ld_c < nchunks;
-    const int n = ld_slab * 32 + r;
-    const uint8_t *wp = p.qw + int64_t(n < p.N ? n : p.N - 1) * kbytes + h * 16;
     const int base = ld_c * kDecodeChunk;
+    const int piece = base + (lane & 7) * 16;     // this lane's 16 bytes of the chunk's 128
 #pragma unroll
     for (int s = 0; s < kDecodeSteps; ++s) {
-      const int off = base + s * 32;
-      if (live && off + h * 16 < kbytes) {
-        b.w[s] = *reinterpret_cast<const v4i *>(wp + off);
-        if constexpr (!XLDS) b.x[s] = *reinterpret_cast<const v4i *>(xp + off);
-      } else {
-        b.w[s] = v4i{0, 0, 0, 0};
-        if constexpr (!XLDS) b.x[s] = v4i{0, 0, 0, 0};
+      const int n = ld_slab * 32 + 8 * s + (lane >> 3);
+      b.w[s] = v4i{0, 0, 0, 0};
+      if (live && piece < kbytes)
+        b.w[s] = *reinterpret_cast<const v4i *>(p.qw + int64_t(n < p.N ? n : p.N - 1) * kbytes + piece);
+      if constexpr (!XLDS) {
+        b.x[s] = v4i{0, 0, 0, 0};
+        if constexpr (FUSED) {  // whole lines as well (the fused form has a second 4 KB per wave to pass them through)
+          const int m = 8 * s + (lane >> 3);
+          if (live && piece < kbytes)
+            b.x[s] = *reinterpret_cast<const v4i *>(p.qx + int64_t(m < p.M ? m : p.M - 1) * kbytes + piece);
+        } else {
+          const int off = base + s * 32;
+          if (live && off + h * 16 < kbytes) b.x[s] = *reinterpret_cast<const v4i *>(xp + off);
+        }
       }
     }
     ld_c += WAVES;
@@ -160,12 +172,23 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_decode_kernel(FusedArgs args,
   for (int v = 0; v < 16; ++v) acc[v] = 0;
   auto multiply = [&](const Buf &b, int chunk) __attribute__((always_inline)) {
     const uint8_t *xs = x_lds + (chunk < nchunks ? chunk : 0) * kDecodeSteps * x_step;  // (empty items: zero weights)
+    uint8_t *tile = smem + wave * 4096;  // this wave's corner of the reduction area, idle between slab ends
+    constexpr bool kXTile = FUSED && !XLDS;
+    uint8_t *xtile = smem + (WAVES + wave) * 4096;  // (the fp32 half of the reduction area)
+#pragma unroll
+    for (int s = 0; s < kDecodeSteps; ++s) {
+      const int at = s * 1024 + (lane >> 3) * 128 + (((lane & 7) ^ ((4 * s + (lane >> 4)) & 7)) << 4);
+      *reinterpret_cast<v4i *>(tile + at) = b.w[s];
+      if constexpr (kXTile) *reinterpret_cast<v4i *>(xtile + at) = b.x[s];
+    }
 #pragma unroll
     for (int s = 0; s < kDecodeSteps; ++s) {
       v4i wu[FragOps<MODE>::H], xu[FragOps<MODE>::H];
-      FragOps<MODE>::unpack(b.w[s], wu);
+      FragOps<MODE>::unpack(*reinterpret_cast<const v4i *>(tile + r * 128 + (((2 * s + h) ^ ((r >> 1) & 7)) << 4)), wu);
       if constexpr (XLDS) {
         FragOps<MODE>::unpack(*reinterpret_cast<const v4i *>(xs + s * x_step), xu);
+      } else if constexpr (kXTile) {
+        FragOps<MODE>::unpack(*reinterpret_cast<const v4i *>(xtile + r * 128 + (((2 * s + h) ^ ((r >> 1) & 7)) << 4)), xu);
       } else {
         FragOps<MODE>::unpack(b.x[s], xu);
       }

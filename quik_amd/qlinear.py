@@ -74,7 +74,7 @@ class MixedQLinear(torch.nn.Module):
     of the row-major kernels; `six_bit_path = False` turns them off."""
 
     six_bit_min_rows = 33    # up to 32 rows the weight-streaming decode kernel on the packed int4 weights is the right one
-    tile8_min_rows = 17      # 8 bits: with its K split the tile-ordered path passes the weight-streaming kernel at 8 to 18 rows (70B to 7B down_proj)
+    tile8_min_rows = 33      # the same switch for 8 bits (the tile-ordered kernel itself takes any row count)
 
     def __init__(self, in_features, out_features, shared_input=None,
                  fp_features_num=0, symm=False, bits=4, dtype=torch.float16, fused=True):

@@ -1193,19 +1193,23 @@ def test_split_k_gives_the_same_bits(case):
     assert int(ws[:4096].view(torch.int32).abs().sum()) == 0               # counters are back at zero
 
 
-@pytest.mark.parametrize("M", [16, 17, 24, 32])
-def test_int8_layers_switch_to_tile_ordered_operands_at_17_rows(M):
-    """W8A8: from 17 token rows the tile-ordered path (with its K split) is faster than the weight-streaming
-    kernel; below, that kernel runs.  Both against the oracle (their fp32 sums differ in order, so not bit for bit
-    against each other)."""
+@pytest.mark.parametrize("M,tiled", [(16, False), (24, True), (32, False), (32, True), (33, True)])
+def test_int8_layers_around_the_switch_of_paths(M, tiled):
+    """W8A8 at small row counts: up to 32 rows the weight-streaming kernel runs, above it the tile-ordered path
+    (with its K split), which also accepts fewer rows when asked (`tile8_min_rows`).  Both against the oracle
+    (their fp32 sums differ in order, so they are not compared bit for bit with each other)."""
+    from quik_amd.qlinear import MixedQLinear
     N, n_in, F, bits = 520, 4096 + 64, 64, 8
     rng = np.random.default_rng(M)
     W, s_w, ii, fi = _layer(rng, N, n_in, F, bits)
     bias = rng.standard_normal(N).astype(np.float16)
     x = _acts(rng, M, n_in, fi).astype(np.float16)
     mod = _module(W, s_w, fi, bits, bias)
+    assert MixedQLinear.tile8_min_rows == 33
+    if tiled:
+        mod.tile8_min_rows = 1
     out = mod(_t(x))[0].float().cpu().numpy()
-    assert (mod._w6 is not None) == (M >= 17)
+    assert (mod._w6 is not None) == tiled
     omod = qo.from_float(W, s_w, fi, bits)
     want, _ = qo.mixed_qlinear_forward(x, omod, bits, bias)
     rms = np.sqrt((want.astype(np.float64) ** 2).mean())
