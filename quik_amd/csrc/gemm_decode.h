@@ -269,7 +269,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_decode_kernel(FusedArgs args,
   };
 
   // ---- the stream
-  constexpr int NB = 3;
+  constexpr int NB = 3;  // (4 and 6 register sets: slower, they cost occupancy)
   Buf buf[NB];
   int slab = blockIdx.x, c = wave;  // the item being multiplied
   slab_begin(slab);
