@@ -36,7 +36,7 @@ typedef int v8i __attribute__((ext_vector_type(8)));
 // kilobytes of a block unit are copied with one source pointer and one LDS base.
 template <int OFFSET>
 __device__ __forceinline__ void dma_load16k(const uint8_t *sbase, uint32_t voff, uint32_t lds_addr) {
-  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2 offset:%3"
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 offset:%3"
                : : "s"(lds_addr), "v"(voff), "s"(sbase), "n"(OFFSET) : "memory", "m0");
 }
 

@@ -223,8 +223,10 @@ __device__ __forceinline__ void mainloop_plain(const uint8_t *__restrict__ X, in
 // costs scalar adds only and a load is two instructions (s_mov m0, global_load_lds).  Written
 // as inline assembly so that the outstanding-load count stays under this file's control: the
 // loop waits with vmcnt(loads per stage), leaving the newest stage in flight across the barrier.
+// (s_nop 0: one wait state between the scalar write of m0 and the copy that reads it, which the compiler
+// keeps for its own LDS copies on this generation and cannot see inside an asm statement.)
 __device__ __forceinline__ void dma_load16(const uint8_t *sbase, uint32_t voff, uint32_t lds_addr) {
-  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(sbase) : "memory", "m0");
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(sbase) : "memory", "m0");
 }
 
 __device__ __forceinline__ uint32_t lds_address(const void *p) {
