@@ -118,9 +118,11 @@ int launch_decode_w(const FusedArgs &p, int32_t *C, int ldc, hipStream_t st) {
   if (int rc = prepare(kern, smem)) return rc;
   // persistent workgroups: as many as are resident at once (8 waves per CU at this register count; the LDS copy
   // of the token rows leaves room for one workgroup)
+  // Every workgroup walks the same number of slabs (one more or less): with 896 slabs, 224 workgroups of 4 slabs
+  // finish when 256 workgroups of 3 or 4 do, and share the memory system among fewer.
   const int64_t slabs = (p.N + 31) / 32, resident = int64_t(kCUs) * (XLDS ? 1 : 8 / WAVES);
-  hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(slabs < resident ? slabs : resident)), dim3(WAVES * 64), smem, st,
-                     p, C, ldc);
+  const int64_t per = (slabs + resident - 1) / resident, grid = (slabs + per - 1) / per;
+  hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(grid)), dim3(WAVES * 64), smem, st, p, C, ldc);
   return check_launch();
 }
 
