@@ -76,8 +76,12 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_decode_kernel(FusedArgs args,
   constexpr int kFpEarly = FUSED ? 2 : 0;                     // outlier pieces requested at slab start
   using FpOps = FragOps<BF16 ? kBF16 : kF16>;
 
+  // Every load below is issued unconditionally, from a clamped (valid) address, and what must read as zero is
+  // masked when it is used: with loads under a branch the number of loads in flight is unknown at compile time
+  // and every wait becomes a wait for all of them, which empties the prefetch queue before each chunk.
   struct Buf {
     v4i w[kDecodeSteps], x[XLDS ? 1 : kDecodeSteps];
+    int keep;  // all ones: this lane's piece of the chunk exists; zero: empty item or past the row's end
   };
   // ---- XLDS: copy the token rows into LDS, 16-byte unit u = ((chunk step) * 2 + K half) * M + row
   const uint8_t *x_lds = smem + decode_smem<WAVES, FUSED, XLDS>();
@@ -101,21 +105,21 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_decode_kernel(FusedArgs args,
     const bool live = ld_slab < slabs && ld_c < nchunks;
     const int base = ld_c * kDecodeChunk;
     const int piece = base + (lane & 7) * 16;     // this lane's 16 bytes of the chunk's 128
+    const bool ok = live && piece < kbytes;
+    b.keep = ok ? -1 : 0;
+    const int piece_c = ok ? piece : 0;
+    const int slab_c = ld_slab < slabs ? ld_slab : slabs - 1;
 #pragma unroll
     for (int s = 0; s < kDecodeSteps; ++s) {
-      const int n = ld_slab * 32 + 8 * s + (lane >> 3);
-      b.w[s] = v4i{0, 0, 0, 0};
-      if (live && piece < kbytes)
-        b.w[s] = *reinterpret_cast<const v4i *>(p.qw + int64_t(n < p.N ? n : p.N - 1) * kbytes + piece);
+      const int n = slab_c * 32 + 8 * s + (lane >> 3);
+      b.w[s] = *reinterpret_cast<const v4i *>(p.qw + int64_t(n < p.N ? n : p.N - 1) * kbytes + piece_c);
       if constexpr (!XLDS) {
-        b.x[s] = v4i{0, 0, 0, 0};
         if constexpr (FUSED) {  // whole lines as well (the fused form has a second 4 KB per wave to pass them through)
           const int m = 8 * s + (lane >> 3);
-          if (live && piece < kbytes)
-            b.x[s] = *reinterpret_cast<const v4i *>(p.qx + int64_t(m < p.M ? m : p.M - 1) * kbytes + piece);
-        } else {
+          b.x[s] = *reinterpret_cast<const v4i *>(p.qx + int64_t(m < p.M ? m : p.M - 1) * kbytes + piece_c);
+        } else {  // (zero weights stand against whatever is read in place of a missing piece)
           const int off = base + s * 32;
-          if (live && off + h * 16 < kbytes) b.x[s] = *reinterpret_cast<const v4i *>(xp + off);
+          b.x[s] = *reinterpret_cast<const v4i *>(xp + (live && off + h * 16 < kbytes ? off : -h * 16));
         }
       }
     }
@@ -129,7 +133,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_decode_kernel(FusedArgs args,
   // ---- per-slab state requested when the slab starts: outlier pieces and epilogue scalars
   const int fbytes = FUSED ? p.F * 2 : 0;
   v4i fwe[kFpEarly > 0 ? kFpEarly : 1], fxe[kFpEarly > 0 ? kFpEarly : 1];
-  float srow = 0.0f, zs = 0.0f, e_sc[VPW], e_wr[VPW], e_bs[VPW];
+  float srow = 0.0f, zs = 0.0f;
+  uint16_t e_sc[VPW], e_wr[VPW], e_bs[VPW];  // raw: converted where they are used, so that nothing waits here
+  const uint16_t *wr_ptr = p.w_red ? p.w_red : p.s_col, *bs_ptr = p.bias ? p.bias : p.s_col;
   const uint8_t *fx = nullptr;
   if constexpr (FUSED) {
     fx = reinterpret_cast<const uint8_t *>(p.fp_x) + int64_t(mrow) * fbytes + h * 16;
@@ -144,15 +150,14 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_decode_kernel(FusedArgs args,
   auto slab_begin = [&](int slab) __attribute__((always_inline)) {
     if constexpr (FUSED) {
       if (slab >= slabs) return;
-      const uint8_t *fw = fp_row(slab);
+      if (fbytes > 0) {  // (uniform over the launch)
+        const uint8_t *fw = fp_row(slab);
 #pragma unroll
-      for (int i = 0; i < kFpEarly; ++i) {
-        const int off = (wave + i * WAVES) * 32;
-        fwe[i] = v4i{0, 0, 0, 0};
-        fxe[i] = v4i{0, 0, 0, 0};
-        if (off + h * 16 < fbytes) {
-          fwe[i] = *reinterpret_cast<const v4i *>(fw + off);
-          fxe[i] = *reinterpret_cast<const v4i *>(fx + off);
+        for (int i = 0; i < kFpEarly; ++i) {
+          const int off = (wave + i * WAVES) * 32;
+          const int off_c = off + h * 16 < fbytes ? off : -h * 16;  // a missing piece reads the row's start, masked in slab_end
+          fwe[i] = *reinterpret_cast<const v4i *>(fw + off_c);
+          fxe[i] = *reinterpret_cast<const v4i *>(fx + off_c);
         }
       }
 #pragma unroll
@@ -160,9 +165,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_decode_kernel(FusedArgs args,
         const int v = wave * VPW + j;
         const int n = slab * 32 + 8 * (v >> 2) + 4 * h + (v & 3);  // accumulator register v of this lane: see acc_col()
         const int nn = n < p.N ? n : p.N - 1;
-        e_sc[j] = to_f32<BF16>(p.s_col[nn]);
-        e_wr[j] = p.w_red ? to_f32<BF16>(p.w_red[nn]) : 0.0f;
-        e_bs[j] = p.bias ? to_f32<BF16>(p.bias[nn]) : 0.0f;
+        e_sc[j] = p.s_col[nn];
+        e_wr[j] = wr_ptr[nn];
+        e_bs[j] = bs_ptr[nn];
       }
     }
   };
@@ -178,7 +183,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_decode_kernel(FusedArgs args,
 #pragma unroll
     for (int s = 0; s < kDecodeSteps; ++s) {
       const int at = s * 1024 + (lane >> 3) * 128 + (((lane & 7) ^ ((4 * s + (lane >> 4)) & 7)) << 4);
-      *reinterpret_cast<v4i *>(tile + at) = b.w[s];
+      *reinterpret_cast<v4i *>(tile + at) = v4i{b.w[s].x & b.keep, b.w[s].y & b.keep, b.w[s].z & b.keep, b.w[s].w & b.keep};
       if constexpr (kXTile) *reinterpret_cast<v4i *>(xtile + at) = b.x[s];
     }
 #pragma unroll
@@ -207,7 +212,11 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_decode_kernel(FusedArgs args,
     for (int v = 0; v < 16; ++v) accf[v] = 0.0f;
     if constexpr (FUSED) {
 #pragma unroll
-      for (int i = 0; i < kFpEarly; ++i) FpOps::mma(fxe[i], fwe[i], accf);
+      for (int i = 0; i < kFpEarly; ++i) {
+        const int keep = fbytes > 0 && (wave + i * WAVES) * 32 + h * 16 < fbytes ? -1 : 0;
+        if (fbytes > 0)
+          FpOps::mma(fxe[i], v4i{fwe[i].x & keep, fwe[i].y & keep, fwe[i].z & keep, fwe[i].w & keep}, accf);
+      }
       const uint8_t *fw = fp_row(slab);
       for (int off = (wave + kFpEarly * WAVES) * 32; off < fbytes; off += WAVES * 32) {
         v4i wv = v4i{0, 0, 0, 0}, xv = v4i{0, 0, 0, 0};
@@ -259,7 +268,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_decode_kernel(FusedArgs args,
       const int n = slab * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
       if (r >= p.M || n >= p.N) continue;
       if constexpr (FUSED) {
-        const float val = (static_cast<float>(ti) * (srow * e_sc[j]) + tf) + (zs * e_wr[j] + e_bs[j]);
+        const float sc = to_f32<BF16>(e_sc[j]);
+        const float wr = p.w_red ? to_f32<BF16>(e_wr[j]) : 0.0f, bs = p.bias ? to_f32<BF16>(e_bs[j]) : 0.0f;
+        const float val = (static_cast<float>(ti) * (srow * sc) + tf) + (zs * wr + bs);
         p.out[int64_t(r) * p.ldo + n] = from_f32<BF16>(val);
       } else {
         Cm[int64_t(r) * ldc + n] = MODE == kInt4 ? (ti >> 8) : ti;
