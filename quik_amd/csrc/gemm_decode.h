@@ -143,6 +143,16 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_decode_kernel(FusedArgs args,
     zs = p.w_red ? to_f32<BF16>(p.meta[2 * int64_t(mrow) + 1]) + p.shift * srow : 0.0f;
     if constexpr (MODE == kInt4) srow *= 0.00390625f;  // the int4 accumulators carry a factor 256
   }
+  // this wave's outlier pieces of the token rows are the same for every slab: loaded once
+  if constexpr (FUSED) {
+    if (fbytes > 0) {
+#pragma unroll
+      for (int i = 0; i < kFpEarly; ++i) {
+        const int off = (wave + i * WAVES) * 32;
+        fxe[i] = *reinterpret_cast<const v4i *>(fx + (off + h * 16 < fbytes ? off : -h * 16));
+      }
+    }
+  }
   auto fp_row = [&](int slab) __attribute__((always_inline)) {
     const int n = slab * 32 + r;
     return reinterpret_cast<const uint8_t *>(p.fp_w) + int64_t(n < p.N ? n : p.N - 1) * fbytes + h * 16;
@@ -157,7 +167,6 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_decode_kernel(FusedArgs args,
           const int off = (wave + i * WAVES) * 32;
           const int off_c = off + h * 16 < fbytes ? off : -h * 16;  // a missing piece reads the row's start, masked in slab_end
           fwe[i] = *reinterpret_cast<const v4i *>(fw + off_c);
-          fxe[i] = *reinterpret_cast<const v4i *>(fx + off_c);
         }
       }
 #pragma unroll
