@@ -437,6 +437,8 @@ FWD_CASES = [
     (7, 100, 200, 8, 8, True, "student"),
     (32, 8200, 1056, 32, 4, False, "x50"),   # decode kernel: several slabs per workgroup
     (20, 64, 8192 + 520, 520, 8, True, "x50"),  # decode kernel: 8 waves per slab, more outlier pieces than prefetched
+    (9, 8300, 1000, 40, 4, True, "x50"),     # decode kernel, token rows in LDS: last K chunk and last outlier piece cut short
+    (12, 70, 456, 24, 8, False, "student"),  # decode kernel, token rows streamed: the same for int8
 ]
 
 
