@@ -37,9 +37,11 @@ constexpr int kDecodeSteps = kDecodeChunk / 32;
 
 // reduction area: int32 partial sums and, for the fused form, fp32 outlier sums; with XLDS the two share one
 // area (one after the other) to leave room for the token rows
+// behind it, in the fused form: 2 KB in which a slab's 32 x 32 outputs are gathered into whole row segments
+constexpr int kDecodeStage = 2048;
 template <int WAVES, bool FUSED, bool XLDS = false>
 constexpr int decode_smem() {
-  return WAVES * 4096 * (FUSED && !XLDS ? 2 : 1);
+  return WAVES * 4096 * (FUSED && !XLDS ? 2 : 1) + (FUSED ? kDecodeStage : 0);
 }
 // bytes of the LDS copy of `rows` token rows of `kbytes` bytes (whole 1 KB copies)
 inline int64_t decode_x_lds_bytes(int64_t rows, int64_t kbytes) {
@@ -269,23 +271,49 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_decode_kernel(FusedArgs args,
         for (int q = 0; q < WAVES; ++q) tfs[j] += red_f[(q * 16 + wave * VPW + j) * 64 + lane];
       }
     }
+    // Fused form: a lane holds single values of 2-byte outputs, one row each: stored as they are, every store
+    // instruction would touch 32 lines for 128 bytes.  They are gathered in LDS and leave as 16-byte pieces of
+    // row segments (when the output's alignment allows it).
+    uint16_t *stage = reinterpret_cast<uint16_t *>(smem + decode_smem<WAVES, FUSED, XLDS>() - kDecodeStage);
+    const bool staged = FUSED && (p.ldo & 7) == 0 && (reinterpret_cast<uintptr_t>(p.out) & 15) == 0;
 #pragma unroll
     for (int j = 0; j < VPW; ++j) {
       const int v = wave * VPW + j;
       const int32_t ti = tis[j];
       const float tf = tfs[j];
-      const int n = slab * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
-      if (r >= p.M || n >= p.N) continue;
+      const int nl = 8 * (v >> 2) + 4 * h + (v & 3), n = slab * 32 + nl;
       if constexpr (FUSED) {
         const float sc = to_f32<BF16>(e_sc[j]);
         const float wr = p.w_red ? to_f32<BF16>(e_wr[j]) : 0.0f, bs = p.bias ? to_f32<BF16>(e_bs[j]) : 0.0f;
         const float val = (static_cast<float>(ti) * (srow * sc) + tf) + (zs * wr + bs);
-        p.out[int64_t(r) * p.ldo + n] = from_f32<BF16>(val);
+        if (staged) {
+          stage[r * 32 + nl] = from_f32<BF16>(val);
+        } else if (r < p.M && n < p.N) {
+          p.out[int64_t(r) * p.ldo + n] = from_f32<BF16>(val);
+        }
       } else {
-        Cm[int64_t(r) * ldc + n] = MODE == kInt4 ? (ti >> 8) : ti;
+        if (r < p.M && n < p.N) Cm[int64_t(r) * ldc + n] = MODE == kInt4 ? (ti >> 8) : ti;
       }
     }
     __syncthreads();  // the next slab's partial sums reuse the area
+    if constexpr (FUSED) {
+      // (the staging area is written again only behind the next slab's barriers)
+      if (staged && threadIdx.x < 128) {
+        const int row = threadIdx.x >> 2, n0 = slab * 32 + (threadIdx.x & 3) * 8;
+        if (row < p.M && n0 < p.N) {
+          const v4i d = *reinterpret_cast<const v4i *>(stage + row * 32 + (threadIdx.x & 3) * 8);
+          uint16_t *dst = p.out + int64_t(row) * p.ldo + n0;
+          if (n0 + 8 <= p.N) {
+            *reinterpret_cast<v4i *>(dst) = d;
+          } else {
+            const int w[4] = {d.x, d.y, d.z, d.w};
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+              if (n0 + e < p.N) dst[e] = static_cast<uint16_t>(static_cast<uint32_t>(w[e >> 1]) >> (16 * (e & 1)));
+          }
+        }
+      }
+    }
   };
 
   // ---- the stream
