@@ -11,7 +11,9 @@ import torch
 
 from . import _lib as L
 
-__all__ = ["int4FusedDequantize", "int8FusedDequantize", "quantize", "dequantize", "find_meta", "quantizeOld", "build_colmap", "quantize_mapped", "quantize_mapped_fp6", "colmap_streams"]
+__all__ = ["int4FusedDequantize", "int8FusedDequantize", "quantize", "dequantize", "find_meta", "quantizeOld",
+           "build_colmap", "quantize_mapped", "quantize_mapped_fp6", "quantize_mapped_tile8", "colmap_streams",
+           "check_mapped_args"]
 
 
 def _check_bits(bits):
@@ -38,16 +40,43 @@ def build_colmap(int_indices: torch.Tensor, fp_indices: torch.Tensor, cols: int)
     return cm
 
 
-def quantize_mapped(src: torch.Tensor, colmap: torch.Tensor, num_int: int, num_fp: int, bits: int):
-    """quantize() with a prebuilt column map: one kernel launch."""
-    _check_bits(bits)
-    L.check_cuda_contiguous("quantize", src=src, colmap=colmap)
+def check_mapped_args(op: str, src: torch.Tensor, colmap: torch.Tensor, num_int: int, num_fp: int,
+                      need_streaming: bool = False):
+    """Argument checks shared by the ops that take a prebuilt column map; returns (rows, cols).
+
+    The column map must be the blob `build_colmap` made for these (cols, num_int, num_fp): a map of another shape has
+    its sections at other offsets.  need_streaming: the op exists on the streaming kernel only (tile-ordered output,
+    symmetric activations); a map built from int_indices in any other than ascending order is refused here, before
+    anything is launched (checked once per column map, the answer is kept on the tensor)."""
+    L.check_cuda_contiguous(op, src=src, colmap=colmap)
     if src.dim() != 2:
-        raise RuntimeError(f"quantize: expected a 2-D src but got {src.dim()} dimensions")
-    dt = L.dtype_id(src, "quantize", allow_bf16=True)
+        raise RuntimeError(f"{op}: expected a 2-D src but got {src.dim()} dimensions")
     rows, cols = src.shape
     if num_fp + num_int != cols:
         raise RuntimeError("Quantize: number of fp and int columns is not equal to total number of columns")
+    if getattr(colmap, "_quik_shape", None) != (cols, num_int, num_fp):      # first use of this map with this shape
+        if colmap.dtype != torch.uint8:
+            raise RuntimeError(f"{op}: the column map is a uint8 blob from build_colmap, got {colmap.dtype}")
+        if colmap.numel() != L.load().quik_colmap_bytes(cols, num_int, num_fp):
+            raise RuntimeError(f"{op}: the column map was not built for {num_int} integer and {num_fp} outlier "
+                               "columns")
+        colmap._quik_shape = (cols, num_int, num_fp)
+        colmap._quik_streams = None
+    if need_streaming:
+        if colmap._quik_streams is None:
+            colmap._quik_streams = colmap_streams(colmap, num_int, num_fp)
+        if not colmap._quik_streams:
+            raise RuntimeError(f"{op}: this op needs ascending int_indices that partition the columns with fp_indices "
+                               "(and a multiple of 8 columns, at most 32768): the column map does not select the "
+                               "streaming kernel")
+    return rows, cols
+
+
+def quantize_mapped(src: torch.Tensor, colmap: torch.Tensor, num_int: int, num_fp: int, bits: int):
+    """quantize() with a prebuilt column map: one kernel launch."""
+    _check_bits(bits)
+    rows, cols = check_mapped_args("quantize", src, colmap, num_int, num_fp)
+    dt = L.dtype_id(src, "quantize", allow_bf16=True)
     if num_int % 2 != 0:
         raise RuntimeError("Quantize: number of int columns has to be even (implementation detail)")
     lib = L.load()
@@ -77,9 +106,8 @@ def colmap_streams(colmap: torch.Tensor, num_int: int, num_fp: int) -> bool:
 def quantize_mapped_fp6(src: torch.Tensor, colmap: torch.Tensor, num_int: int, num_fp: int):
     """quantize_mapped with bits = 4 whose codes and outlier values go to an operand buffer for
     matmul.mixed_linear_fp6 (internal format, see include/quik_hip.h).  Returns (x6 uint8 buffer, meta)."""
-    L.check_cuda_contiguous("quantize", src=src)
+    rows, cols = check_mapped_args("quantize", src, colmap, num_int, num_fp, need_streaming=True)
     dt = L.dtype_id(src, "quantize", allow_bf16=True)
-    rows, cols = src.shape
     lib = L.load()
     nbytes = lib.quik_fp6_operand_bytes(max(rows, 1), num_int, num_fp)
     if nbytes == 0:
@@ -96,9 +124,8 @@ def quantize_mapped_fp6(src: torch.Tensor, colmap: torch.Tensor, num_int: int, n
 def quantize_mapped_tile8(src: torch.Tensor, colmap: torch.Tensor, num_int: int, num_fp: int):
     """quantize_mapped with bits = 8 whose codes and outlier values go to a tile-ordered operand buffer for
     matmul.mixed_linear_tile8 (internal format, see include/quik_hip.h).  Returns (x8 uint8 buffer, meta)."""
-    L.check_cuda_contiguous("quantize", src=src)
+    rows, cols = check_mapped_args("quantize", src, colmap, num_int, num_fp, need_streaming=True)
     dt = L.dtype_id(src, "quantize", allow_bf16=True)
-    rows, cols = src.shape
     lib = L.load()
     nbytes = lib.quik_tile8_operand_bytes(max(rows, 1), num_int, num_fp)
     if nbytes == 0:

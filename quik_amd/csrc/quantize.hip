@@ -334,8 +334,10 @@ __device__ __forceinline__ void gather_rows(
         drow[p] = static_cast<uint16_t>((v0 | (v1 << 8)) ^ kFlip);
       }
     }
-    uint16_t *frow = fp_x + row * num_fp;
-    for (int64_t f = tid; f < num_fp; f += TPR) frow[f] = row_s[fp_col[f]];
+    if (fp_x != nullptr) {
+      uint16_t *frow = fp_x + row * num_fp;
+      for (int64_t f = tid; f < num_fp; f += TPR) frow[f] = row_s[fp_col[f]];
+    }
     __syncthreads();  // the next row overwrites row_s
   }
 }
@@ -771,6 +773,10 @@ __global__ __launch_bounds__(TPR) void asym_quantize_stream_kernel(
                                           reinterpret_cast<const uint16_t *>(fp_col), num_int, num_fp, dst, meta, fp_x,
                                           codes_s, red, vec_out, &rowsum_s, sym_divisor);
   } else if constexpr (!SYM) {
+    // Tile-ordered output exists on the streaming path only: a column map that does not stream (any other index
+    // order) must not reach the row-major gather code with an operand buffer as `dst` and no `fp_x`.  Nothing is
+    // written then; the host wrappers refuse such a column map before launching.
+    if (vec_out >= 2) return;
     gather_rows<IdxT, BITS, BF16, TPR>(x, rows, cols, src_col, fp_col, mask, num_int, num_fp, dst, meta, fp_x, 1,
                                        row_s, red);
   }

@@ -149,7 +149,13 @@ class MixedQLinear(torch.nn.Module):
         """True if the column map selects the streaming quantize kernel (cached; one synchronisation per map)."""
         colmap = self._column_map()
         if self._streams is None:
-            self._streams = asymmetric.colmap_streams(colmap, self.int_features_num, self.fp_features_num)
+            flag = getattr(colmap, "_quik_streams", None)
+            if flag is None:
+                flag = asymmetric.colmap_streams(colmap, self.int_features_num, self.fp_features_num)
+            # the ops that need the streaming kernel look for the answer on the tensor (asymmetric.check_mapped_args)
+            colmap._quik_shape = (self.in_features, self.int_features_num, self.fp_features_num)
+            colmap._quik_streams = flag
+            self._streams = flag
         return self._streams
 
     def _quantize_input(self, x, shared_input):

@@ -104,11 +104,11 @@ def quantize_mapped(src: torch.Tensor, colmap: torch.Tensor, num_int: int, num_f
     the streaming kernel (asymmetric.colmap_streams).  Returns (q, scale [rows, 1], fp_x) with q / fp_x as
     symmetric.quantize would give them, or, with tiled=True, (operand buffer, scale, None) for
     matmul.mixed_linear_fp6 (bits=4) / matmul.mixed_linear_tile8 (bits=8)."""
-    L.check_cuda_contiguous("quantize", src=src)
+    from .asymmetric import check_mapped_args
     if bits not in (4, 8):
         raise RuntimeError("Unsupported data type")
+    rows, cols = check_mapped_args("quantize", src, colmap, num_int, num_fp, need_streaming=True)
     L.dtype_id(src, "quantize", allow_bf16=False)
-    rows, cols = src.shape
     lib = L.load()
     with L.device_guard(src.device):
         if tiled:

@@ -61,6 +61,41 @@ def test_argument_validation_without_gpu():
     assert lib.quik_mixed_linear_fwd(one, one, null, one, one, one, one, null, 0, 4, 4, 32, 8, 4, one, null) == -5
 
 
+def test_tile_ordered_entry_points_validate_without_gpu():
+    """The entry points that write or read tile-ordered operand buffers reject shapes, alignments and NULL
+    pointers before any HIP call (the column map's streaming flag lives on the device: a map that does not
+    stream makes the kernel write nothing, and the Python wrappers refuse it before launching)."""
+    from quik_amd import _lib as L
+    lib = L.load()
+    null = ctypes.c_void_p(None)
+    one = ctypes.c_void_p(256)  # aligned, never dereferenced
+    odd = ctypes.c_void_p(264)  # 8 mod 256
+    f = ctypes.c_float
+    assert lib.quik_fp6_operand_bytes(2048, 7936, 256) == 32 * (124 + 16) * 3072 + 2048 * 4
+    assert lib.quik_fp6_operand_bytes(2048, 7936 + 64, 256) == 0           # K % 128
+    assert lib.quik_tile8_operand_bytes(2048, 28416, 256) == 32 * (888 + 16) * 2048
+    assert lib.quik_tile8_operand_bytes(2048, 28416, 8) == 0               # F % 32
+    assert lib.quik_asym_quantize_fp6(one, 0, 64, 8192, one, 7936 - 64, 256 + 64, one, one, null) == -4
+    assert lib.quik_asym_quantize_fp6(one, 0, 64, 8192, one, 7936, 256, odd, one, null) == -4
+    assert lib.quik_asym_quantize_fp6(one, 0, 64, 8192, null, 7936, 256, one, one, null) == -5
+    assert lib.quik_asym_quantize_fp6(one, 3, 64, 8192, one, 7936, 256, one, one, null) == -3
+    assert lib.quik_asym_quantize_fp6(one, 0, 64, 8192, one, 7936, 250, one, one, null) == -2
+    assert lib.quik_asym_quantize_fp6(one, 0, 0, 8192, one, 7936, 256, one, one, null) == 0     # empty batch
+    assert lib.quik_asym_quantize_tile8(one, 0, 64, 8192, one, 8192 - 32, 32, one, one, null) == -4   # K % 64
+    assert lib.quik_asym_quantize_tile8(one, 0, 64, 8192, one, 7936, 256, one, null, null) == -5
+    assert lib.quik_sym_quantize_mapped(one, 64, 8192, one, 7936, 256, 5, f(4.0), 1, one, one, null, null) == -1
+    assert lib.quik_sym_quantize_mapped(one, 64, 8192, one, 7936, 256, 4, f(0.0), 1, one, one, null, null) == -2
+    assert lib.quik_sym_quantize_mapped(one, 64, 8190, one, 7934, 256, 4, f(4.0), 0, one, one, one, null) == -2
+    assert lib.quik_sym_quantize_mapped(one, 64, 8192, one, 7936, 256, 4, f(4.0), 0, one, one, null, null) == -5
+    assert lib.quik_sym_quantize_mapped(one, 64, 8192, one, 7936, 256, 4, f(4.0), 1, odd, one, null, null) == -4
+    assert lib.quik_mixed_linear_fwd_fp6(one, one, one, one, one, null, 0, 32, 256, 7936, 256, one, null) == -2  # decode size
+    assert lib.quik_mixed_linear_fwd_fp6(one, odd, one, one, one, null, 0, 64, 256, 7936, 256, one, null) == -4
+    assert lib.quik_mixed_linear_fwd_fp6(one, one, one, one, one, null, 0, 64, 256, 74496 + 128, 256, one, null) == -6
+    assert lib.quik_mixed_linear_fwd_tile8(one, one, null, one, one, null, 0, 64, 256, 28416, 256, one, null) == -5
+    assert lib.quik_splitk_workspace_bytes(64, 8192, 28416, 8) > 4096
+    assert lib.quik_splitk_workspace_bytes(2048, 28672, 7936, 4) == 0
+
+
 def test_python_surface_matches_reference_names():
     """Names and keyword arguments of the pybind module (src/asymmetric/asymmetric.cpp:144-180,
     src/symmetric/symmetric.cpp:120-136, src/matmul/matmul.cpp:85,109 of the reference)."""

@@ -1,0 +1,140 @@
+"""The route MixedQLinear.forward takes by default, at the full sizes of the benchmark configurations.
+
+A module built with `from_float` is called as `mod(x)`, so the dispatch of the module decides the kernels:
+tile-ordered operands on the 6-bit matrix-core GEMM (W4A4) or the tile-ordered int8 GEMM (W8A8) above 32 token
+rows, their K split where the tiles are few, the wide + narrow tile plan in one launch.  Checks per shape:
+  * output bits equal those of the same module on the row-major int8-MFMA kernels (`six_bit_path = False`),
+    which tests/test_gpu_parity.py::test_full_size_properties holds against the oracle at the same shapes
+    through exact row / column checksums of the integer GEMM;
+  * the oracle's MixedQLinear forward (experiments/qlinear.py:80-148 restated on the CPU) on three spot tiles
+    and on the first and last rows, within 1e-2 x output RMS (max abs), the stated tolerance, and within a
+    few fp16 ulps of the largest term in practice.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import quik_oracle as qo
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _lib():
+    from quik_amd import _lib as L
+    L.load()
+    assert torch.cuda.is_available()
+    yield
+
+
+def _bits(t):
+    return t.detach().contiguous().view(torch.int16)
+
+
+def make_full_size_layer(M, n_in, N, F, bits, symm, kind, seed):
+    """Inputs of the measurement protocol, made on the device: x ~ N(0, 1) (or Student-t, 3 degrees of freedom) with
+    the outlier columns scaled up, W = codes x per-row scale on the integer columns, N(0, 0.02) on the outlier
+    columns.  Returns the module (through from_float), x and the float weight matrix / scales / outlier indices."""
+    from quik_amd.qlinear import MixedQLinear
+    g = torch.Generator(device=DEV).manual_seed(seed)
+    x = torch.randn(M, n_in, generator=g, device=DEV)
+    if kind == "student":
+        chi2 = torch.zeros(M, n_in, device=DEV)
+        for _ in range(3):
+            chi2 += torch.randn(M, n_in, generator=g, device=DEV) ** 2
+        x = x / torch.sqrt(chi2 / 3)
+    fi = torch.randperm(n_in, generator=g, device=DEV)[:F]
+    x[:, fi] *= 20 if kind == "student" else 50
+    x = x.clamp(-6e4, 6e4).half()
+    keep = torch.ones(n_in, dtype=torch.bool, device=DEV)
+    keep[fi] = False
+    ii = torch.arange(n_in, device=DEV)[keep]
+    K = n_in - F
+    lo, hi = (-8, 8) if bits == 4 else (-127, 128)
+    s_w = (torch.rand(N, 1, generator=g, device=DEV) * 0.009 + 0.001).half()
+    W = torch.empty(N, n_in, dtype=torch.float16, device=DEV)
+    for s in range(0, N, 4096):
+        e = min(N, s + 4096)
+        codes = torch.randint(lo, hi, (e - s, K), generator=g, device=DEV).float()
+        W[s:e, ii] = (codes * s_w[s:e].float()).half()
+        W[s:e, fi] = (0.02 * torch.randn(e - s, F, generator=g, device=DEV)).half()
+    lin = torch.nn.Linear(n_in, N, bias=False, dtype=torch.float16, device="meta")
+    mod = MixedQLinear.from_float(lin, W, s_w.cpu(), None, fi.cpu(), symm=symm, bits=bits).to(DEV)
+    return mod, x, W, s_w, fi
+
+
+def check_against_oracle(out, x, W, s_w, fi, bits, symm, tiles):
+    """out [M, N] (device) against the oracle's forward on row / column index sets `tiles`."""
+    fin = fi.cpu().numpy()
+    for rows, cols in tiles:
+        omod = qo.from_float(W[cols].cpu().numpy(), s_w[cols].cpu().numpy(), fin, bits, symm=symm)
+        want, _ = qo.mixed_qlinear_forward(x[rows].cpu().numpy(), omod, bits, None, symm=symm)
+        got = out[rows][:, cols].float().cpu().numpy().astype(np.float64)
+        w64 = want.astype(np.float64)
+        assert np.isfinite(w64).all()
+        err = np.abs(got - w64).max()
+        assert err <= 1e-2 * np.sqrt((w64 ** 2).mean()), (err, rows[0], cols[0])
+        assert err <= 4 * np.abs(w64).max() * 2.0 ** -10, (err, rows[0], cols[0])
+
+
+def spot_tiles(M, N):
+    th, tw = min(48, M), min(64, N)
+    r = lambda a: np.arange(a, a + th)
+    c = lambda a: np.arange(a, a + tw)
+    mid_c = min(N - tw, (N // 2 // 256) * 256 + 200)     # straddles a 256-column tile boundary
+    edge = np.r_[0:min(4, M), max(M - 4, 0):M]          # first and last rows ...
+    return [(r(0), c(0)), (r((M - th) // 2), c(mid_c)), (r(M - th), c(N - tw)),
+            (np.unique(edge), np.r_[0:8, N // 2:N // 2 + 8, N - 8:N])]   # ... over the first, middle and last columns
+
+
+DEFAULT_ROUTE = [
+    # tokens, in, out, outliers, bits, symmetric, activations
+    (2048, 8192, 28672, 256, 4, False, "x50"),      # Llama-2-70B gate/up: the benchmark's shape and its tile plan
+    (2048, 8192, 28672, 256, 4, True, "x50"),       # ... symmetric activations
+    (8192, 8192, 28672, 256, 4, False, "x50"),      # ... 16 x 512 tokens, the decoder block's prefill
+    (2048, 28672, 8192, 256, 8, False, "x50"),      # Llama-2-70B down_proj, W8A8
+    (2048, 8192, 8192, 256, 4, False, "x50"),       # Llama-2-70B q/o
+    (2048, 8192, 8192, 256, 4, True, "x50"),        # ... symmetric
+    (2048, 8192, 1024, 256, 4, False, "x50"),       # Llama-2-70B k/v (GQA)
+    (2048, 4096, 11008, 256, 4, False, "x50"),      # Llama-2-7B gate/up
+    (2048, 4096, 4096, 256, 4, False, "x50"),       # Llama-2-7B q/k/v/o
+    (2048, 11008, 4096, 256, 8, False, "x50"),      # Llama-2-7B down_proj, W8A8
+    (2048, 5120, 13824, 256, 4, False, "student"),  # Llama-2-13B gate/up
+    (2048, 13824, 5120, 256, 8, False, "student"),  # Llama-2-13B down_proj, W8A8
+    (128, 5120, 13824, 256, 4, False, "student"),   # Llama-2-13B gate/up, 128 tokens
+    (128, 13824, 5120, 256, 8, False, "student"),   # Llama-2-13B down_proj, 128 tokens: K split
+    (128, 5120, 5120, 256, 4, False, "student"),    # Llama-2-13B q/k/v/o, 128 tokens
+    (64, 28672, 8192, 256, 8, False, "x50"),        # Llama-2-70B down_proj, 64 single-token rows: K split
+]
+
+
+@pytest.mark.parametrize("case", DEFAULT_ROUTE)
+def test_default_route_at_benchmark_shapes(case):
+    M, n_in, N, F, bits, symm, kind = case
+    mod, x, W, s_w, fi = make_full_size_layer(M, n_in, N, F, bits, symm, kind, seed=sum(case[:5]) + symm)
+    assert mod._six_bit_ok(M)                      # the shape is one the tile-ordered path takes
+    out = mod(x)
+    assert mod._w6 is not None                     # ... and it did run
+    assert out.shape == (1, M, N) and out.dtype == torch.float16
+    out = out[0]
+    assert torch.isfinite(out).all()
+    mod.six_bit_path = False
+    mod._w6 = None
+    ref = mod(x)[0]                                # row-major operands, int8 MFMA
+    assert mod._w6 is None
+    assert torch.equal(_bits(out), _bits(ref))
+    del ref
+    check_against_oracle(out, x, W, s_w, fi, bits, symm, spot_tiles(M, N))
+
+
+def test_default_route_three_dimensional_prefill_input():
+    """The decoder block's prefill hands (16, 512, 8192); the module flattens it and returns (16, 512, N)."""
+    M, n_in, N, F, bits = 8192, 8192, 1024, 256, 4
+    mod, x, W, s_w, fi = make_full_size_layer(M, n_in, N, F, bits, False, "x50", seed=5)
+    out = mod(x.reshape(16, 512, n_in))
+    assert out.shape == (16, 512, N)
+    flat = mod(x)[0]
+    assert torch.equal(_bits(out.reshape(M, N)), _bits(flat))
+    check_against_oracle(flat, x, W, s_w, fi, bits, False, spot_tiles(M, N))

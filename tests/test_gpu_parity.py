@@ -1287,3 +1287,45 @@ def test_tile_ordered_paths_random_shapes():
         case = (it, bits, M, N, K, F, dt)
         assert np.array_equal(_bits(meta), _bits(meta2)), case
         assert np.array_equal(_bits(got), _bits(want)), case
+
+
+def test_tile_ordered_ops_refuse_a_column_map_that_does_not_stream():
+    """int_indices in any other than ascending order (which the reference's quantize accepts, and the row-major
+    op serves through the gather kernel) have no tile-ordered form: the wrappers raise before anything is launched,
+    for a wrong-size column map as well, and the row-major op still agrees with the oracle."""
+    import quik
+    from quik_amd import asymmetric, symmetric
+    rng = np.random.default_rng(99)
+    M, n_in, F = 64, 1024 + 64, 64
+    K = n_in - F
+    ii, fi = _split(rng, n_in, F, shuffle=True)
+    x = _acts(rng, M, n_in, fi).astype(np.float16)
+    xt = _t(x)
+    cm = asymmetric.build_colmap(_t(ii), _t(fi), n_in)
+    assert not asymmetric.colmap_streams(cm, K, F)
+    for bits, fn in ((4, asymmetric.quantize_mapped_fp6), (8, asymmetric.quantize_mapped_tile8)):
+        with pytest.raises(RuntimeError, match="streaming kernel"):
+            fn(xt, cm, K, F)
+    for tiled in (False, True):
+        with pytest.raises(RuntimeError, match="streaming kernel"):
+            symmetric.quantize_mapped(xt, cm, K, F, 4, 4.0, tiled)
+    q, meta, fp = asymmetric.quantize_mapped(xt, cm, K, F, 4)          # the gather kernel serves this order
+    dst, m, f = qo.asym_quantize(x, ii, fi, 4)
+    assert np.array_equal(q.cpu().numpy(), dst) and np.array_equal(_bits(fp), f.view(np.uint16))
+    ii2, fi2 = _split(rng, n_in, F)
+    cm_ok = asymmetric.build_colmap(_t(ii2), _t(fi2), n_in)
+    with pytest.raises(RuntimeError, match="column map was not built"):
+        asymmetric.quantize_mapped_fp6(xt[:, :1024 + 32].contiguous(), cm_ok, 1024, 32)
+    with pytest.raises(RuntimeError, match="uint8 blob"):
+        asymmetric.quantize_mapped(xt, cm_ok.view(torch.int8), K, F, 4)
+    with pytest.raises(RuntimeError, match="CUDA"):
+        asymmetric.quantize_mapped_fp6(xt, cm_ok.cpu(), K, F)
+    # the C entry point itself, called with such a map, writes nothing (and does not fault)
+    from quik_amd import _lib as L
+    lib = L.load()
+    nbytes = lib.quik_fp6_operand_bytes(M, K, F)
+    buf = torch.full((nbytes,), 0x5A, dtype=torch.uint8, device=DEV)
+    meta6 = torch.zeros(2 * M, dtype=torch.float16, device=DEV)
+    rc = lib.quik_asym_quantize_fp6(L.ptr(xt), L.QUIK_F16, M, n_in, L.ptr(cm), K, F, L.ptr(buf), L.ptr(meta6), L.stream())
+    torch.cuda.synchronize()
+    assert rc == 0 and bool((buf == 0x5A).all()) and bool((meta6 == 0).all())
