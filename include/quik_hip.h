@@ -7,7 +7,8 @@
  *
  * Each entry point names the interface of the reference it replaces (paths relative to
  * the reference checkout).  The reference returns freshly allocated tensors; here the
- * thin host layer (quik_amd/_ops.py) allocates and this library only fills.
+ * thin host layer (quik_amd/asymmetric.py, symmetric.py, matmul.py) allocates and this
+ * library only fills.
  */
 #ifndef QUIK_HIP_H_
 #define QUIK_HIP_H_
@@ -199,10 +200,13 @@ int quik_mixed_linear_fwd_tile8(const void *x8, const void *w8, const void *meta
  * their exact accumulators through it, and the one that finishes last does the outlier product and
  * the epilogue: same output bits, the weights stream through all CUs.
  * quik_splitk_workspace_bytes: bytes with which the _ws entry points split this shape (0: they do
- * not; bits = 4: the 6-bit path, bits = 8: the int8 path).  The workspace must be zero before its
- * first use (its head holds arrival counters, which every launch leaves at zero again), 16-byte
- * aligned, and must not be shared by launches that may overlap (other streams).  workspace == NULL
- * or too small: no split, as the entry points without _ws. */
+ * not; bits = 4: the 6-bit path, bits = 8: the int8 path).  The first 4096 bytes of the workspace hold
+ * the arrival counters and MUST be zero when a launch starts: zero the workspace before its first use;
+ * every launch that completes leaves the counters at zero again, but after a launch that failed (a
+ * returned QUIK_ERR_LAUNCH, an aborted process that shared the buffer) zero them again before the next
+ * call, otherwise tiles are finished on incomplete sums or never.  The workspace is 16-byte aligned and
+ * must not be shared by launches that may overlap (other streams).  workspace == NULL or too small: no
+ * split, as the entry points without _ws. */
 int64_t quik_splitk_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits);
 int quik_mixed_linear_fwd_fp6_ws(const void *x6, const void *w6, const void *meta, const void *s_col,
                                  const void *w_reduced, const void *bias, int dtype, int64_t M, int64_t N,

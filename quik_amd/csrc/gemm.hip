@@ -1,6 +1,8 @@
 // Host side of the GEMM entry points: argument checks, tile planning, launches.
 // The kernels live in gemm_kernels.h.
+#include <atomic>
 #include <cstdint>
+#include <mutex>
 
 #include "gemm_decode.h"
 #include "gemm_tile8.h"
@@ -19,18 +21,60 @@ using CfgL8 = Cfg<256, 256, 2, 4, 2>;  // 6-bit path, launches of 256x256 tiles 
 using CfgLp = Cfg<256, 256, 2, 2, 0>;  // plain fallbacks
 using CfgMp = Cfg<128, 128, 2, 2, 0>;
 
-constexpr int kCUs = 256;
+constexpr int kMaxCUs = 256;  // MI355X; sizes the static K-split scratch array
+// Compute units of the GPU (all GPUs of a box are the same part: asked once per process; 256 when no device answers,
+// e.g. for the size queries on a machine without a GPU).
+int num_cus() {
+  static const int n = [] {
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) {
+      (void)hipGetLastError();
+      return kMaxCUs;
+    }
+    return cus;
+  }();
+  return n;
+}
 constexpr int kLdsBytes = 160 * 1024;  // per CU, and the most one workgroup may ask for
+
+// Kernels that ask for more than 48 KB of dynamic LDS need the attribute raised once per device; the (kernel,
+// device) pairs already done are remembered, so a launch costs a table look-up, not a runtime call.
+struct PreparedKernels {
+  static constexpr int kSlots = 512;  // open addressing; far more than the instantiations in this file
+  std::atomic<uintptr_t> key[kSlots];
+  bool seen_or_insert(uintptr_t k, bool insert) {
+    for (int i = 0, h = static_cast<int>((k >> 4) % kSlots); i < kSlots; ++i, h = (h + 1) % kSlots) {
+      uintptr_t cur = key[h].load(std::memory_order_acquire);
+      if (cur == k) return true;
+      if (cur == 0) {
+        if (!insert) return false;
+        if (key[h].compare_exchange_strong(cur, k, std::memory_order_acq_rel) || cur == k) return true;
+      }
+    }
+    return false;
+  }
+};
+PreparedKernels g_prepared;
 
 template <typename K>
 int prepare(K kern, int smem) {
   if (smem > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) {
       set_last_hip_error(e);
       return QUIK_ERR_LAUNCH;
     }
+    // kernel entry addresses are at least 16-byte aligned: the low bits carry the device, bit 0 marks a used slot
+    const uintptr_t k = (reinterpret_cast<uintptr_t>(kern) << 8) | (static_cast<uintptr_t>(dev & 0x7F) << 1) | 1u;
+    if (g_prepared.seen_or_insert(k, false)) return QUIK_OK;
+    e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) {
+      set_last_hip_error(e);
+      return QUIK_ERR_LAUNCH;
+    }
+    g_prepared.seen_or_insert(k, true);
   }
   return QUIK_OK;
 }
@@ -60,7 +104,7 @@ SplitGrid split_grid(int64_t M, int64_t n_wide, int64_t n_tail, int &tail_blocks
   g.wide_blocks = grid_of<CW>(M, n_wide, g.tiles_m, g.tiles_n_wide);
   tail_blocks = grid_of<CT>(M, n_tail, g.tiles_m, g.tiles_n_tail);
   int lead = (tail_blocks / 2) & ~7;
-  if (lead > kCUs / 2) lead = kCUs / 2;
+  if (lead > num_cus() / 2) lead = num_cus() / 2;
   g.lead = lead;
   return g;
 }
@@ -108,7 +152,7 @@ int launch_fused_split(const FusedArgs &wide, const FusedArgs &tail, hipStream_t
 // chunks per row; otherwise 4 waves, which lets two workgroups share a CU.
 int decode_waves(int64_t N, int64_t kbytes) {
   const int64_t slabs = (N + 31) / 32, chunks = (kbytes + kDecodeChunk - 1) / kDecodeChunk;
-  return (chunks >= 16 && slabs <= kCUs) ? 8 : 4;
+  return (chunks >= 16 && slabs <= num_cus()) ? 8 : 4;
 }
 
 template <int MODE, bool BF16, bool FUSED, int WAVES, bool XLDS>
@@ -120,7 +164,7 @@ int launch_decode_w(const FusedArgs &p, int32_t *C, int ldc, hipStream_t st) {
   // of the token rows leaves room for one workgroup)
   // Every workgroup walks the same number of slabs (one more or less): with 896 slabs, 224 workgroups of 4 slabs
   // finish when 256 workgroups of 3 or 4 do, and share the memory system among fewer.
-  const int64_t slabs = (p.N + 31) / 32, resident = int64_t(kCUs) * (XLDS ? 1 : 8 / WAVES);
+  const int64_t slabs = (p.N + 31) / 32, resident = int64_t(num_cus()) * (XLDS ? 1 : 8 / WAVES);
   const int64_t per = (slabs + resident - 1) / resident, grid = (slabs + per - 1) / per;
   hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(grid)), dim3(WAVES * 64), smem, st, p, C, ldc);
   return check_launch();
@@ -131,7 +175,7 @@ int launch_decode_w(const FusedArgs &p, int32_t *C, int ldc, hipStream_t st) {
 template <int WAVES, bool FUSED>
 bool decode_x_fits(const FusedArgs &p) {
   return p.M >= 4 && decode_smem<WAVES, FUSED, true>() + decode_x_lds_bytes(p.M, p.kbytes) <= kLdsBytes &&
-         (p.N + 31) / 32 > kCUs;
+         (p.N + 31) / 32 > num_cus();
 }
 
 template <int MODE, bool BF16, bool FUSED>
@@ -153,11 +197,11 @@ struct Plan {
 // relative tile costs in percent of a 256x256 tile (measured)
 constexpr int kCostWide = 100, kCostHalf = 55, kCostMid = 28;
 
-// Makespan of `wide` tiles followed by `half` tiles on kCUs CUs under greedy list scheduling.
+// Makespan of `wide` tiles followed by `half` tiles on the GPU's CUs under greedy list scheduling.
 int64_t makespan(int64_t wide, int64_t half, int cost_half = kCostHalf) {
   // after the wide tiles: `rem` CUs carry one tile more than the others
-  const int64_t full = wide / kCUs, rem = wide % kCUs;
-  int64_t lo_level = full * kCostWide, lo_count = kCUs - rem;  // less loaded CUs
+  const int64_t full = wide / num_cus(), rem = wide % num_cus();
+  int64_t lo_level = full * kCostWide, lo_count = num_cus() - rem;  // less loaded CUs
   int64_t hi_level = lo_level + kCostWide, hi_count = rem;
   // the half tiles go to the least loaded CUs, a whole level at a time
   while (half > 0) {
@@ -199,9 +243,9 @@ int64_t makespan(int64_t wide, int64_t half, int cost_half = kCostHalf) {
 Plan make_plan(int64_t M, int64_t N, bool dma_ok) {
   if (M <= 32) return {Plan::kSmall, 0};
   const int64_t tiles_m = (M + 255) / 256;
-  auto rounds = [](int64_t tiles) { return (tiles + kCUs - 1) / kCUs; };
+  auto rounds = [](int64_t tiles) { return (tiles + num_cus() - 1) / num_cus(); };
   if (!dma_ok) {
-    if (M <= 128 || tiles_m * ((N + 255) / 256) < kCUs / 2) return {Plan::kMidPlain, 0};
+    if (M <= 128 || tiles_m * ((N + 255) / 256) < num_cus() / 2) return {Plan::kMidPlain, 0};
     return {Plan::kLargePlain, 0};
   }
   const int64_t mid = rounds(((M + 127) / 128) * ((N + 127) / 128)) * kCostMid;
@@ -268,8 +312,8 @@ Plan make_plan6(int64_t M, int64_t N, int64_t min_rows = 33) {
   if (M < min_rows) return {Plan::kSmall, 0};
   const int64_t tiles_m = (M + 255) / 256;
   const int64_t mid_tiles = ((M + 127) / 128) * ((N + 127) / 128);
-  const int64_t pairs = mid_tiles / (2 * kCUs), left = mid_tiles % (2 * kCUs);
-  const int64_t mid = pairs * 66 + (left == 0 ? 0 : left <= kCUs ? 36 : 66);
+  const int64_t pairs = mid_tiles / (2 * num_cus()), left = mid_tiles % (2 * num_cus());
+  const int64_t mid = pairs * 66 + (left == 0 ? 0 : left <= num_cus() ? 36 : 66);
   int64_t best = INT64_MAX, best_n = 0;
   for (int64_t n_wide = 0; n_wide <= N + 255; n_wide += 256) {
     const int64_t nw = n_wide < N ? n_wide : N;   // the last candidate: wide tiles only, the last one ragged
@@ -298,8 +342,8 @@ SplitPlan plan_splitk(int64_t M, int64_t N, int64_t steps, int64_t min_steps, in
   SplitPlan none{1, 0, 0};
   if (make_plan6(M, N, min_rows).kind != Plan::kMid) return none;
   const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
-  if (tiles > kCUs / 2 || tiles * 4 > kSplitCounterBytes) return none;
-  for (int64_t splits = kCUs / tiles < 8 ? kCUs / tiles : 8; splits >= min_splits; --splits) {
+  if (tiles > num_cus() / 2 || tiles * 4 > kSplitCounterBytes) return none;
+  for (int64_t splits = num_cus() / tiles < 8 ? num_cus() / tiles : 8; splits >= min_splits; --splits) {
     const int64_t per = ((steps + splits - 1) / splits + 1) / 2 * 2;
     if (per >= min_steps && (splits - 1) * per < steps)
       return {static_cast<int>(splits), static_cast<int>(per), kSplitCounterBytes + tiles * splits * 128 * 128 * 4};
