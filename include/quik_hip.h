@@ -217,6 +217,22 @@ int quik_mixed_linear_fwd_tile8_ws(const void *x8, const void *w8, const void *m
                                    int64_t K, int64_t F, void *out, void *workspace, int64_t workspace_bytes,
                                    void *stream);
 
+/* ---- one entry point that allocates nothing ---------------------------------------------------------
+ * No counterpart in the reference.  For callers that cannot allocate device memory around the call and
+ * have no workspace to hand in: code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc.  It is quik_mixed_linear_fwd_tile8_ws with the K-split workspace (arrival counters
+ * and partial accumulators) in a device array that lives inside the library: 4 KB + 256 x 64 KB = 16 MB
+ * + 4 KB per GPU, held from the first use of the library on that GPU until the process ends.  Same
+ * arguments, same checks and the same output bits as quik_mixed_linear_fwd_tile8_ws with a workspace of
+ * quik_splitk_workspace_bytes(M, N, K, 8) bytes; a shape whose K split would need more than the array
+ * holds returns QUIK_ERR_RANGE.  The call makes no hipMalloc / hipFree: it looks up the array's address
+ * once per device (on the first call there, which should therefore happen outside a graph capture),
+ * clears the counters with a small kernel and launches the GEMM.  All calls on one GPU share the array:
+ * calls that may overlap on that GPU (different streams) race on it and must be serialised by the caller. */
+int quik_mixed_linear_fwd_tile8_noalloc(const void *x8, const void *w8, const void *meta, const void *s_col,
+                                        const void *w_reduced, const void *bias, int dtype, int64_t M,
+                                        int64_t N, int64_t K, int64_t F, void *out, void *stream);
+
 /* quik.matmul.int4Matmul(A, B) -> C int32 [M, N]
  * replaces int4MatmulCUDA, src/matmul/matmul.cu:17-55.
  *   A [M, K/2], B [N, K/2] uint8 nibble-packed, K = number of int4 elements per row.

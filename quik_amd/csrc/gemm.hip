@@ -639,3 +639,75 @@ extern "C" int quik_mixed_linear_fwd_tile8_ws(const void *x8, const void *w8, co
   return dtype == QUIK_F16 ? run_fused8t<false>(p, st, workspace, workspace_bytes)
                            : run_fused8t<true>(p, st, workspace, workspace_bytes);
 }
+
+// ---- the entry point that allocates nothing ------------------------------------------------------------------
+// quik_mixed_linear_fwd_tile8_ws with the K-split workspace in a file-scope device array instead of a caller
+// buffer: counters (kSplitCounterBytes) followed by the partial accumulators, the size of the largest plan
+// plan_splitk makes (tiles x splits <= kMaxCUs workgroups of one 128x128 int32 tile each).  Every GPU that loads this
+// library holds its own copy of the array until the process ends.
+constexpr int64_t kStaticScratchBytes = kSplitCounterBytes + int64_t(kMaxCUs) * 128 * 128 * 4;
+static __device__ __align__(256) uint8_t scratch[kStaticScratchBytes];
+
+namespace quik {
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+std::atomic<uint8_t *> g_scratch_ptr[kMaxDevices];
+
+// Device address of `scratch` on the current device.  In host code the array's name is only a handle for
+// hipGetSymbolAddress: the address is looked up once per device, with that device current, and kept.
+int scratch_of_current_device(uint8_t **out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) {
+    set_last_hip_error(e);
+    return QUIK_ERR_LAUNCH;
+  }
+  if (dev < 0 || dev >= kMaxDevices) return QUIK_ERR_RANGE;
+  uint8_t *p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!p) {
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    p = g_scratch_ptr[dev].load(std::memory_order_relaxed);
+    if (!p) {
+      void *sym = nullptr;
+      e = hipGetSymbolAddress(&sym, HIP_SYMBOL(scratch));
+      if (e != hipSuccess || !sym) {
+        set_last_hip_error(e != hipSuccess ? e : hipErrorInvalidSymbol);
+        return QUIK_ERR_LAUNCH;
+      }
+      p = static_cast<uint8_t *>(sym);
+      g_scratch_ptr[dev].store(p, std::memory_order_release);
+    }
+  }
+  *out = p;
+  return QUIK_OK;
+}
+
+// The arrival counters must be zero when a launch starts.  Launches leave them at zero, but a launch that failed
+// half way would not, and this array outlives every caller: clear them in front of each launch that uses them,
+// with a kernel (a memset node in a captured graph is not reliable on replays).
+__global__ __launch_bounds__(256) void clear_words_kernel(uint32_t *p, int words) {
+  for (int i = blockIdx.x * 256 + threadIdx.x; i < words; i += gridDim.x * 256) p[i] = 0u;
+}
+}  // namespace
+}  // namespace quik
+
+extern "C" int quik_mixed_linear_fwd_tile8_noalloc(const void *x8, const void *w8, const void *meta, const void *s_col,
+                                                   const void *w_reduced, const void *bias, int dtype, int64_t M,
+                                                   int64_t N, int64_t K, int64_t F, void *out, void *stream) {
+  if (dtype != QUIK_F16 && dtype != QUIK_BF16) return QUIK_ERR_DTYPE;
+  if (M < 0 || N < 0 || K <= 0 || F < 0) return QUIK_ERR_SHAPE;
+  if (K % 64 != 0 || F % 32 != 0) return QUIK_ERR_ALIGN;
+  const int64_t need = quik_splitk_workspace_bytes(M, N, K, 8);
+  if (need > kStaticScratchBytes) return QUIK_ERR_RANGE;  // a K split larger than the static array holds
+  if (need == 0 || M == 0 || N == 0)                      // no K split for this shape: no scratch memory involved
+    return quik_mixed_linear_fwd_tile8_ws(x8, w8, meta, s_col, w_reduced, bias, dtype, M, N, K, F, out, nullptr, 0, stream);
+  if (!x8 || !w8 || !meta || !s_col || !out) return QUIK_ERR_NULL;
+  uint8_t *ws = nullptr;
+  if (int rc = scratch_of_current_device(&ws)) return rc;
+  hipLaunchKernelGGL(clear_words_kernel, dim3(static_cast<unsigned>(kSplitCounterBytes / 4 / 256)), dim3(256), 0,
+                     as_stream(stream), reinterpret_cast<uint32_t *>(ws), static_cast<int>(kSplitCounterBytes / 4));
+  if (int rc = check_launch()) return rc;
+  return quik_mixed_linear_fwd_tile8_ws(x8, w8, meta, s_col, w_reduced, bias, dtype, M, N, K, F, out, ws,
+                                        kStaticScratchBytes, stream);
+}
