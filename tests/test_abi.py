@@ -122,6 +122,23 @@ def test_python_surface_matches_reference_names():
                                                         "fp_features_num", "symm", "bits", "dtype"]
 
 
+def test_typed_stubs_describe_the_modules():
+    """quik/_C/*.pyi (the reference ships the same three, quik/_C/{asymmetric,matmul,symmetric}.pyi): every function a
+    stub declares exists in the module with the same parameter names in the same order."""
+    import ast
+    import importlib
+    for name in ("asymmetric", "matmul", "symmetric"):
+        mod = importlib.import_module("quik_amd." + name)
+        tree = ast.parse(open(os.path.join(ROOT, "quik", "_C", name + ".pyi")).read())
+        funcs = [n for n in tree.body if isinstance(n, ast.FunctionDef)]
+        assert len(funcs) >= 2
+        for f in funcs:
+            assert [a.arg for a in f.args.args] == list(inspect.signature(getattr(mod, f.name)).parameters), f.name
+        for public in mod.__all__:
+            if public != "check_mapped_args":
+                assert public in {f.name for f in funcs}, (name, public)
+
+
 def test_ops_reject_cpu_tensors_and_bad_bits():
     import torch
 

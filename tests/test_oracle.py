@@ -106,6 +106,72 @@ def test_asym_quantize_vs_torch_half_formula(bits, heavy):
 
 
 @pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("heavy", [False, True])
+def test_asym_quantize_bf16_vs_torch_bfloat16_formula(bits, heavy):
+    """The bf16 mode of the oracle against torch's CPU bfloat16 kernels, which round every operation to bfloat16
+    (the semantic of __hsub / __hdiv on __nv_bfloat16 and of __bfloat162int_rn, include/util.h:45-110;
+    dispatch src/asymmetric/asymmetric.cu:531-579): scale, zero and every code bit-equal, edge rows included."""
+    rng = _rng(11 + bits)
+    M, n_in, F = 40, 512, 32
+    ii, fi = _split(rng, n_in, F)
+    x32 = _x_with_outliers(rng, M, n_in, fi, heavy).astype(np.float32)
+    x32[0, :] = 1.5                                             # constant row: the scale clamps at 1e-6
+    x32[1, ii[:8]] = [0, 0.5, 1.5, 2.5, 3.5, 4.5, 15, 7.5]      # exact ties
+    x32[2, :] *= 1e-7
+    x32[3, ii[3]], x32[3, ii[4]] = 3e38, -3e38                  # the range overflows fp32: scale = inf
+    x32[4, ii[5]] = np.inf
+    x32[5, ii[6]] = np.nan
+    x32[6, :] = 0.0
+    xb = torch.from_numpy(x32).to(torch.bfloat16)               # round-to-nearest-even, torch's own conversion
+    xs = xb.float().numpy()
+    assert np.array_equal(qo.bf16_round(x32)[~np.isnan(x32)], xs[~np.isnan(x32)])
+    dst, meta, fp_x = qo.asym_quantize(xs, ii, fi, bits, qo.BF16)
+    xi = xb[:, torch.from_numpy(ii)]
+    # torch.max / min propagate NaN where __hmax / __hmin skip it: take them over the non-NaN entries
+    big = torch.tensor(float("inf"), dtype=torch.bfloat16)
+    mx = torch.where(torch.isnan(xi), -big, xi).max(1)[0]
+    mn = torch.where(torch.isnan(xi), big, xi).min(1)[0]
+    scale = torch.clamp((mx.float() - mn.float()) / float(2 ** bits - 1), min=1e-6).to(torch.bfloat16)
+    got_scale = torch.from_numpy(meta[0::2].copy()).to(torch.bfloat16)
+    got_zero = torch.from_numpy(meta[1::2].copy()).to(torch.bfloat16)
+    assert torch.equal(got_scale.view(torch.int16), scale.view(torch.int16))
+    assert torch.equal(got_zero.view(torch.int16), mn.view(torch.int16))
+    assert np.array_equal(meta[0::2], scale.float().numpy())   # the oracle's meta is exactly bf16-representable
+    d = xi - mn[:, None]
+    assert d.dtype == torch.bfloat16
+    t = d / scale[:, None]
+    assert t.dtype == torch.bfloat16
+    r = torch.nan_to_num(t.float().round(), nan=0.0, posinf=2.0 ** 31, neginf=-2.0 ** 31)   # NaN -> 0, as the intrinsic
+    q = torch.clamp(r, 0, 2 ** bits - 1).to(torch.int32) - 2 ** (bits - 1)
+    got = qo.unpack_i4(dst) if bits == 4 else dst
+    assert np.array_equal(got, q.numpy().astype(np.int8))
+    assert np.array_equal(fp_x, xs[:, fi])
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_asym_dequantize_bf16_vs_torch(bits):
+    """asym_dequantize in bf16 mode: fp32 arithmetic in the reference's association order (asymmetric.cu:134-163)
+    evaluated by torch fp32 ops on bfloat16-stored inputs, one rounding to bfloat16 by torch's conversion."""
+    rng = _rng(17 + bits)
+    M, N = 24, 40
+    acc = rng.integers(-3_000_000, 3_000_000, (M, N)).astype(np.int32)
+    acc[0, :4] = [0, 1, -1, 2 ** 24 + 1]
+    bf = lambda a: torch.from_numpy(np.asarray(a, np.float32)).to(torch.bfloat16)
+    meta = bf(np.stack([rng.uniform(1e-3, 0.2, M), rng.standard_normal(M)], 1).reshape(-1))
+    s_col = bf(rng.uniform(1e-3, 1e-2, N))
+    w_red = bf(rng.standard_normal(N) * 3)
+    y = bf(rng.standard_normal((M, N)))
+    got = qo.asym_dequantize(acc, meta.float().numpy(), s_col.float().numpy(), w_red.float().numpy(),
+                             y.float().numpy(), bits, qo.BF16)
+    s, z = meta.float()[0::2][:, None], meta.float()[1::2][:, None]
+    shift = 8.0 if bits == 4 else 128.0
+    t = torch.from_numpy(acc).float() * (s * s_col.float()[None, :])
+    t = t + ((z + shift * s) * w_red.float()[None, :] + y.float())
+    want = t.to(torch.bfloat16)
+    assert np.array_equal(qo.f32_to_bf16_bits(got), want.view(torch.int16).numpy().view(np.uint16))
+
+
+@pytest.mark.parametrize("bits", [4, 8])
 def test_asym_quantize_invariants(bits):
     """test/python/test_quant.py: meta vs torch to 3 places; indexed == gather-then-quantise;
     plus: row minimum -> lowest code, row maximum -> highest code when the scale is not
