@@ -133,9 +133,15 @@ int quik_sym_fused_dequantize(const void *A, const void *B, const void *scale_ro
 int64_t quik_fp6_operand_bytes(int64_t rows, int64_t K, int64_t F);
 
 /* weights [N, K/2] nibble-packed int4 (MixedQLinear.int_weight) and [N, F] fp16/bf16
- * (MixedQLinear.fp_weight, may be NULL when F == 0) -> operand buffer; once per layer */
-int quik_fp6_pack_weight(const uint8_t *qw, const void *fp_w, int64_t N, int64_t K, int64_t F, void *out,
-                         void *stream);
+ * (MixedQLinear.fp_weight, may be NULL when F == 0) -> operand buffer; once per layer.
+ * Along K the operand buffers of this path are in the column map's in-place order (position k = source
+ * column k of the activation, outlier positions filled by the integer columns of the last F source
+ * columns), which lets the quantize kernel write a row without moving data sideways; `colmap` is the
+ * layer's column map (quik_colmap_build for cols = K + F; quik_colmap_streaming(...) must be 1), from
+ * which the weights take the same order.  Buffers packed for one column map must only meet activations
+ * quantized with the same one. */
+int quik_fp6_pack_weight(const uint8_t *qw, const void *fp_w, int64_t N, int64_t K, int64_t F,
+                         const void *colmap, void *out, void *stream);
 
 /* 1 if the column map selects the streaming quantize kernel (ascending int_indices, ...), 0 if not,
  * negative on error; copies one word from the device and synchronises the stream: call once per layer */

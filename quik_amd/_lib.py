@@ -30,7 +30,7 @@ SIGNATURES = {
                                           _vp, _vp, _vp]),
     "quik_sym_fused_dequantize": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp, _vp, _vp]),
     "quik_fp6_operand_bytes": (_i64, [_i64, _i64, _i64]),
-    "quik_fp6_pack_weight": (_int, [_vp, _vp, _i64, _i64, _i64, _vp, _vp]),
+    "quik_fp6_pack_weight": (_int, [_vp, _vp, _i64, _i64, _i64, _vp, _vp, _vp]),
     "quik_colmap_streaming": (_int, [_vp, _i64, _i64, _i64, _vp]),
     "quik_asym_quantize_fp6": (_int, [_vp, _int, _i64, _i64, _vp, _i64, _i64, _vp, _vp, _vp]),
     "quik_mixed_linear_fwd_fp6": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _i64, _vp, _vp]),

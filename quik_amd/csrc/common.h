@@ -11,6 +11,7 @@ namespace quik {
 // Last HIP error text, for quik_last_hip_error().
 void set_last_hip_error(hipError_t e);
 int check_launch();  // QUIK_OK or QUIK_ERR_LAUNCH after a kernel launch
+int num_cus();       // compute units of the GPU (asked once per process; 256 when no device answers)
 
 inline hipStream_t as_stream(void *s) { return reinterpret_cast<hipStream_t>(s); }
 
@@ -99,5 +100,24 @@ __device__ __forceinline__ float wave_min(float v) {
   const float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 48));
   return fminf(fminf(r0, r1), fminf(r2, r3));
 }
+
+// ---- direct global -> LDS copies ---------------------------------------------------------
+// One wave-wide 64 x 16-byte copy global -> LDS: lane i reads 16 bytes at sbase + voff_i and
+// they land at LDS address m0 + 16 i.  sbase (scalar) and m0 are wave-uniform, so advancing K
+// costs scalar adds only and a load is two instructions (s_mov m0, global_load_lds).  Written
+// as inline assembly so that the outstanding-load count stays under this file's control: the
+// loop waits with vmcnt(loads per stage), leaving the newest stage in flight across the barrier.
+// (s_nop 0: one wait state between the scalar write of m0 and the copy that reads it, which the compiler
+// keeps for its own LDS copies on this generation and cannot see inside an asm statement.)
+__device__ __forceinline__ void dma_load16(const uint8_t *sbase, uint32_t voff, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(sbase) : "memory", "m0");
+}
+
+__device__ __forceinline__ uint32_t lds_address(const void *p) {
+  return static_cast<uint32_t>(reinterpret_cast<uintptr_t>((const __attribute__((address_space(3))) void *)p));
+}
+
+// s_waitcnt immediate for "vmcnt <= n", every other counter unconstrained (gfx9 encoding)
+constexpr int vmcnt_imm(int n) { return (n & 0xF) | ((n >> 4) << 14) | 0x0F70; }
 
 }  // namespace quik

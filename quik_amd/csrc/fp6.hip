@@ -1,5 +1,6 @@
 // Weight repacking for the GEMMs that read their operands in tile order (kernels: gemm_fp6.h, gemm_tile8.h;
 // operand formats: fp6_format.h; the activation side is produced by the quantize kernel).
+#include "colmap.h"
 #include "gemm_fp6.h"
 
 namespace quik {
@@ -7,39 +8,44 @@ namespace {
 
 constexpr int kThreads = 256;
 
-// 8 nibbles of a packed int4 dword (two's complement codes) -> two dwords of level bytes
-__device__ __forceinline__ void nibbles_to_level_bytes(uint32_t w, uint32_t &lo, uint32_t &hi) {
-  w ^= 0x88888888u;  // code + 8
-  // element 2i is the low nibble of byte i: bytes (e0 e1 e2 e3) come from nibbles 0..3 = bytes 0, 1 of w
-  const uint32_t even = w & 0x0F0F0F0Fu, odd = (w >> 4) & 0x0F0F0F0Fu;   // e0 e2 e4 e6 / e1 e3 e5 e7
-  lo = __builtin_amdgcn_perm(odd, even, 0x05010400u);   // e0 e1 e2 e3
-  hi = __builtin_amdgcn_perm(odd, even, 0x07030602u);   // e4 e5 e6 e7
-}
-
-// weights [N, K/2] packed int4 and outlier weights [N, F] (16-bit patterns) -> operand buffer; one
-// workgroup per row, one lane per fragment / 16-byte outlier chunk
+// weights [N, K/2] packed int4 (columns in ascending int_indices order) and outlier weights [N, F] (16-bit
+// patterns) -> operand buffer; one workgroup per row, one lane per fragment / 16-byte outlier chunk.
+// Position k of the operand takes weight column kperm[k] (the in-place order of the column map, which the
+// quantize kernel writes the activation in); the row is staged in LDS and gathered nibble by nibble.
 __global__ __launch_bounds__(kThreads) void pack_weight_kernel(const uint8_t *__restrict__ qw,
-                                                               const uint16_t *__restrict__ fp_w, int64_t rows,
+                                                               const uint16_t *__restrict__ fp_w,
+                                                               const uint16_t *__restrict__ kperm,
+                                                               const uint32_t *__restrict__ flags, int64_t rows,
                                                                int64_t K, int64_t F, uint8_t *__restrict__ out) {
+  extern __shared__ __align__(16) uint8_t row_s[];  // K / 2 bytes
+  if (!(flags[0] & 2u)) return;  // the column map has no in-place order (the host refuses such a map first)
   const Fp6Layout l = fp6_layout(rows, K, F);
   const int64_t frags_per_row = l.steps * 2;
   const int64_t row = blockIdx.x;
   for (int64_t c = threadIdx.x; c < F / 8; c += kThreads)
     *reinterpret_cast<uint4 *>(out + fp6_outlier_offset(l, row, c >> 1, static_cast<int>(c & 1))) =
         *reinterpret_cast<const uint4 *>(fp_w + row * F + c * 8);
+  for (int64_t c = threadIdx.x; c < K / 32; c += kThreads)
+    reinterpret_cast<uint4 *>(row_s)[c] = *reinterpret_cast<const uint4 *>(qw + row * (K / 2) + c * 16);
   __shared__ int total;
   if (threadIdx.x == 0) total = 0;
   __syncthreads();
   int sum = 0;
   for (int64_t f = threadIdx.x; f < frags_per_row; f += kThreads) {
-    const uint4 v = *reinterpret_cast<const uint4 *>(qw + row * (K / 2) + f * 16);  // 32 nibbles
     uint32_t b[8];
-    nibbles_to_level_bytes(v.x, b[0], b[1]);
-    nibbles_to_level_bytes(v.y, b[2], b[3]);
-    nibbles_to_level_bytes(v.z, b[4], b[5]);
-    nibbles_to_level_bytes(v.w, b[6], b[7]);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) sum = __builtin_amdgcn_udot4(b[i], 0x01010101u, sum, false);
+    for (int i = 0; i < 8; ++i) {
+      const uint2 kp = *reinterpret_cast<const uint2 *>(kperm + f * 32 + i * 4);  // four positions
+      const uint32_t k[4] = {kp.x & 0xFFFFu, kp.x >> 16, kp.y & 0xFFFFu, kp.y >> 16};
+      uint32_t w = 0;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const uint32_t nib = (row_s[k[e] >> 1] >> ((k[e] & 1u) * 4u)) & 0xFu;  // two's complement code
+        w |= (nib ^ 8u) << (8 * e);                                              // level = code + 8
+      }
+      b[i] = w;
+      sum = __builtin_amdgcn_udot4(w, 0x01010101u, sum, false);
+    }
     uint32_t o[6];
     fp6_pack_fragment(b, o);
     fp6_store_fragment(out, l, row, f, o);
@@ -93,16 +99,20 @@ extern "C" int64_t quik_fp6_operand_bytes(int64_t rows, int64_t K, int64_t F) {
   return fp6_layout(rows, K, F).bytes;
 }
 
-extern "C" int quik_fp6_pack_weight(const uint8_t *qw, const void *fp_w, int64_t N, int64_t K, int64_t F, void *out,
-                                    void *stream) {
+extern "C" int quik_fp6_pack_weight(const uint8_t *qw, const void *fp_w, int64_t N, int64_t K, int64_t F,
+                                    const void *colmap, void *out, void *stream) {
   if (N <= 0 || K <= 0 || F < 0) return QUIK_ERR_SHAPE;
   if (K % 128 != 0 || F % 32 != 0) return QUIK_ERR_ALIGN;
-  if (!qw || !out || (F > 0 && !fp_w)) return QUIK_ERR_NULL;
+  if (!qw || !out || !colmap || (F > 0 && !fp_w)) return QUIK_ERR_NULL;
   if (reinterpret_cast<uintptr_t>(qw) % 16 != 0 || reinterpret_cast<uintptr_t>(out) % 256 != 0 ||
-      reinterpret_cast<uintptr_t>(fp_w) % 16 != 0)
+      reinterpret_cast<uintptr_t>(fp_w) % 16 != 0 || reinterpret_cast<uintptr_t>(colmap) % 16 != 0)
     return QUIK_ERR_ALIGN;
-  if (N > (1 << 30) || K > 74496) return QUIK_ERR_RANGE;
-  hipLaunchKernelGGL(pack_weight_kernel, dim3(static_cast<unsigned>(N)), dim3(kThreads), 0, as_stream(stream), qw,
-                     static_cast<const uint16_t *>(fp_w), N, K, F, static_cast<uint8_t *>(out));
+  if (N > (1 << 30) || K > 74496 || K + F > kStreamMaxCols) return QUIK_ERR_RANGE;
+  const ColmapLayout cl = colmap_layout(K + F, K, F);
+  const uint8_t *cm = static_cast<const uint8_t *>(colmap);
+  hipLaunchKernelGGL(pack_weight_kernel, dim3(static_cast<unsigned>(N)), dim3(kThreads), static_cast<size_t>(K / 2),
+                     as_stream(stream), qw, static_cast<const uint16_t *>(fp_w),
+                     reinterpret_cast<const uint16_t *>(cm + cl.off_kperm),
+                     reinterpret_cast<const uint32_t *>(cm + cl.off_flags), N, K, F, static_cast<uint8_t *>(out));
   return check_launch();
 }

@@ -14,6 +14,9 @@
 //                 different 16-byte bank groups of the 64-bank LDS)
 //   [1024, 2048)  the same for rows 32..63
 //   [2048, 3072)  tails: fragment h of row q (0..63) at 512 h + 8 q
+// Element order along K: the in-place order of the column map (colmap.h): position k holds source column k of
+// the activation, holes (outlier columns) filled by the integer columns of the tail; the weights are packed in
+// the same order (the column map's kperm table), so the order cancels in the products.
 // The outlier columns (fp16 / bf16, 16 per step t, i.e. two 16-byte chunks c per row and step) follow as
 // further units of the same size whose third kilobyte is unused:
 //   [0, 1024) rows 0..31, [1024, 2048) rows 32..63, row r at 32 r, chunk c in slot c ^ ((r >> 3) & 1).
@@ -73,9 +76,12 @@ __host__ __device__ inline int64_t tile8_offset(const Tile8Layout &l, int64_t ro
          ((h ^ ((row >> 3) & 1)) << 4);
 }
 
-// 4 levels in the bytes of w -> 24 bits, 6 per level
+// 4 levels (at most 63 each) in the bytes of w -> 24 bits, 6 per level: two byte dot products with the
+// weights (1, 64) give b0 + 64 b1 and b2 + 64 b3, one shift-or joins them
 __device__ __forceinline__ uint32_t fp6_squeeze4(uint32_t w) {
-  return (w & 0x3Fu) | ((w >> 2) & 0xFC0u) | ((w >> 4) & 0x3F000u) | ((w >> 6) & 0xFC0000u);
+  const uint32_t lo = __builtin_amdgcn_udot4(w, 0x00004001u, 0u, false);
+  const uint32_t hi = __builtin_amdgcn_udot4(w, 0x40010000u, 0u, false);
+  return lo | (hi << 12);
 }
 
 // 32 levels, one per byte of b[0..7] in element order, -> the fragment's 6 dwords (head: 0..3, tail: 4..5)

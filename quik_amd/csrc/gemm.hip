@@ -22,20 +22,6 @@ using CfgLp = Cfg<256, 256, 2, 2, 0>;  // plain fallbacks
 using CfgMp = Cfg<128, 128, 2, 2, 0>;
 
 constexpr int kMaxCUs = 256;  // MI355X; sizes the static K-split scratch array
-// Compute units of the GPU (all GPUs of a box are the same part: asked once per process; 256 when no device answers,
-// e.g. for the size queries on a machine without a GPU).
-int num_cus() {
-  static const int n = [] {
-    int dev = 0, cus = 0;
-    if (hipGetDevice(&dev) != hipSuccess ||
-        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) {
-      (void)hipGetLastError();
-      return kMaxCUs;
-    }
-    return cus;
-  }();
-  return n;
-}
 constexpr int kLdsBytes = 160 * 1024;  // per CU, and the most one workgroup may ask for
 
 // Kernels that ask for more than 48 KB of dynamic LDS need the attribute raised once per device; the (kernel,

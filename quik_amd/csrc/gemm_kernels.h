@@ -218,25 +218,8 @@ __device__ __forceinline__ void mainloop_plain(const uint8_t *__restrict__ X, in
 // wave per SIMD never waits on an LDS round trip.
 // Requires kbytes % 64 == 0: a ragged last stage cannot be zero-filled by the copy engine.
 
-// One wave-wide 64 x 16-byte copy global -> LDS: lane i reads 16 bytes at sbase + voff_i and
-// they land at LDS address m0 + 16 i.  sbase (scalar) and m0 are wave-uniform, so advancing K
-// costs scalar adds only and a load is two instructions (s_mov m0, global_load_lds).  Written
-// as inline assembly so that the outstanding-load count stays under this file's control: the
-// loop waits with vmcnt(loads per stage), leaving the newest stage in flight across the barrier.
-// (s_nop 0: one wait state between the scalar write of m0 and the copy that reads it, which the compiler
-// keeps for its own LDS copies on this generation and cannot see inside an asm statement.)
-__device__ __forceinline__ void dma_load16(const uint8_t *sbase, uint32_t voff, uint32_t lds_addr) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(sbase) : "memory", "m0");
-}
-
-__device__ __forceinline__ uint32_t lds_address(const void *p) {
-  return static_cast<uint32_t>(reinterpret_cast<uintptr_t>((const __attribute__((address_space(3))) void *)p));
-}
-
 __device__ __forceinline__ int swizzle_f(int r) { return (((r >> 1) ^ (r >> 3)) & 1) | (((r >> 2) & 1) << 1); }
 
-// s_waitcnt immediate for "vmcnt <= n", every other counter unconstrained (gfx9 encoding)
-constexpr int vmcnt_imm(int n) { return (n & 0xF) | ((n >> 4) << 14) | 0x0F70; }
 
 // The pipe streams up to two operand sets back to back through the same LDS ring: set 0 is the
 // integer GEMM (qx, qw), set 1 the outlier GEMM (fp_x, fp_w).  Stages are numbered across both,

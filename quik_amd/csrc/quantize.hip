@@ -26,6 +26,7 @@
 // 1e-20 (bf16 only), take the plain IEEE division instead.
 #include <type_traits>
 
+#include "colmap.h"
 #include "common.h"
 #include "fp6_format.h"
 
@@ -33,51 +34,6 @@ namespace quik {
 namespace {
 
 constexpr int kThreads = 256;
-
-// ---------------------------------------------------------------------------------------
-// column map layout: [src_col: num_int idx][fp_col: num_fp idx][mask: ceil(cols/32) u32]
-//                    [grp: ceil(cols/8) u32][dirty: min(num_fp, ceil(cols/8)) u32][dirty_grp: same count, u16]
-//                    [flags: 4 u32]
-// idx is uint16_t when cols <= 65536, else uint32_t.  Section offsets are 16-byte aligned.
-// A "group" is 8 consecutive source columns (one 16-byte load).  A group without outliers is
-// clean, one with outliers is dirty; dirty groups are numbered in ascending order (slots).
-//   grp[g]   clean: (destination column of the group's first element) << 8
-//            dirty: (slot << 8) | mask byte (bit e set = column 8g+e is an outlier)
-//   dirty[s] (destination column of the group's first non-outlier element) << 8 | mask byte
-//   dirty_grp[s] the group index of dirty group s
-//   flags[0] bit 0: int_indices ascending, the two lists partition the columns and the shape
-//            fits the streaming kernel;  flags[1] = number of dirty groups.
-// grp, dirty and dirty_grp exist only when cols <= kStreamMaxCols.
-struct ColmapLayout {
-  bool idx16;
-  int64_t off_fp, off_mask, off_grp, off_dirty, off_slot, off_flags, bytes;
-};
-
-__host__ __device__ inline int64_t align16(int64_t v) { return (v + 15) & ~int64_t(15); }
-
-// Streaming (source-order) quantisation needs ascending int_indices, whole 16-byte chunks and at
-// most kStreamMaxCols columns (16 chunks per thread held in registers).
-constexpr int64_t kStreamMaxCols = 32768;
-
-__host__ __device__ inline int64_t max_dirty_groups(int64_t cols, int64_t num_fp) {
-  const int64_t groups = (cols + 7) / 8;
-  return num_fp < groups ? num_fp : groups;
-}
-
-__host__ __device__ inline ColmapLayout colmap_layout(int64_t cols, int64_t num_int, int64_t num_fp) {
-  ColmapLayout l;
-  l.idx16 = cols <= 65536;
-  const int64_t isz = l.idx16 ? 2 : 4;
-  l.off_fp = align16(num_int * isz);
-  l.off_mask = l.off_fp + align16(num_fp * isz);
-  l.off_grp = l.off_mask + align16(((cols + 31) / 32) * 4);
-  const bool stream = cols <= kStreamMaxCols;
-  l.off_dirty = l.off_grp + align16(stream ? ((cols + 7) / 8) * 4 : 0);
-  l.off_slot = l.off_dirty + align16(stream ? max_dirty_groups(cols, num_fp) * 4 : 0);
-  l.off_flags = l.off_slot + align16(stream ? max_dirty_groups(cols, num_fp) * 2 : 0);
-  l.bytes = l.off_flags + 16;
-  return l;
-}
 
 // number of non-zero bytes among the low `nbytes` bytes of w
 __device__ __forceinline__ uint32_t nonzero_bytes(uint32_t w, int nbytes) {
@@ -93,9 +49,11 @@ __global__ __launch_bounds__(1024) void colmap_build_kernel(const int64_t *__res
                                                             IdxT *__restrict__ fp_col, uint32_t *__restrict__ mask,
                                                             uint32_t *__restrict__ grp, uint32_t *__restrict__ dirty,
                                                             uint16_t *__restrict__ dirty_grp,
+                                                            uint16_t *__restrict__ kperm, uint32_t *__restrict__ patch,
                                                             uint32_t *__restrict__ flags) {
   // single workgroup: the mask is cleared before any bit is set
   __shared__ int ascending;
+  __shared__ uint32_t prefix[kStreamMaxCols / 32 + 1];  // outliers in columns [0, 32 w)
   if (threadIdx.x == 0) ascending = 1;
   const int64_t words = (cols + 31) / 32;
   for (int64_t i = threadIdx.x; i < words; i += blockDim.x) mask[i] = 0u;
@@ -122,9 +80,47 @@ __global__ __launch_bounds__(1024) void colmap_build_kernel(const int64_t *__res
       total += __popc(mask[w]);
       total_dirty += nonzero_bytes(mask[w], 4);
     }
-    flags[0] = (ascending && stream_shape && total == num_fp) ? 1u : 0u;
+    const bool streams = ascending && stream_shape && total == num_fp;
+    const bool in_place = streams && num_int % 32 == 0 && num_fp % 32 == 0;
+    flags[0] = (streams ? 1u : 0u) | (in_place ? 2u : 0u);
     flags[1] = total_dirty;
     flags[2] = flags[3] = 0u;
+    if (cols <= kStreamMaxCols) {
+      uint32_t run = 0;
+      for (int64_t w = 0; w < words; ++w) {
+        prefix[w] = run;
+        run += __popc(mask[w]);
+      }
+      prefix[words] = run;
+    }
+  }
+  __syncthreads();
+  if (cols <= kStreamMaxCols && (flags[0] & 2u)) {
+    // outliers in columns [0, c)
+    auto before = [&](int64_t c) {
+      return prefix[c >> 5] + ((c & 31) ? __popc(mask[c >> 5] & ((1u << (c & 31)) - 1u)) : 0);
+    };
+    auto is_outlier = [&](int64_t c) { return (mask[c >> 5] >> (c & 31)) & 1u; };
+    const uint32_t holes = before(num_int);   // = integer columns in the tail
+    if (threadIdx.x == 0) flags[2] = holes;
+    uint16_t *hole_col = reinterpret_cast<uint16_t *>(patch), *filler_col = hole_col + 1;  // interleaved halves
+    for (int64_t c = threadIdx.x; c < cols; c += blockDim.x) {
+      const uint32_t ob = before(c);
+      if (c < num_int) {
+        if (is_outlier(c)) {
+          hole_col[2 * ob] = static_cast<uint16_t>(c);
+        } else {
+          kperm[c] = static_cast<uint16_t>(c - ob);
+        }
+      } else if (!is_outlier(c)) {
+        filler_col[2 * ((c - num_int) - (ob - holes))] = static_cast<uint16_t>(c);
+      }
+    }
+    __syncthreads();
+    for (int64_t i = threadIdx.x; i < holes; i += blockDim.x) {
+      const int64_t f = filler_col[2 * i];
+      kperm[hole_col[2 * i]] = static_cast<uint16_t>(f - before(f));
+    }
   }
   if (cols <= kStreamMaxCols) {
     const int64_t groups = (cols + 7) / 8;
@@ -452,14 +448,13 @@ __device__ __forceinline__ void stream_rows(const uint16_t *__restrict__ x, int6
                                             const uint16_t *__restrict__ fp_col, int64_t num_int, int64_t num_fp,
                                             uint8_t *__restrict__ dst, uint16_t *__restrict__ meta,
                                             uint16_t *__restrict__ fp_x, uint8_t *codes_s, float *red, int vec_out,
-                                            int *rowsum_s, float sym_divisor = 1.0f) {
-  // vec_out: 0 byte-wise output, 1 16-byte output, 2 (4 bits only): dst is a 6-bit operand buffer
-  // (fp6_format.h) for the matrix-core path of gemm_fp6.h, which also takes the outlier values (fp_x is
-  // not written); needs num_int % 128 == 0 and num_fp % 32 == 0
-  // 3 (8 bits only): dst is an int8 operand buffer in tile order for gemm_tile8.h (same conditions)
-  const Fp6Layout l6 = fp6_layout(rows, num_int, num_fp);
+                                            float sym_divisor = 1.0f) {
+  // vec_out: 0 byte-wise output, 1 16-byte output,
+  // 3 (8 bits only): dst is an int8 operand buffer in tile order for gemm_tile8.h, which also takes the outlier
+  // values (fp_x is not written); needs num_int % 64 == 0 and num_fp % 32 == 0
+  // (the 6-bit operand buffers of gemm_fp6.h are written by quantize_fp6_wave_kernel below)
   const Tile8Layout l8 = tile8_layout(rows, num_int, num_fp);
-  const bool to6 = BITS == 4 && vec_out == 2, to8 = BITS == 8 && vec_out == 3;
+  const bool to8 = BITS == 8 && vec_out == 3;
   const int tid = threadIdx.x;
   const int nvec = static_cast<int>(cols >> 3);
   const float inf = __builtin_inff();
@@ -578,8 +573,6 @@ __device__ __forceinline__ void stream_rows(const uint16_t *__restrict__ x, int6
     }
     // ---- outliers, in the caller's order
     auto fp_slot = [&](int64_t f) -> uint16_t * {
-      if (to6)
-        return reinterpret_cast<uint16_t *>(dst + fp6_outlier_offset(l6, row, f >> 4, static_cast<int>((f >> 3) & 1))) + (f & 7);
       if (to8)
         return reinterpret_cast<uint16_t *>(dst + tile8_offset(l8, row, l8.steps + (f >> 4), static_cast<int>((f >> 3) & 1))) + (f & 7);
       return fp_x + row * num_fp + f;
@@ -656,33 +649,7 @@ __device__ __forceinline__ void stream_rows(const uint16_t *__restrict__ x, int6
     }
     __syncthreads();
 
-    // ---- pack pass: 16 code bytes per lane -> 8 bytes (int4) or 16 bytes (int8), or 32 code bytes -> one
-    // 24-byte fragment of 6-bit levels
-    if (to6) {
-      const int frags = static_cast<int>(num_int >> 5);
-      int sum = 0;
-      for (int f = tid; f < frags; f += TPR) {
-        const uint4 c0 = *reinterpret_cast<const uint4 *>(codes_s + f * 32);
-        const uint4 c1 = *reinterpret_cast<const uint4 *>(codes_s + f * 32 + 16);
-        // code nibble (two's complement) -> level = code + 8
-        const uint32_t b[8] = {c0.x ^ 0x08080808u, c0.y ^ 0x08080808u, c0.z ^ 0x08080808u, c0.w ^ 0x08080808u,
-                               c1.x ^ 0x08080808u, c1.y ^ 0x08080808u, c1.z ^ 0x08080808u, c1.w ^ 0x08080808u};
-#pragma unroll
-        for (int i = 0; i < 8; ++i) sum = __builtin_amdgcn_udot4(b[i], 0x01010101u, sum, false);
-        uint32_t o[6];
-        fp6_pack_fragment(b, o);
-        fp6_store_fragment(dst, l6, row, f, o);
-      }
-#pragma unroll
-      for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
-      if ((tid & 63) == 0) atomicAdd(rowsum_s, sum);
-      __syncthreads();
-      if (tid == 0) {
-        reinterpret_cast<int32_t *>(dst + l6.sums_off)[row] = *rowsum_s;
-        *rowsum_s = 0;   // for the next row of this workgroup (ordered by that row's barriers)
-      }
-      return;
-    }
+    // ---- pack pass: 16 code bytes per lane -> 8 bytes (int4) or 16 bytes (int8)
     const int units = static_cast<int>((num_int + 15) >> 4);
     for (int u = tid; u < units; u += TPR) {
       const uint4 c = *reinterpret_cast<const uint4 *>(codes_s + u * 16);
@@ -720,10 +687,10 @@ __device__ __forceinline__ void stream_rows(const uint16_t *__restrict__ x, int6
   // Workgroups are dealt round-robin to the 8 XCDs, so workgroup w takes row (w % 8) * rows / 8 + w / 8: rows
   // that share lines then run at about the same time on the same XCD and meet in its L2.
   const int64_t per_xcd = (rows + 7) >> 3;
-  const int64_t items = (to6 || to8) ? per_xcd * 8 : rows;
+  const int64_t items = to8 ? per_xcd * 8 : rows;
   int parity = 0;
   for (int64_t w = blockIdx.x; w < items; w += gridDim.x) {
-    const int64_t row = (to6 || to8) ? (w & 7) * per_xcd + (w >> 3) : w;
+    const int64_t row = to8 ? (w & 7) * per_xcd + (w >> 3) : w;
     if (row >= rows) continue;
     parity ^= 1;
     uint4 cur[NV], dv[ND];
@@ -765,13 +732,11 @@ __global__ __launch_bounds__(TPR) void asym_quantize_stream_kernel(
   static_assert(sizeof(IdxT) == 2, "streaming needs cols <= 32768");
   extern __shared__ __align__(16) uint16_t row_s[];
   __shared__ float red[16];
-  __shared__ int rowsum_s;
-  if (threadIdx.x == 0) rowsum_s = 0;
   if (flags[0] & 1u) {
     uint8_t *codes_s = reinterpret_cast<uint8_t *>(row_s);
     stream_rows<BITS, BF16, NV, TPR, SYM>(x, rows, cols, grp, dirty, dirty_grp, static_cast<int>(flags[1]),
                                           reinterpret_cast<const uint16_t *>(fp_col), num_int, num_fp, dst, meta, fp_x,
-                                          codes_s, red, vec_out, &rowsum_s, sym_divisor);
+                                          codes_s, red, vec_out, sym_divisor);
   } else if constexpr (!SYM) {
     // Tile-ordered output exists on the streaming path only: a column map that does not stream (any other index
     // order) must not reach the row-major gather code with an operand buffer as `dst` and no `fp_x`.  Nothing is
@@ -779,6 +744,230 @@ __global__ __launch_bounds__(TPR) void asym_quantize_stream_kernel(
     if (vec_out >= 2) return;
     gather_rows<IdxT, BITS, BF16, TPR>(x, rows, cols, src_col, fp_col, mask, num_int, num_fp, dst, meta, fp_x, 1,
                                        row_s, red);
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// 6-bit operand buffers (consumer: gemm_fp6.h), written in the in-place order of the column map.
+//
+// One wave per row.  The wave copies the row global -> LDS with 16-byte-per-lane direct copies (no
+// registers are held while the row is in flight), in the order its lanes read it back: 16-byte slot
+// (4 j + i) * 64 + L of the row image holds source group 4 (L + 64 j) + i, i.e. lane L owns the
+// fragments (32 consecutive source columns each) L, L + 64, ..., and every LDS read of the wave covers
+// 64 consecutive slots.  In the image the holes (outlier columns among the first num_int columns) are
+// overwritten with their fillers (integer columns of the tail), two-byte LDS copies with row-invariant
+// addresses held in registers; after that the first num_int columns ARE the integer operand, in place:
+// one pass over the image for min / max, a second one that turns each fragment into 32 levels, packs
+// them to 24 bytes in registers and stores head and tail.  No barrier, no cross-wave reduction (a wave's
+// LDS operations execute in order), no data moved between lanes except the two reductions.
+// A workgroup (= wave) walks over rows w, w + grid, ...; with JT > 0 (fragments per lane known at
+// compile time, rows up to 10240 columns) the image is double-buffered and the next row's copy is in
+// flight while the current row is processed; the first two rows of a wave are requested back to back,
+// so across the chip the first rows' requests queue ahead of the second rows' and arrive first.
+template <bool BF16, bool SYM, int JT>
+__global__ __launch_bounds__(64) void quantize_fp6_wave_kernel(
+    const uint16_t *__restrict__ x, int64_t rows, int cols, const uint32_t *__restrict__ patch,
+    const uint16_t *__restrict__ fp_col, const uint32_t *__restrict__ flags, int num_int, int num_fp,
+    uint8_t *__restrict__ dst, uint16_t *__restrict__ meta, float sym_divisor) {
+  static_assert(!(BF16 && SYM), "symmetric activations are fp16");
+  extern __shared__ __align__(16) uint8_t row_img[];
+  if (!(flags[0] & 2u)) return;  // the column map has no in-place order: nothing is written (the host refuses first)
+  const int lane = threadIdx.x;
+  const int frags_all = cols >> 5, frags = num_int >> 5, nchunk = num_fp >> 3;
+  const int J = JT > 0 ? JT : (frags_all + 63) >> 6;
+  const uint32_t img_bytes = static_cast<uint32_t>(J) * 4096u;
+  constexpr int NBUF = JT > 0 ? 2 : 1;
+  const int nholes = static_cast<int>(flags[2]);
+  const Fp6Layout l6 = fp6_layout(rows, num_int, num_fp);
+  const uint32_t lds0 = lds_address(row_img);
+
+  // byte offset of source column c inside a row image
+  auto img_of_col = [](uint32_t c) -> uint32_t {
+    const uint32_t g = c >> 3, f = g >> 2, i = g & 3u;
+    return ((((f >> 6) * 4u + i) * 64u + (f & 63u)) << 4) + ((c & 7u) << 1);
+  };
+  // row-invariant addresses in registers: this lane's first four patches and its first chunk of 8 outliers
+  constexpr int PREG = 4;
+  uint32_t p_hole[PREG], p_fill[PREG], o_addr[8];
+#pragma unroll
+  for (int k = 0; k < PREG; ++k) {
+    const uint32_t e = (lane + 64 * k) < nholes ? patch[lane + 64 * k] : 0u;
+    p_hole[k] = img_of_col(e & 0xFFFFu);
+    p_fill[k] = img_of_col(e >> 16);
+  }
+#pragma unroll
+  for (int k = 0; k < 8; ++k) o_addr[k] = lane < nchunk ? img_of_col(fp_col[lane * 8 + k]) : 0u;
+
+  // body(j) for this lane's fragment slots j = 0 .. J-1, unrolled when their number is known at compile time
+  auto for_j = [&](auto body) {
+    if constexpr (JT > 0) {
+#pragma unroll
+      for (int j = 0; j < JT; ++j) body(j);
+    } else {
+      for (int j = 0; j < J; ++j) body(j);
+    }
+  };
+  auto issue = [&](int64_t row, uint32_t buf) {
+    const uint64_t a = reinterpret_cast<uint64_t>(x + row * cols);
+    // (the intrinsic returns int: each half goes through uint32_t, or the low half would be sign-extended)
+    const uint32_t a_hi = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(a >> 32)));
+    const uint32_t a_lo = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(a & 0xFFFFFFFFu)));
+    const uint8_t *rp = reinterpret_cast<const uint8_t *>((static_cast<uint64_t>(a_hi) << 32) | a_lo);
+    for_j([&](int j) {
+      const int f = lane + 64 * j < frags_all ? lane + 64 * j : frags_all - 1;  // past the row: any valid fragment
+      const uint32_t voff = static_cast<uint32_t>(f) * 64u;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) dma_load16(rp + i * 16, voff, lds0 + buf + (4 * j + i) * 1024);
+    });
+  };
+
+  auto process = [&](int64_t row, uint8_t *img) {
+    auto ld16 = [&](uint32_t off) { return *reinterpret_cast<const uint16_t *>(img + off); };
+    // ---- outlier values, 8 per lane, to the outlier units of the operand buffer (before the holes are patched:
+    // holes are outlier columns)
+    if (lane < nchunk) {
+      uint4 o;
+      o.x = ld16(o_addr[0]) | (static_cast<uint32_t>(ld16(o_addr[1])) << 16);
+      o.y = ld16(o_addr[2]) | (static_cast<uint32_t>(ld16(o_addr[3])) << 16);
+      o.z = ld16(o_addr[4]) | (static_cast<uint32_t>(ld16(o_addr[5])) << 16);
+      o.w = ld16(o_addr[6]) | (static_cast<uint32_t>(ld16(o_addr[7])) << 16);
+      *reinterpret_cast<uint4 *>(dst + fp6_outlier_offset(l6, row, lane >> 1, lane & 1)) = o;
+    }
+    for (int c = lane + 64; c < nchunk; c += 64) {
+      uint32_t w[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+        w[k] = ld16(img_of_col(fp_col[c * 8 + 2 * k])) |
+               (static_cast<uint32_t>(ld16(img_of_col(fp_col[c * 8 + 2 * k + 1]))) << 16);
+      *reinterpret_cast<uint4 *>(dst + fp6_outlier_offset(l6, row, c >> 1, c & 1)) = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+    // ---- holes <- fillers
+#pragma unroll
+    for (int k = 0; k < PREG; ++k)
+      if (lane + 64 * k < nholes) *reinterpret_cast<uint16_t *>(img + p_hole[k]) = ld16(p_fill[k]);
+    for (int e = lane + 64 * PREG; e < nholes; e += 64) {
+      const uint32_t pe = patch[e];
+      *reinterpret_cast<uint16_t *>(img + img_of_col(pe & 0xFFFFu)) = ld16(img_of_col(pe >> 16));
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");  // other lanes read the patched halves below
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+    auto load_fragment = [&](int j, uint4 (&v)[4]) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] = *reinterpret_cast<const uint4 *>(img + (((4 * j + i) * 64 + lane) << 4));
+    };
+    // ---- pass 1: min / max (symmetric: largest |x| pattern) over this lane's fragments
+    const float inf = __builtin_inff();
+    float mn = inf, mx = -inf;
+    const h2 pinf = h2{static_cast<_Float16>(inf), static_cast<_Float16>(inf)};
+    h2 pmn = pinf, pmx = -pinf;
+    u2 amax = u2{0, 0};
+    for_j([&](int j) {
+      if (lane + 64 * j < frags) {
+        uint4 v[4];
+        load_fragment(j, v);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const uint32_t w[4] = {v[i].x, v[i].y, v[i].z, v[i].w};
+          if constexpr (SYM) {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) amax = __builtin_elementwise_max(amax, __builtin_bit_cast(u2, w[k] & 0x7FFF7FFFu));
+          } else if constexpr (!BF16) {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+              pmn = __builtin_elementwise_min(pmn, __builtin_bit_cast(h2, w[k]));
+              pmx = __builtin_elementwise_max(pmx, __builtin_bit_cast(h2, w[k]));
+            }
+          } else {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+              const float f0 = __uint_as_float(w[k] << 16), f1 = __uint_as_float(w[k] & 0xFFFF0000u);
+              mn = fminf(mn, fminf(f0, f1));
+              mx = fmaxf(mx, fmaxf(f0, f1));
+            }
+          }
+        }
+      }
+    });
+    if constexpr (SYM) {
+      mn = 0.0f;
+      mx = static_cast<float>(amax.x > amax.y ? amax.x : amax.y);  // a 15-bit integer: exact, ordered like the patterns
+    } else if constexpr (!BF16) {
+      mn = fminf(static_cast<float>(pmn.x), static_cast<float>(pmn.y));
+      mx = fmaxf(static_cast<float>(pmx.x), static_cast<float>(pmx.y));
+    }
+    mn = wave_min(mn);
+    mx = wave_max(mx);
+    RowQuant<BF16> rq;
+    if constexpr (SYM) {
+      rq.init_sym(static_cast<uint32_t>(mx), sym_divisor);
+      if (lane == 0) meta[row] = rq.scale_bits;
+    } else {
+      rq.init(mn, mx, 4);
+      if (lane == 0) {
+        meta[2 * row] = rq.scale_bits;
+        meta[2 * row + 1] = rq.zero_bits;
+      }
+    }
+    // ---- pass 2: fragment -> 32 levels -> 24 bytes
+    int sum = 0;
+    auto quantise = [&](auto slow_c) {
+      constexpr bool SLOW = decltype(slow_c)::value;
+      for_j([&](int j) {
+        const int f = lane + 64 * j;
+        if (f < frags) {
+          uint4 v[4];
+          load_fragment(j, v);
+          uint32_t b[8];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const uint2 c = group_codes<4, BF16, SLOW, SYM>(v[i], rq);  // code nibbles (two's complement), one per byte
+            b[2 * i] = c.x ^ 0x08080808u;                               // level = code + 8
+            b[2 * i + 1] = c.y ^ 0x08080808u;
+          }
+#pragma unroll
+          for (int i = 0; i < 8; ++i) sum = __builtin_amdgcn_udot4(b[i], 0x01010101u, sum, false);
+          uint32_t o[6];
+          fp6_pack_fragment(b, o);
+          fp6_store_fragment(dst, l6, row, f, o);
+        }
+      });
+    };
+    if (__builtin_amdgcn_readfirstlane(rq.slow ? 1 : 0)) {
+      quantise(std::true_type{});
+    } else {
+      quantise(std::false_type{});
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+    if (lane == 0) reinterpret_cast<int32_t *>(dst + l6.sums_off)[row] = sum;
+  };
+
+  // Workgroup w takes row (w % 8) * rows / 8 + w / 8 (a cache line of the operand buffer takes pieces of 4 (heads) or
+  // 16 (tails) consecutive rows; workgroups are dealt round-robin to the 8 XCDs, so rows that share lines run on
+  // the same XCD at about the same time and meet in its L2), then every gridDim.x-th further item.
+  const int64_t per_xcd = (rows + 7) >> 3, items = per_xcd * 8;
+  auto row_of = [&](int64_t w) { return (w & 7) * per_xcd + (w >> 3); };
+  auto clamped = [&](int64_t r) { return r < rows ? r : rows - 1; };
+  int64_t w = blockIdx.x;
+  if (w >= items) return;
+  issue(clamped(row_of(w)), 0);
+  for (int it = 0; w < items; w += gridDim.x, ++it) {
+    const int64_t next = w + gridDim.x;
+    const uint32_t cur = NBUF == 2 ? (it & 1) * img_bytes : 0u;
+    if (NBUF == 2 && next < items) {
+      issue(clamped(row_of(next)), img_bytes - cur);
+      __builtin_amdgcn_s_waitcnt(vmcnt_imm(JT > 0 ? 4 * JT : 0));  // everything but the copy just requested has landed
+    } else {
+      __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+    }
+    const int64_t row = row_of(w);
+    if (row < rows) process(row, row_img + cur);
+    if (NBUF == 1 && next < items) {
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // this row's LDS reads are done before the image is overwritten
+      issue(clamped(row_of(next)), 0);
+    }
   }
 }
 
@@ -1005,6 +1194,44 @@ int launch_asym(const void *x, int64_t rows, int64_t cols, const uint8_t *cm, co
   return check_launch();
 }
 
+
+// 6-bit operand output through quantize_fp6_wave_kernel; meta: (scale, zero) pairs, or one scale per row (SYM)
+template <bool BF16, bool SYM>
+int launch_fp6_wave(const void *x, int64_t rows, int64_t cols, const uint8_t *cm, const ColmapLayout &l, int64_t num_int,
+                    int64_t num_fp, void *dst, void *meta, hipStream_t st, float sym_divisor = 1.0f) {
+  const int J = static_cast<int>((cols / 32 + 63) / 64);
+  const int64_t items = (rows + 7) / 8 * 8;
+  auto go = [&](auto kern, int nbuf, int per_cu) {
+    const int lds = nbuf * J * 4096;
+    if (lds > 48 * 1024) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+      if (e != hipSuccess) {
+        set_last_hip_error(e);
+        return static_cast<int>(QUIK_ERR_LAUNCH);
+      }
+    }
+    const int64_t resident = int64_t(num_cus()) * per_cu / 8 * 8;
+    const int grid = static_cast<int>(items < resident ? items : resident);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(64), static_cast<size_t>(lds), st, static_cast<const uint16_t *>(x), rows,
+                       static_cast<int>(cols), reinterpret_cast<const uint32_t *>(cm + l.off_patch),
+                       reinterpret_cast<const uint16_t *>(cm + l.off_fp), reinterpret_cast<const uint32_t *>(cm + l.off_flags),
+                       static_cast<int>(num_int), static_cast<int>(num_fp), static_cast<uint8_t *>(dst),
+                       static_cast<uint16_t *>(meta), sym_divisor);
+    return check_launch();
+  };
+  // one wave per SIMD, two row images each (at most 2 x 20 KB per wave)
+  switch (J) {
+    case 1: return go(quantize_fp6_wave_kernel<BF16, SYM, 1>, 2, 4);
+    case 2: return go(quantize_fp6_wave_kernel<BF16, SYM, 2>, 2, 4);
+    case 3: return go(quantize_fp6_wave_kernel<BF16, SYM, 3>, 2, 4);
+    case 4: return go(quantize_fp6_wave_kernel<BF16, SYM, 4>, 2, 4);
+    case 5: return go(quantize_fp6_wave_kernel<BF16, SYM, 5>, 2, 4);
+    default: break;
+  }
+  // longer rows: one image per wave, as many waves per CU as their images fit (160 KB of LDS)
+  const int per_cu = 160 / (J * 4) < 8 ? 160 / (J * 4) : 8;
+  return go(quantize_fp6_wave_kernel<BF16, SYM, 0>, 1, per_cu);
+}
 }  // namespace
 }  // namespace quik
 
@@ -1028,12 +1255,14 @@ extern "C" int quik_colmap_build(const int64_t *int_indices, int64_t num_int, co
                        num_int, fp_indices, num_fp, cols, reinterpret_cast<uint16_t *>(cm),
                        reinterpret_cast<uint16_t *>(cm + l.off_fp), mask, reinterpret_cast<uint32_t *>(cm + l.off_grp),
                        reinterpret_cast<uint32_t *>(cm + l.off_dirty), reinterpret_cast<uint16_t *>(cm + l.off_slot),
+                       reinterpret_cast<uint16_t *>(cm + l.off_kperm), reinterpret_cast<uint32_t *>(cm + l.off_patch),
                        reinterpret_cast<uint32_t *>(cm + l.off_flags));
   } else {
     hipLaunchKernelGGL(colmap_build_kernel<uint32_t>, dim3(1), dim3(1024), 0, as_stream(stream), int_indices,
                        num_int, fp_indices, num_fp, cols, reinterpret_cast<uint32_t *>(cm),
                        reinterpret_cast<uint32_t *>(cm + l.off_fp), mask, reinterpret_cast<uint32_t *>(cm + l.off_grp),
                        reinterpret_cast<uint32_t *>(cm + l.off_dirty), reinterpret_cast<uint16_t *>(cm + l.off_slot),
+                       reinterpret_cast<uint16_t *>(cm + l.off_kperm), reinterpret_cast<uint32_t *>(cm + l.off_patch),
                        reinterpret_cast<uint32_t *>(cm + l.off_flags));
   }
   return check_launch();
@@ -1092,13 +1321,11 @@ extern "C" int quik_asym_quantize_fp6(const void *x, int dtype, int64_t rows, in
   if (rows == 0) return QUIK_OK;
   if (!x || !colmap || !out6 || !meta) return QUIK_ERR_NULL;
   if (reinterpret_cast<uintptr_t>(x) % 16 != 0 || reinterpret_cast<uintptr_t>(out6) % 256 != 0) return QUIK_ERR_ALIGN;
-  void *fp_x = nullptr;
   const ColmapLayout l = colmap_layout(cols, num_int, num_fp);
   const uint8_t *cm = static_cast<const uint8_t *>(colmap);
   hipStream_t st = as_stream(stream);
-  return dtype == QUIK_F16
-             ? launch_asym<uint16_t, 4, false>(x, rows, cols, cm, l, num_int, num_fp, out6, meta, fp_x, st, true)
-             : launch_asym<uint16_t, 4, true>(x, rows, cols, cm, l, num_int, num_fp, out6, meta, fp_x, st, true);
+  return dtype == QUIK_F16 ? launch_fp6_wave<false, false>(x, rows, cols, cm, l, num_int, num_fp, out6, meta, st)
+                           : launch_fp6_wave<true, false>(x, rows, cols, cm, l, num_int, num_fp, out6, meta, st);
 }
 
 extern "C" int quik_asym_quantize_tile8(const void *x, int dtype, int64_t rows, int64_t cols, const void *colmap,
@@ -1132,6 +1359,7 @@ extern "C" int quik_sym_quantize_mapped(const void *x, int64_t rows, int64_t col
   const ColmapLayout l = colmap_layout(cols, num_int, num_fp);
   const uint8_t *cm = static_cast<const uint8_t *>(colmap);
   hipStream_t st = as_stream(stream);
+  if (bits == 4 && tiled) return launch_fp6_wave<false, true>(x, rows, cols, cm, l, num_int, num_fp, dst, scale, st, divisor);
   return bits == 4 ? launch_sym_stream<4>(x, rows, cols, cm, l, num_int, num_fp, dst, scale, fp_x, st, tiled != 0, divisor)
                    : launch_sym_stream<8>(x, rows, cols, cm, l, num_int, num_fp, dst, scale, fp_x, st, tiled != 0, divisor);
 }

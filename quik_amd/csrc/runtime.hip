@@ -14,6 +14,21 @@ void set_last_hip_error(hipError_t e) {
   g_last_error[sizeof(g_last_error) - 1] = '\0';
 }
 
+// Compute units of the GPU (all GPUs of a box are the same part: asked once per process; 256 when no device answers,
+// e.g. for the size queries on a machine without a GPU).
+int num_cus() {
+  static const int n = [] {
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) {
+      (void)hipGetLastError();
+      return 256;
+    }
+    return cus;
+  }();
+  return n;
+}
+
 int check_launch() {
   hipError_t e = hipGetLastError();
   if (e == hipSuccess) return QUIK_OK;

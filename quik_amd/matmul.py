@@ -112,10 +112,11 @@ def _splitk_workspace(device, M, N, K, bits):
     return ws, ws.numel()
 
 
-def pack_weight_fp6(int_weight: torch.Tensor, fp_weight: torch.Tensor) -> torch.Tensor:
+def pack_weight_fp6(int_weight: torch.Tensor, fp_weight: torch.Tensor, colmap: torch.Tensor) -> torch.Tensor:
     """Nibble-packed int4 weights [N, K/2] and outlier weights [N, F] -> operand buffer for mixed_linear_fp6
-    (once per layer)."""
-    L.check_cuda_contiguous("pack_weight_fp6", int_weight=int_weight, fp_weight=fp_weight)
+    (once per layer).  `colmap` is the layer's column map (asymmetric.build_colmap): the operand buffers of this
+    path keep the integer columns in the map's in-place order, weights and activations alike."""
+    L.check_cuda_contiguous("pack_weight_fp6", int_weight=int_weight, fp_weight=fp_weight, colmap=colmap)
     if int_weight.dtype != torch.uint8 or int_weight.dim() != 2:
         raise RuntimeError("pack_weight_fp6: expected a uint8 [N, K/2] int_weight")
     if fp_weight.dtype not in (torch.float16, torch.bfloat16) or fp_weight.dim() != 2 or \
@@ -126,10 +127,19 @@ def pack_weight_fp6(int_weight: torch.Tensor, fp_weight: torch.Tensor) -> torch.
     nbytes = lib.quik_fp6_operand_bytes(N, K, F)
     if nbytes == 0:
         raise RuntimeError("pack_weight_fp6: K must be a multiple of 128 and F a multiple of 32")
+    if colmap.dtype != torch.uint8 or colmap.numel() != lib.quik_colmap_bytes(K + F, K, F):
+        raise RuntimeError(f"pack_weight_fp6: the column map was not built for {K} integer and {F} outlier columns")
+    from .asymmetric import colmap_streams
+    if getattr(colmap, "_quik_streams", None) is None:
+        colmap._quik_shape = (K + F, K, F)
+        colmap._quik_streams = colmap_streams(colmap, K, F)
+    if not colmap._quik_streams:
+        raise RuntimeError("pack_weight_fp6: the column map does not select the streaming kernel (ascending "
+                           "int_indices that partition the columns with fp_indices)")
     with L.device_guard(int_weight.device):
         out = torch.empty((nbytes,), dtype=torch.uint8, device=int_weight.device)
-        L.check(lib.quik_fp6_pack_weight(L.ptr(int_weight), L.ptr(fp_weight) if F else None, N, K, F, L.ptr(out),
-                                         L.stream()), "pack_weight_fp6")
+        L.check(lib.quik_fp6_pack_weight(L.ptr(int_weight), L.ptr(fp_weight) if F else None, N, K, F, L.ptr(colmap),
+                                         L.ptr(out), L.stream()), "pack_weight_fp6")
     return out
 
 

@@ -138,10 +138,12 @@ class MixedQLinear(torch.nn.Module):
         fp_w = self.fp_weight if self.fp_features_num > 0 else \
             torch.empty((self.out_features, 0), dtype=self.dtype, device=self.int_weight.device)
         key = (self.int_weight.data_ptr(), self.int_weight._version, fp_w.data_ptr(), fp_w._version,
-               self.int_weight.device)
+               self.int_weight.device, self._column_map().data_ptr())
         if self._w6 is None or self._w6_key != key:
-            pack = matmul.pack_weight_fp6 if self.bits == 4 else matmul.pack_weight_tile8
-            self._w6 = pack(self.int_weight, fp_w)
+            if self.bits == 4:    # in the column map's in-place order, as the activation is quantized
+                self._w6 = matmul.pack_weight_fp6(self.int_weight, fp_w, self._column_map())
+            else:
+                self._w6 = matmul.pack_weight_tile8(self.int_weight, fp_w)
             self._w6_key = key
         return self._w6
 

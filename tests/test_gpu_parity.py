@@ -943,10 +943,28 @@ def _decode_operand6(buf, rows, K, F):
     return levels, outl, sums
 
 
-@pytest.mark.parametrize("rows,K,F,bf16", [(70, 256, 32, False), (130, 128, 64, True), (64, 384, 0, False)])
+def _in_place_order(ii, fi, n_in):
+    """Position k of the 6-bit operand buffers -> index into ascending int_indices (restated from the rule in
+    quik_amd/csrc/colmap.h): source column k keeps its place when it is an integer column; the outlier columns among
+    the first K columns (holes, ascending) are filled by the integer columns of the last F columns (ascending)."""
+    K = len(ii)
+    outlier = np.zeros(n_in, bool)
+    outlier[fi] = True
+    holes = [c for c in range(K) if outlier[c]]
+    fillers = [c for c in range(K, n_in) if not outlier[c]]
+    assert len(holes) == len(fillers)
+    col = np.arange(K)
+    col[holes] = fillers
+    return np.searchsorted(np.sort(ii), col)
+
+
+@pytest.mark.parametrize("rows,K,F,bf16", [(70, 256, 32, False), (130, 128, 64, True), (64, 384, 0, False),
+                                           (9, 2048 + 128, 160, False), (200, 8192 + 2048, 512 + 64, False)])
 def test_six_bit_operand_buffers_hold_the_int4_codes(rows, K, F, bf16):
     """quantize_mapped_fp6 and pack_weight_fp6 write the codes of quantize_mapped / int_weight (bit-exact against
-    the oracle elsewhere) as levels code + 8, the outlier values and the level sums, in the documented layout."""
+    the oracle elsewhere) as levels code + 8, the outlier values and the level sums, in the documented layout,
+    with the integer columns in the column map's in-place order (the last cases: several fragments per lane, more
+    holes than a lane keeps in registers, rows longer than the double-buffered kernel takes)."""
     from quik_amd import asymmetric, matmul
     rng = np.random.default_rng(rows + K + F)
     n_in = K + F
@@ -964,8 +982,9 @@ def test_six_bit_operand_buffers_hold_the_int4_codes(rows, K, F, bf16):
     want = np.empty((rows, K), np.int64)
     want[:, 0::2] = (qn & 0xF) ^ 8
     want[:, 1::2] = (qn >> 4) ^ 8
+    order = _in_place_order(ii, fi, n_in)
     levels, outl, sums = _decode_operand6(x6.cpu().numpy(), rows, K, F)
-    assert np.array_equal(levels, want)
+    assert np.array_equal(levels, want[:, order])
     assert np.array_equal(outl, _bits(fp_x).reshape(rows, F))
     assert np.array_equal(sums, want.sum(1))
     # weights
@@ -973,12 +992,12 @@ def test_six_bit_operand_buffers_hold_the_int4_codes(rows, K, F, bf16):
     qw = rng.integers(0, 256, (N, K // 2)).astype(np.uint8)
     fpw = (0.02 * rng.standard_normal((N, F))).astype(np.float16)
     fpw_t = _bf16_t(fpw.astype(np.float32)) if bf16 else _t(fpw)
-    w6 = matmul.pack_weight_fp6(_t(qw), fpw_t)
+    w6 = matmul.pack_weight_fp6(_t(qw), fpw_t, colmap)
     want = np.empty((N, K), np.int64)
     want[:, 0::2] = (qw & 0xF) ^ 8
     want[:, 1::2] = (qw >> 4) ^ 8
     levels, outl, sums = _decode_operand6(w6.cpu().numpy(), N, K, F)
-    assert np.array_equal(levels, want)
+    assert np.array_equal(levels, want[:, order])
     assert np.array_equal(outl, _bits(fpw_t).reshape(N, F))
     assert np.array_equal(sums, want.sum(1))
 
@@ -1280,7 +1299,7 @@ def test_tile_ordered_paths_random_shapes():
         want = matmul.mixed_linear(q, qw, meta, s_w, wred, fp if F else None, fpw if F else None, bias, bits, dt)
         if bits == 4:
             xb, meta2 = asymmetric.quantize_mapped_fp6(x, cm, K, F)
-            got = matmul.mixed_linear_fp6(xb, matmul.pack_weight_fp6(qw, fpw), meta2, s_w, wred, bias, M, N, K, F, dt)
+            got = matmul.mixed_linear_fp6(xb, matmul.pack_weight_fp6(qw, fpw, cm), meta2, s_w, wred, bias, M, N, K, F, dt)
         else:
             xb, meta2 = asymmetric.quantize_mapped_tile8(x, cm, K, F)
             got = matmul.mixed_linear_tile8(xb, matmul.pack_weight_tile8(qw, fpw), meta2, s_w, wred, bias, M, N, K, F, dt)
