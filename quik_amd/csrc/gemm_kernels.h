@@ -487,8 +487,18 @@ struct BlockStore {
   static __device__ __forceinline__ void write_block(const v4i (&piece)[kIters], int lane, T *g, int64_t ld) {
 #pragma unroll
     for (int it = 0; it < kIters; ++it)
-      *reinterpret_cast<v4i *>(g + int64_t(it * kRowsPerInstr + lane / kLanesPerRow) * ld +
-                               (lane % kLanesPerRow) * kElems) = piece[it];
+      store_piece(piece[it], g + int64_t(it * kRowsPerInstr + lane / kLanesPerRow) * ld + (lane % kLanesPerRow) * kElems);
+  }
+  // One 16-byte piece of an output row.  The fp16 / bf16 layer output is written once and not read again by this
+  // launch: a streaming (non-temporal) store keeps its 100+ MB from displacing the operand lines that the tiles of
+  // an XCD share through L2 (70B gate_proj, 2048 tokens: GEMM 0.274 -> 0.242 ms).  The int32 product of the
+  // stand-alone GEMMs is read back at once by a dequantize kernel and keeps the default policy.
+  static __device__ __forceinline__ void store_piece(const v4i &piece, T *dst) {
+    if constexpr (sizeof(T) == 2) {
+      __builtin_nontemporal_store(piece, reinterpret_cast<v4i *>(dst));
+    } else {
+      *reinterpret_cast<v4i *>(dst) = piece;
+    }
   }
 
   // staged block -> g[row * ld + col], rows < rows_valid, cols < cols_valid
@@ -505,8 +515,7 @@ struct BlockStore {
                                                    (lane % kLanesPerRow) * 16);
 #pragma unroll
       for (int it = 0; it < kIters; ++it)
-        *reinterpret_cast<v4i *>(g + int64_t(it * kRowsPerInstr + lane / kLanesPerRow) * ld +
-                                 (lane % kLanesPerRow) * kElems) = piece[it];
+        store_piece(piece[it], g + int64_t(it * kRowsPerInstr + lane / kLanesPerRow) * ld + (lane % kLanesPerRow) * kElems);
       __builtin_amdgcn_wave_barrier();
       return;
     }
@@ -518,7 +527,7 @@ struct BlockStore {
       if (r >= rows_valid) continue;
       T *dst = g + int64_t(r) * ld + c;
       if (vec && c + kElems <= cols_valid) {
-        *reinterpret_cast<v4i *>(dst) = piece;
+        store_piece(piece, dst);
       } else {
         T tmp[kElems];
         __builtin_memcpy(tmp, &piece, 16);
