@@ -747,23 +747,62 @@ __global__ __launch_bounds__(TPR) void asym_quantize_stream_kernel(
   }
 }
 
+// Packed fp16 min / max as single instructions.  (The compiler's own minnum / maxnum first quiet a possible
+// signalling NaN with an extra v_pk_max x, x whenever it cannot prove that the operand is not one.)
+__device__ __forceinline__ uint32_t pk_min_f16(uint32_t a, uint32_t b) {
+  uint32_t r;
+  asm("v_pk_min_f16 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+__device__ __forceinline__ uint32_t pk_max_f16(uint32_t a, uint32_t b) {
+  uint32_t r;
+  asm("v_pk_max_f16 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+
+// 4-bit LEVELS (code + 8, 0 .. 15) of the two fp16 halves of w in bytes 0 and 2 of the result, for rows on the fast
+// path (finite range, scale >= 1e-6; RowQuant::slow == false); same levels as code_pair gives.
+//   asymmetric: d = fp16(x - zero); t = fp16(f32(d) * rcp); t = max(t, 0) (a NaN element becomes 0, as the
+//   reference's integer conversion makes it); t + 1024 holds rne(t) in its low mantissa bits.  No upper clamp:
+//   on this path t < 15.5 for every fp16 scale (x - zero <= max - min, the scale is at least fp16((max - min) / 15),
+//   and over all fp16 scales >= 1e-6 the largest quotient, reached at the smallest, subnormal scale, is 15.47;
+//   tests/test_quotient_levels.py enumerates them).
+//   symmetric: t = fp16(f32(x) * rcp) with |t| <= 4.2 (scale = fp16(max|x| / 4), at most 3 % below the quotient
+//   for the smallest scale); t + 1544 holds rne(t) + 8 in its low mantissa bits.
+template <bool SYM, class RQ>
+__device__ __forceinline__ uint32_t level_pair_fast(uint32_t w, const RQ &rq) {
+  uint32_t d = w, tb;
+  if constexpr (!SYM) {
+    const _Float16 zh = static_cast<_Float16>(rq.zero);
+    d = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, w) - h2{zh, zh});
+  }
+  asm("v_fma_mixlo_f16 %0, %1, %2, 0 op_sel_hi:[1,0,0]\n\t"
+      "v_fma_mixhi_f16 %0, %1, %2, 0 op_sel:[1,0,0] op_sel_hi:[1,0,0]"
+      : "=&v"(tb)
+      : "v"(d), "v"(rq.rcp));
+  if constexpr (!SYM) tb = pk_max_f16(tb, 0u);
+  constexpr _Float16 magic = static_cast<_Float16>(SYM ? 1544 : 1024);
+  return __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, tb) + h2{magic, magic});
+}
+
 // ---------------------------------------------------------------------------------------
 // 6-bit operand buffers (consumer: gemm_fp6.h), written in the in-place order of the column map.
 //
 // One wave per row.  The wave copies the row global -> LDS with 16-byte-per-lane direct copies (no
-// registers are held while the row is in flight), in the order its lanes read it back: 16-byte slot
-// (4 j + i) * 64 + L of the row image holds source group 4 (L + 64 j) + i, i.e. lane L owns the
-// fragments (32 consecutive source columns each) L, L + 64, ..., and every LDS read of the wave covers
-// 64 consecutive slots.  In the image the holes (outlier columns among the first num_int columns) are
+// registers are held while the row is in flight).  A copy instruction moves one contiguous kilobyte
+// (64 groups of 8 columns = 16 fragments of 32 consecutive source columns; whole cache lines) and deals
+// it to the LDS slots transposed: slot 16 i + m of the kilobyte holds group 4 m + i, i.e. the i-th group
+// of the kilobyte's fragment m.  Lane L owns the fragments L, L + 64, ...; its i-th 16-byte read of a
+// fragment and those of its 15 neighbours cover 256 consecutive bytes, so all reads are free of bank
+// conflicts.  In the image the holes (outlier columns among the first num_int columns) are
 // overwritten with their fillers (integer columns of the tail), two-byte LDS copies with row-invariant
 // addresses held in registers; after that the first num_int columns ARE the integer operand, in place:
 // one pass over the image for min / max, a second one that turns each fragment into 32 levels, packs
 // them to 24 bytes in registers and stores head and tail.  No barrier, no cross-wave reduction (a wave's
 // LDS operations execute in order), no data moved between lanes except the two reductions.
-// A workgroup (= wave) walks over rows w, w + grid, ...; with JT > 0 (fragments per lane known at
-// compile time, rows up to 10240 columns) the image is double-buffered and the next row's copy is in
-// flight while the current row is processed; the first two rows of a wave are requested back to back,
-// so across the chip the first rows' requests queue ahead of the second rows' and arrive first.
+// A workgroup (= wave) walks over rows w, w + grid, ...; up to eight of them share a CU (two per SIMD),
+// so one wave's arithmetic covers the other's transfer and LDS waits.  JT > 0: fragments per lane known at
+// compile time (rows up to 10240 columns); 0: a run-time loop over them.
 template <bool BF16, bool SYM, int JT>
 __global__ __launch_bounds__(64) void quantize_fp6_wave_kernel(
     const uint16_t *__restrict__ x, int64_t rows, int cols, const uint32_t *__restrict__ patch,
@@ -775,29 +814,17 @@ __global__ __launch_bounds__(64) void quantize_fp6_wave_kernel(
   const int lane = threadIdx.x;
   const int frags_all = cols >> 5, frags = num_int >> 5, nchunk = num_fp >> 3;
   const int J = JT > 0 ? JT : (frags_all + 63) >> 6;
-  const uint32_t img_bytes = static_cast<uint32_t>(J) * 4096u;
-  constexpr int NBUF = JT > 0 ? 2 : 1;
   const int nholes = static_cast<int>(flags[2]);
   const Fp6Layout l6 = fp6_layout(rows, num_int, num_fp);
   const uint32_t lds0 = lds_address(row_img);
 
+  constexpr int PREG = 4;
+  uint32_t p_hole[PREG], p_fill[PREG], o_addr[8];
   // byte offset of source column c inside a row image
   auto img_of_col = [](uint32_t c) -> uint32_t {
     const uint32_t g = c >> 3, f = g >> 2, i = g & 3u;
-    return ((((f >> 6) * 4u + i) * 64u + (f & 63u)) << 4) + ((c & 7u) << 1);
+    return ((f >> 4) << 10) + ((16u * i + (f & 15u)) << 4) + ((c & 7u) << 1);
   };
-  // row-invariant addresses in registers: this lane's first four patches and its first chunk of 8 outliers
-  constexpr int PREG = 4;
-  uint32_t p_hole[PREG], p_fill[PREG], o_addr[8];
-#pragma unroll
-  for (int k = 0; k < PREG; ++k) {
-    const uint32_t e = (lane + 64 * k) < nholes ? patch[lane + 64 * k] : 0u;
-    p_hole[k] = img_of_col(e & 0xFFFFu);
-    p_fill[k] = img_of_col(e >> 16);
-  }
-#pragma unroll
-  for (int k = 0; k < 8; ++k) o_addr[k] = lane < nchunk ? img_of_col(fp_col[lane * 8 + k]) : 0u;
-
   // body(j) for this lane's fragment slots j = 0 .. J-1, unrolled when their number is known at compile time
   auto for_j = [&](auto body) {
     if constexpr (JT > 0) {
@@ -807,17 +834,21 @@ __global__ __launch_bounds__(64) void quantize_fp6_wave_kernel(
       for (int j = 0; j < J; ++j) body(j);
     }
   };
-  auto issue = [&](int64_t row, uint32_t buf) {
+  auto issue = [&](int64_t row) {
     const uint64_t a = reinterpret_cast<uint64_t>(x + row * cols);
     // (the intrinsic returns int: each half goes through uint32_t, or the low half would be sign-extended)
     const uint32_t a_hi = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(a >> 32)));
     const uint32_t a_lo = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(a & 0xFFFFFFFFu)));
     const uint8_t *rp = reinterpret_cast<const uint8_t *>((static_cast<uint64_t>(a_hi) << 32) | a_lo);
+    // kilobyte q = 4 j + t of the row: this lane copies group 64 q + 4 (lane % 16) + lane / 16 to slot 64 q + lane
+    const int g_in = 4 * (lane & 15) + (lane >> 4), g_last = (cols >> 3) - 1;
     for_j([&](int j) {
-      const int f = lane + 64 * j < frags_all ? lane + 64 * j : frags_all - 1;  // past the row: any valid fragment
-      const uint32_t voff = static_cast<uint32_t>(f) * 64u;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) dma_load16(rp + i * 16, voff, lds0 + buf + (4 * j + i) * 1024);
+      for (int t = 0; t < 4; ++t) {
+        const int g = 64 * (4 * j + t) + g_in;
+        const uint32_t voff = static_cast<uint32_t>(g < g_last ? g : g_last) * 16u;  // past the row: any valid group
+        dma_load16(rp, voff, lds0 + (4 * j + t) * 1024);
+      }
     });
   };
 
@@ -855,13 +886,13 @@ __global__ __launch_bounds__(64) void quantize_fp6_wave_kernel(
 
     auto load_fragment = [&](int j, uint4 (&v)[4]) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) v[i] = *reinterpret_cast<const uint4 *>(img + (((4 * j + i) * 64 + lane) << 4));
+      for (int i = 0; i < 4; ++i)
+        v[i] = *reinterpret_cast<const uint4 *>(img + ((4 * j + (lane >> 4)) << 10) + ((16 * i + (lane & 15)) << 4));
     };
     // ---- pass 1: min / max (symmetric: largest |x| pattern) over this lane's fragments
     const float inf = __builtin_inff();
     float mn = inf, mx = -inf;
-    const h2 pinf = h2{static_cast<_Float16>(inf), static_cast<_Float16>(inf)};
-    h2 pmn = pinf, pmx = -pinf;
+    uint32_t pmn_b = 0x7C007C00u, pmx_b = 0xFC00FC00u;  // +inf / -inf in both halves
     u2 amax = u2{0, 0};
     for_j([&](int j) {
       if (lane + 64 * j < frags) {
@@ -874,11 +905,11 @@ __global__ __launch_bounds__(64) void quantize_fp6_wave_kernel(
 #pragma unroll
             for (int k = 0; k < 4; ++k) amax = __builtin_elementwise_max(amax, __builtin_bit_cast(u2, w[k] & 0x7FFF7FFFu));
           } else if constexpr (!BF16) {
-#pragma unroll
-            for (int k = 0; k < 4; ++k) {
-              pmn = __builtin_elementwise_min(pmn, __builtin_bit_cast(h2, w[k]));
-              pmx = __builtin_elementwise_max(pmx, __builtin_bit_cast(h2, w[k]));
-            }
+            // packed fp16 min / max skip NaN operands, as the reference's __hmin / __hmax do
+            const uint32_t lo = pk_min_f16(pk_min_f16(w[0], w[1]), pk_min_f16(w[2], w[3]));
+            const uint32_t hi = pk_max_f16(pk_max_f16(w[0], w[1]), pk_max_f16(w[2], w[3]));
+            pmn_b = pk_min_f16(pmn_b, lo);
+            pmx_b = pk_max_f16(pmx_b, hi);
           } else {
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
@@ -890,6 +921,7 @@ __global__ __launch_bounds__(64) void quantize_fp6_wave_kernel(
         }
       }
     });
+    const h2 pmn = __builtin_bit_cast(h2, pmn_b), pmx = __builtin_bit_cast(h2, pmx_b);
     if constexpr (SYM) {
       mn = 0.0f;
       mx = static_cast<float>(amax.x > amax.y ? amax.x : amax.y);  // a 15-bit integer: exact, ordered like the patterns
@@ -919,12 +951,19 @@ __global__ __launch_bounds__(64) void quantize_fp6_wave_kernel(
         if (f < frags) {
           uint4 v[4];
           load_fragment(j, v);
-          uint32_t b[8];
+          uint32_t b[8];  // 32 levels, one per byte
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            const uint2 c = group_codes<4, BF16, SLOW, SYM>(v[i], rq);  // code nibbles (two's complement), one per byte
-            b[2 * i] = c.x ^ 0x08080808u;                               // level = code + 8
-            b[2 * i + 1] = c.y ^ 0x08080808u;
+            if constexpr (!SLOW && !BF16) {
+              const uint32_t p0 = level_pair_fast<SYM>(v[i].x, rq), p1 = level_pair_fast<SYM>(v[i].y, rq);
+              const uint32_t p2 = level_pair_fast<SYM>(v[i].z, rq), p3 = level_pair_fast<SYM>(v[i].w, rq);
+              b[2 * i] = __builtin_amdgcn_perm(p1, p0, 0x06040200u);  // bytes 0, 2 of p0 then bytes 0, 2 of p1
+              b[2 * i + 1] = __builtin_amdgcn_perm(p3, p2, 0x06040200u);
+            } else {
+              const uint2 c = group_codes<4, BF16, SLOW, SYM>(v[i], rq);  // code nibbles (two's complement), one per byte
+              b[2 * i] = c.x ^ 0x08080808u;                               // level = code + 8
+              b[2 * i + 1] = c.y ^ 0x08080808u;
+            }
           }
 #pragma unroll
           for (int i = 0; i < 8; ++i) sum = __builtin_amdgcn_udot4(b[i], 0x01010101u, sum, false);
@@ -952,21 +991,36 @@ __global__ __launch_bounds__(64) void quantize_fp6_wave_kernel(
   auto clamped = [&](int64_t r) { return r < rows ? r : rows - 1; };
   int64_t w = blockIdx.x;
   if (w >= items) return;
-  issue(clamped(row_of(w)), 0);
-  for (int it = 0; w < items; w += gridDim.x, ++it) {
-    const int64_t next = w + gridDim.x;
-    const uint32_t cur = NBUF == 2 ? (it & 1) * img_bytes : 0u;
-    if (NBUF == 2 && next < items) {
-      issue(clamped(row_of(next)), img_bytes - cur);
-      __builtin_amdgcn_s_waitcnt(vmcnt_imm(JT > 0 ? 4 * JT : 0));  // everything but the copy just requested has landed
-    } else {
-      __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+  issue(clamped(row_of(w)));
+  // Row-invariant addresses in registers: this lane's first four patches and its first chunk of 8 outliers.  The
+  // loads are unconditional (clamped indices, one 16-byte load for the eight outlier columns) and come after the
+  // first row's copies, so they are all in flight together and behind the row, not in front of it.
+  {
+    const int last_hole = nholes > 0 ? nholes - 1 : 0;
+    uint32_t e[PREG];
+#pragma unroll
+    for (int k = 0; k < PREG; ++k) e[k] = patch[lane + 64 * k < nholes ? lane + 64 * k : last_hole];
+    const int chunk = lane < nchunk ? lane : 0;
+    const uint4 oc = nchunk > 0 ? *reinterpret_cast<const uint4 *>(fp_col + chunk * 8) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+    for (int k = 0; k < PREG; ++k) {
+      p_hole[k] = img_of_col(e[k] & 0xFFFFu);
+      p_fill[k] = img_of_col(e[k] >> 16);
     }
+    const uint32_t ow[4] = {oc.x, oc.y, oc.z, oc.w};
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      o_addr[2 * k] = img_of_col(ow[k] & 0xFFFFu);
+      o_addr[2 * k + 1] = img_of_col(ow[k] >> 16);
+    }
+  }
+  for (; w < items; w += gridDim.x) {
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));  // this row's image has landed
     const int64_t row = row_of(w);
-    if (row < rows) process(row, row_img + cur);
-    if (NBUF == 1 && next < items) {
+    if (row < rows) process(row, row_img);
+    if (w + gridDim.x < items) {
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // this row's LDS reads are done before the image is overwritten
-      issue(clamped(row_of(next)), 0);
+      issue(clamped(row_of(w + gridDim.x)));
     }
   }
 }
@@ -1201,8 +1255,11 @@ int launch_fp6_wave(const void *x, int64_t rows, int64_t cols, const uint8_t *cm
                     int64_t num_fp, void *dst, void *meta, hipStream_t st, float sym_divisor = 1.0f) {
   const int J = static_cast<int>((cols / 32 + 63) / 64);
   const int64_t items = (rows + 7) / 8 * 8;
-  auto go = [&](auto kern, int nbuf, int per_cu) {
-    const int lds = nbuf * J * 4096;
+  // as many waves per CU as their row images fit (160 KB of LDS), at most 8: two waves per SIMD cover each other's
+  // waits (measured at 2048 x 8192: 12.9 us against 14.0 us for one wave per SIMD with two images each)
+  const int per_cu = 160 / (J * 4) < 8 ? 160 / (J * 4) : 8;
+  auto go = [&](auto kern) {
+    const int lds = J * 4096;  // one row image
     if (lds > 48 * 1024) {
       hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
       if (e != hipSuccess) {
@@ -1219,18 +1276,15 @@ int launch_fp6_wave(const void *x, int64_t rows, int64_t cols, const uint8_t *cm
                        static_cast<uint16_t *>(meta), sym_divisor);
     return check_launch();
   };
-  // one wave per SIMD, two row images each (at most 2 x 20 KB per wave)
-  switch (J) {
-    case 1: return go(quantize_fp6_wave_kernel<BF16, SYM, 1>, 2, 4);
-    case 2: return go(quantize_fp6_wave_kernel<BF16, SYM, 2>, 2, 4);
-    case 3: return go(quantize_fp6_wave_kernel<BF16, SYM, 3>, 2, 4);
-    case 4: return go(quantize_fp6_wave_kernel<BF16, SYM, 4>, 2, 4);
-    case 5: return go(quantize_fp6_wave_kernel<BF16, SYM, 5>, 2, 4);
+  switch (J) {  // fragments per lane known at compile time: the loops over them unroll
+    case 1: return go(quantize_fp6_wave_kernel<BF16, SYM, 1>);
+    case 2: return go(quantize_fp6_wave_kernel<BF16, SYM, 2>);
+    case 3: return go(quantize_fp6_wave_kernel<BF16, SYM, 3>);
+    case 4: return go(quantize_fp6_wave_kernel<BF16, SYM, 4>);
+    case 5: return go(quantize_fp6_wave_kernel<BF16, SYM, 5>);
     default: break;
   }
-  // longer rows: one image per wave, as many waves per CU as their images fit (160 KB of LDS)
-  const int per_cu = 160 / (J * 4) < 8 ? 160 / (J * 4) : 8;
-  return go(quantize_fp6_wave_kernel<BF16, SYM, 0>, 1, per_cu);
+  return go(quantize_fp6_wave_kernel<BF16, SYM, 0>);
 }
 }  // namespace
 }  // namespace quik

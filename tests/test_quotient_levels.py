@@ -47,3 +47,38 @@ def test_uncorrected_reciprocal_product_never_changes_a_level():
     assert (two_step != want).sum() > 0
     for maxq in (15, 255):
         assert np.array_equal(_levels(two_step, maxq), _levels(want, maxq))
+
+
+def test_four_bit_quotient_never_reaches_the_upper_clamp_on_the_fast_path():
+    """The kernel that writes the 6-bit operand buffers drops the upper clamp min(t, 15) for rows with a finite
+    range.  That is safe if fp16(d * r) < 15.5 for every numerator d = fp16(x - zero) a row can hold.  d is at most
+    the fp16 round-up of the row's range, and the scale is fp16(max(range / 15, 1e-6)): for every fp16 scale this
+    takes the largest range that still rounds to that scale (plus the slack of the fp32 division) and the largest
+    numerator it allows, and evaluates the quotient both ways.  The largest value, 15.47, belongs to the smallest,
+    subnormal scale, whose rounding error is the largest relative to its size."""
+    pat = np.arange(0x0011, 0x7C00, dtype=np.uint16)                    # fp16(1e-6) = 0x0011 is the smallest scale
+    assert np.float16(1e-6).view(np.uint16) == 0x0011
+    s = pat.view(np.float16).astype(np.float64)
+    nxt = (pat + 1).view(np.float16).astype(np.float64)
+    nxt[-1] = 65536.0
+    hi = (s + nxt) / 2                                                  # fp32 values up to here round to s
+    r_max = 15 * hi * (1 + 2.0 ** -22)
+    keep = r_max <= 65504.0 * (1 + 2.0 ** -10)                          # a larger range takes the IEEE-divide path
+    with np.errstate(over="ignore"):
+        d = r_max.astype(np.float32).astype(np.float16)
+        d = np.where(d.astype(np.float64) < r_max, np.nextafter(d, np.float16(np.inf)), d).astype(np.float16)
+    keep &= np.isfinite(d)
+    d64, s64 = d.astype(np.float64)[keep], s[keep]
+    r = (1.0 / s64).astype(np.float32).astype(np.float64)
+    two_step = (d64 * r).astype(np.float32).astype(np.float16).astype(np.float64)
+    one_step = (d64 * r).astype(np.float16).astype(np.float64)
+    exact = (d64 / s64).astype(np.float16).astype(np.float64)
+    top = np.maximum(np.maximum(two_step, one_step), exact)
+    assert keep.sum() > 25000 and top.max() < 15.5
+    assert top.max() > 15.4 and s64[top.argmax()] == np.float16(1e-6)    # the bound is tight where the text says
+    # symmetric activations: scale = fp16(max|x| / 4) >= 1e-6 on the fast path, so |t| stays near 4
+    a = np.arange(0x0001, 0x7C00, dtype=np.uint16).view(np.float16)
+    sc = (a.astype(np.float32) / np.float32(4)).astype(np.float16)
+    ok = sc >= np.float16(1e-6)
+    t = (a[ok].astype(np.float64) * (1.0 / sc[ok].astype(np.float64)).astype(np.float32)).astype(np.float16)
+    assert np.abs(t.astype(np.float64)).max() < 4.5
