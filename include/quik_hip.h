@@ -223,6 +223,18 @@ int quik_mixed_linear_fwd_tile8_ws(const void *x8, const void *w8, const void *m
                                    int64_t K, int64_t F, void *out, void *workspace, int64_t workspace_bytes,
                                    void *stream);
 
+/* ---- the reference's simulated (fake-quant) activation path ---------------------------------------
+ * replaces the tensor-op sequence of ActQuantWrapper.forward, experiments/quant_sim.py:227-256
+ * (ActQuantizer.find_params :167-188, asymmetric_quantize :5-7), which the reference uses for its
+ * accuracy experiments: per row, over the columns whose bit in outlier_mask is clear,
+ *   xmin = min(min x, 0), xmax = max(max x, 0) (both zero -> -1, +1), scale = (xmax - xmin) / (2^bits - 1),
+ *   zero = round(-xmin / scale), out = scale * (clamp(round(x / scale) + zero, 0, 2^bits - 1) - zero);
+ * columns whose bit is set are copied.  fp32 arithmetic, one rounding to dtype.
+ *   x, out [rows, cols] dtype; outlier_mask [ceil(cols / 32)] uint32, bit c % 32 of word c / 32 = column c;
+ *   bits 2 .. 8. */
+int quik_sim_act_fake_quant(const void *x, int dtype, int64_t rows, int64_t cols, const uint32_t *outlier_mask,
+                            int bits, void *out, void *stream);
+
 /* ---- one entry point that allocates nothing ---------------------------------------------------------
  * No counterpart in the reference.  For callers that cannot allocate device memory around the call and
  * have no workspace to hand in: code under HIP graph capture, tight serving loops, harnesses that

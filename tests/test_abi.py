@@ -94,6 +94,12 @@ def test_tile_ordered_entry_points_validate_without_gpu():
     assert lib.quik_mixed_linear_fwd_tile8(one, one, null, one, one, null, 0, 64, 256, 28416, 256, one, null) == -5
     assert lib.quik_splitk_workspace_bytes(64, 8192, 28416, 8) > 4096
     assert lib.quik_splitk_workspace_bytes(2048, 28672, 7936, 4) == 0
+    assert lib.quik_sim_act_fake_quant(one, 0, 4, 64, one, 1, one, null) == -1
+    assert lib.quik_sim_act_fake_quant(one, 0, 4, 64, one, 9, one, null) == -1
+    assert lib.quik_sim_act_fake_quant(one, 2, 4, 64, one, 4, one, null) == -3
+    assert lib.quik_sim_act_fake_quant(one, 0, 4, 0, one, 4, one, null) == -2
+    assert lib.quik_sim_act_fake_quant(one, 0, 4, 64, null, 4, one, null) == -5
+    assert lib.quik_sim_act_fake_quant(one, 0, 0, 64, one, 4, one, null) == 0
 
 
 def test_python_surface_matches_reference_names():
