@@ -90,6 +90,29 @@ def make_layer(name, device, seed=0):
     return mod, x, W, int_idx, fp_idx
 
 
+def verify_spot_tile(name, out, x_cpu, W_cpu, fp_idx, mod, rows=48, cols=64):
+    """Three spot tiles of the layer output (first, middle straddling a tile boundary, last) against the CPU oracle's
+    MixedQLinear forward (oracle/quik_oracle.py), tolerance 1e-2 x output RMS: the check of the exact configuration
+    that is timed.  Runs once, before the warm-up; returns the largest error relative to the RMS."""
+    import numpy as np
+
+    from oracle import quik_oracle as qo
+    M, n_in, N, F, bits = WORKLOADS[name]
+    th, tw = min(rows, M), min(cols, N)
+    mid_c = min(N - tw, (N // 2 // 256) * 256 + 200)
+    worst = 0.0
+    for r0, c0 in ((0, 0), ((M - th) // 2, mid_c), (M - th, N - tw)):
+        r, c = slice(r0, r0 + th), slice(c0, c0 + tw)
+        omod = qo.from_float(W_cpu[c].numpy(), mod.weights_scales[c].cpu().numpy(), fp_idx.numpy(), bits)
+        want, _ = qo.mixed_qlinear_forward(x_cpu[r].numpy(), omod, bits)
+        got = out[r, c].float().cpu().numpy().astype(np.float64)
+        w64 = want.astype(np.float64)
+        rel = float(np.abs(got - w64).max() / np.sqrt((w64 ** 2).mean()))
+        assert rel <= 1e-2, f"bench.py: output differs from the oracle on tile ({r0}, {c0}): {rel:.3e} x RMS"
+        worst = max(worst, rel)
+    return worst
+
+
 def cpu_baseline(name, x, W, int_idx, fp_idx, budget_s=25.0):
     """CPU restatement of the reference's simulated path on the host cores (oracle/sim_path.py)."""
     import torch
@@ -154,87 +177,126 @@ def make_device_layer(n_in, N, F, bits, fp_idx, shared, gen, device):
     return mod
 
 
-def bench_block(args):
-    import torch
-    import torch.nn.functional as Fn
+class DecoderBlock:
+    """One Llama-2-70B-sized decoder block whose seven linears are MixedQLinear (q/k/v/o/gate/up W4A4, down_proj
+    W8A8, 256 fp16 outlier columns each; q/k/v and gate/up share their quantized input as experiments/llama.py:394-440
+    sets them up).  The same weights also exist as two fused groups (one quantize and ONE GEMM for q/k/v and for
+    gate/up).  RMSNorm, attention (torch SDPA, causal for prefill, no rotary embedding) and SiLU stay in PyTorch.
+    `hook(name, module, x, out)`, when given, is called after every linear with the tensors it consumed and produced."""
 
-    from quik_amd.qlinear import FusedMixedQLinearGroup, SharedQuantizedInput
-    dev = torch.device("cuda:0")
-    B, S, past = BLOCK_WORKLOADS[args.workload]
-    d = BLOCK_DIMS
-    H, heads, kvh, hd, mlp, F = d["hidden"], d["heads"], d["kv_heads"], d["head_dim"], d["mlp"], d["F"]
-    gen = torch.Generator(device=dev).manual_seed(0)
-    fp_h = torch.randperm(H, generator=gen, device=dev)[:F]
-    fp_m = torch.randperm(mlp, generator=gen, device=dev)[:F]
-    sh_qkv, sh_mlp = SharedQuantizedInput(3), SharedQuantizedInput(2)
-    L = {
-        "q": make_device_layer(H, heads * hd, F, 4, fp_h, sh_qkv, gen, dev),
-        "k": make_device_layer(H, kvh * hd, F, 4, fp_h, sh_qkv, gen, dev),
-        "v": make_device_layer(H, kvh * hd, F, 4, fp_h, sh_qkv, gen, dev),
-        "o": make_device_layer(heads * hd, H, F, 4, fp_h, None, gen, dev),
-        "gate": make_device_layer(H, mlp, F, 4, fp_h, sh_mlp, gen, dev),
-        "up": make_device_layer(H, mlp, F, 4, fp_h, sh_mlp, gen, dev),
-        "down": make_device_layer(mlp, H, F, 8, fp_m, None, gen, dev),
-    }
-    # the same weights as two fused groups: one quantize and ONE GEMM for q/k/v and for gate/up
-    import copy
-    members = {n: copy.copy(L[n]) for n in ("q", "k", "v", "gate", "up")}
-    for m in members.values():
-        m.shared_input = None
-    g_qkv = FusedMixedQLinearGroup([members["q"], members["k"], members["v"]])
-    g_mlp = FusedMixedQLinearGroup([members["gate"], members["up"]])
-    norm1 = torch.ones(H, dtype=torch.float16, device=dev)
-    norm2 = torch.ones(H, dtype=torch.float16, device=dev)
-    x = torch.randn(B, S, H, generator=gen, device=dev)
-    x[..., fp_h] *= 50
-    x = x.half()
-    k_cache = torch.randn(B, kvh, past, hd, generator=gen, device=dev).half() if past else None
-    v_cache = torch.randn(B, kvh, past, hd, generator=gen, device=dev).half() if past else None
+    def __init__(self, dev, dims=None, seed=0):
+        import copy
 
+        import torch
+
+        from quik_amd.qlinear import FusedMixedQLinearGroup, SharedQuantizedInput
+        d = dict(BLOCK_DIMS if dims is None else dims)
+        self.dims, self.dev = d, dev
+        H, heads, kvh, hd, mlp, F = d["hidden"], d["heads"], d["kv_heads"], d["head_dim"], d["mlp"], d["F"]
+        gen = torch.Generator(device=dev).manual_seed(seed)
+        self.gen = gen
+        self.fp_h = torch.randperm(H, generator=gen, device=dev)[:F]
+        self.fp_m = torch.randperm(mlp, generator=gen, device=dev)[:F]
+        sh_qkv, sh_mlp = SharedQuantizedInput(3), SharedQuantizedInput(2)
+        self.L = {
+            "q": make_device_layer(H, heads * hd, F, 4, self.fp_h, sh_qkv, gen, dev),
+            "k": make_device_layer(H, kvh * hd, F, 4, self.fp_h, sh_qkv, gen, dev),
+            "v": make_device_layer(H, kvh * hd, F, 4, self.fp_h, sh_qkv, gen, dev),
+            "o": make_device_layer(heads * hd, H, F, 4, self.fp_h, None, gen, dev),
+            "gate": make_device_layer(H, mlp, F, 4, self.fp_h, sh_mlp, gen, dev),
+            "up": make_device_layer(H, mlp, F, 4, self.fp_h, sh_mlp, gen, dev),
+            "down": make_device_layer(mlp, H, F, 8, self.fp_m, None, gen, dev),
+        }
+        members = {n: copy.copy(self.L[n]) for n in ("q", "k", "v", "gate", "up")}
+        for m in members.values():
+            m.shared_input = None
+        self.g_qkv = FusedMixedQLinearGroup([members["q"], members["k"], members["v"]])
+        self.g_mlp = FusedMixedQLinearGroup([members["gate"], members["up"]])
+        self.norm1 = torch.ones(H, dtype=torch.float16, device=dev)
+        self.norm2 = torch.ones(H, dtype=torch.float16, device=dev)
+
+    def inputs(self, B, S, past):
+        """Hidden states with the outlier columns scaled up, and a KV cache of `past` tokens (or None)."""
+        import torch
+        d, dev, gen = self.dims, self.dev, self.gen
+        x = torch.randn(B, S, d["hidden"], generator=gen, device=dev)
+        x[..., self.fp_h] *= 50
+        cache = None
+        if past:
+            cache = tuple(torch.randn(B, d["kv_heads"], past, d["head_dim"], generator=gen, device=dev).half()
+                          for _ in range(2))
+        return x.half(), cache
+
+    @staticmethod
     def rmsnorm(t, w):
+        import torch
         v = t.float()
         return (v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + 1e-5)).half() * w
 
-    def attention(q, k, v):
+    def attention(self, q, k, v, cache):
+        import torch
+        import torch.nn.functional as Fn
+        d = self.dims
+        B, S = q.shape[:2]
+        heads, kvh, hd = d["heads"], d["kv_heads"], d["head_dim"]
         q = q.view(B, S, heads, hd).transpose(1, 2)
         k = k.view(B, S, kvh, hd).transpose(1, 2)
         v = v.view(B, S, kvh, hd).transpose(1, 2)
-        if past:
-            k, v = torch.cat([k_cache, k], 2), torch.cat([v_cache, v], 2)
+        if cache is not None:
+            k, v = torch.cat([cache[0], k], 2), torch.cat([cache[1], v], 2)
         k = k.repeat_interleave(heads // kvh, 1)
         v = v.repeat_interleave(heads // kvh, 1)
-        o = Fn.scaled_dot_product_attention(q, k, v, is_causal=(past == 0 and S > 1))
+        o = Fn.scaled_dot_product_attention(q, k, v, is_causal=(cache is None and S > 1))
         return o.transpose(1, 2).reshape(B, S, heads * hd)
 
-    def block(t, fused_groups):
-        h = rmsnorm(t, norm1)
+    def forward(self, t, fused_groups, cache=None, hook=None):
+        import torch.nn.functional as Fn
+
+        def lin(name, x):
+            out = self.L[name](x)
+            if hook is not None:
+                hook(name, self.L[name], x, out)
+            return out
+
+        h = self.rmsnorm(t, self.norm1)
         if fused_groups:
-            q, k, v = g_qkv(h)
+            q, k, v = self.g_qkv(h)
         else:
-            q, k, v = L["q"](h), L["k"](h), L["v"](h)
-        t = t + L["o"](attention(q, k, v))
-        h = rmsnorm(t, norm2)
+            q, k, v = lin("q", h), lin("k", h), lin("v", h)
+        t = t + lin("o", self.attention(q, k, v, cache))
+        h = self.rmsnorm(t, self.norm2)
         if fused_groups:
-            g, u = g_mlp(h)
+            g, u = self.g_mlp(h)
         else:
-            g, u = L["gate"](h), L["up"](h)
-        return t + L["down"](Fn.silu(g) * u)
+            g, u = lin("gate", h), lin("up", h)
+        return t + lin("down", Fn.silu(g) * u)
+
+
+def bench_block(args):
+    import torch
+
+    dev = torch.device("cuda:0")
+    B, S, past = BLOCK_WORKLOADS[args.workload]
+    blk = DecoderBlock(dev)
+    d, L, gen = blk.dims, blk.L, blk.gen
+    heads, hd, mlp = d["heads"], d["head_dim"], d["mlp"]
+    x, cache = blk.inputs(B, S, past)
 
     # inputs of realistic scale for timing the seven linears alone
-    h_in = rmsnorm(x, norm1)
+    h_in = blk.rmsnorm(x, blk.norm1)
     a_in = torch.randn(B, S, heads * hd, generator=gen, device=dev).half()
     m_in = torch.randn(B, S, mlp, generator=gen, device=dev)
-    m_in[..., fp_m] *= 50
+    m_in[..., blk.fp_m] *= 50
     m_in = m_in.half()
 
     def linears(fused_groups):
         if fused_groups:
-            g_qkv(h_in)
+            blk.g_qkv(h_in)
         else:
             L["q"](h_in), L["k"](h_in), L["v"](h_in)
         L["o"](a_in)
         if fused_groups:
-            g_mlp(h_in)
+            blk.g_mlp(h_in)
         else:
             L["gate"](h_in), L["up"](h_in)
         L["down"](m_in)
@@ -249,11 +311,11 @@ def bench_block(args):
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) * 1e3 / args.steps
 
-    out = block(x, False)
-    out_f = block(x, True)
+    out = blk.forward(x, False, cache)
+    out_f = blk.forward(x, True, cache)
     assert torch.isfinite(out).all() and torch.equal(out, out_f)       # the fused groups give the same bits
-    block_ms = timed(lambda: block(x, False))
-    block_f_ms = timed(lambda: block(x, True))
+    block_ms = timed(lambda: blk.forward(x, False, cache))
+    block_f_ms = timed(lambda: blk.forward(x, True, cache))
     lin_ms = timed(lambda: linears(False))
     lin_f_ms = timed(lambda: linears(True))
     M = B * S
@@ -280,6 +342,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="llama2-70b.gate_proj", choices=sorted(WORKLOADS) + sorted(BLOCK_WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-verify", action="store_true", help="skip the spot check of the output against the CPU oracle")
     ap.add_argument("--unfused", action="store_true", help="run the reference's three-op sequence instead")
     ap.add_argument("--int8-mfma", action="store_true",
                     help="row-major operands on the int8 MFMA kernels instead of the tile-ordered paths (same output bits)")
@@ -364,6 +427,9 @@ def main():
         if ev is not None:
             ev[2].record()
         return out
+
+    # One spot tile of what the timed step computes, against the CPU oracle, outside the timed region.
+    spot = None if (args.no_verify or args.unfused) else verify_spot_tile(name, step(), x_cpu, W_cpu, fp_idx, mod)
 
     for _ in range(args.warmup):
         step()
@@ -483,6 +549,8 @@ def main():
         "pct_int8_mfma_peak": round(100.0 * tops / PEAK_INT8_TOPS, 2),
         "graph_replay_ms_per_step": None if graph_ms is None else round(graph_ms, 4),
         "cold_ms_per_forward": None if cold_ms is None else round(cold_ms, 4),
+        "verified_vs_oracle": None if spot is None else {"tiles": 3, "max_abs_err_over_rms": round(spot, 6),
+                                                         "tolerance": 1e-2},
         "roofline": {"kernel": gemm_kernel,
                      "bound": "mfma", "achieved": round(gemm_tops, 2), "peak": peak,
                      "unit": "TOP/s", "frac": round(gemm_tops / peak, 4),

@@ -138,3 +138,50 @@ def test_default_route_three_dimensional_prefill_input():
     flat = mod(x)[0]
     assert torch.equal(_bits(out.reshape(M, N)), _bits(flat))
     check_against_oracle(flat, x, W, s_w, fi, bits, False, spot_tiles(M, N))
+
+
+def _oracle_module_slice(mod, cols):
+    """The oracle's view of output columns `cols` of a MixedQLinear, from the module's own packed buffers."""
+    c = torch.as_tensor(cols, device=mod.int_weight.device)
+    return {
+        "weights_scales": mod.weights_scales[c].cpu().numpy(),
+        "int_weight": mod.int_weight[c].cpu().numpy(),
+        "int_indices": mod.int_indices.cpu().numpy(),
+        "fp_indices": mod.fp_indices.cpu().numpy(),
+        "fp_weight": mod.fp_weight[c].cpu().numpy(),
+        "reduced_w": mod.reduced_w[:, c].cpu().numpy(),
+    }
+
+
+@pytest.mark.parametrize("B,S,past", [(16, 512, 0), (64, 1, 512)])
+def test_decoder_block_at_llama2_70b_dims(B, S, past):
+    """The full decoder block of the benchmark (bench.DecoderBlock: hidden 8192, 64 heads, 8 KV heads, MLP 28672;
+    seven MixedQLinear, q/k/v and gate/up sharing their quantized inputs, W8A8 down_proj; norms / attention /
+    SiLU in PyTorch), prefill of 16 x 512 tokens and a decode step of 64 single tokens over a 512-token cache.
+    Every linear's output is checked on spot tiles against the oracle's forward of the very tensor that linear
+    consumed (experiments/qlinear.py:80-148 restated on the CPU), and the block with q/k/v and gate/up as fused
+    groups gives the same bits."""
+    import bench
+    blk = bench.DecoderBlock(torch.device(DEV), seed=B)
+    x, cache = blk.inputs(B, S, past)
+    seen = {}
+
+    def hook(name, mod, inp, out):
+        M = B * S
+        assert out.shape == (B, S, mod.out_features) and out.dtype == torch.float16
+        x2, o2 = inp.reshape(M, -1), out.reshape(M, -1)
+        bits = mod.bits
+        for rows, cols in spot_tiles(M, mod.out_features)[:3]:
+            omod = _oracle_module_slice(mod, cols)
+            want, _ = qo.mixed_qlinear_forward(x2[rows].cpu().numpy(), omod, bits)
+            got = o2[rows][:, cols].float().cpu().numpy().astype(np.float64)
+            w64 = want.astype(np.float64)
+            err = np.abs(got - w64).max()
+            assert err <= 1e-2 * np.sqrt((w64 ** 2).mean()), (name, err)
+        seen[name] = True
+
+    out = blk.forward(x, False, cache, hook)
+    assert sorted(seen) == ["down", "gate", "k", "o", "q", "up", "v"]
+    assert torch.isfinite(out).all()
+    out_f = blk.forward(x, True, cache)
+    assert torch.equal(_bits(out), _bits(out_f))
