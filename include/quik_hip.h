@@ -102,8 +102,12 @@ int quik_sym_dequantize(const void *x, int x_bits, const void *scale_row,
  *   out = ((h(acc) * scale_col) * scale_row + (zero_row + h(shift) * scale_row) * w_reduced) + y
  * in fp16 arithmetic, one rounding per operation, exactly as the reference's epilogue
  * (include/asymmetric/epilogue/thread/linear_combination_dequant.h:155-162).
- * Two launches: the exact int32 product goes to acc_workspace ([M, N] int32, caller-provided),
- * the epilogue reads it back. */
+ * One launch: the epilogue runs on the accumulators of the GEMM tiles; no int32 matrix goes through
+ * memory.  Calls with at most 32 rows (quik_fused_dequantize_workspace_bytes(M, N) > 0) run on the
+ * weight-streaming kernel, which has no such epilogue: for those the exact int32 product goes to
+ * acc_workspace ([M, N] int32, caller-provided) and a second launch applies the epilogue; otherwise
+ * acc_workspace may be NULL. */
+int64_t quik_fused_dequantize_workspace_bytes(int64_t M, int64_t N);
 int quik_asym_fused_dequantize(const void *A, const void *B, const void *scale_row,
                                const void *scale_col, float shift_value, const void *zero_row,
                                const void *w_reduced, const void *y, int64_t M, int64_t N,

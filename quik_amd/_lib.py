@@ -29,6 +29,7 @@ SIGNATURES = {
     "quik_asym_fused_dequantize": (_int, [_vp, _vp, _vp, _vp, ctypes.c_float, _vp, _vp, _vp, _i64, _i64, _i64, _int,
                                           _vp, _vp, _vp]),
     "quik_sym_fused_dequantize": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp, _vp, _vp]),
+    "quik_fused_dequantize_workspace_bytes": (_i64, [_i64, _i64]),
     "quik_fp6_operand_bytes": (_i64, [_i64, _i64, _i64]),
     "quik_fp6_pack_weight": (_int, [_vp, _vp, _i64, _i64, _i64, _vp, _vp, _vp]),
     "quik_colmap_streaming": (_int, [_vp, _i64, _i64, _i64, _vp]),

@@ -240,7 +240,9 @@ def _fused_dequantize(op, bits, A, B, scale_row, scale_col, shift_value, zero_ro
             raise RuntimeError(f"{op}: expected {name} to have {n} elements but got {t.numel()}")
     lib = L.load()
     with L.device_guard(A.device):
-        acc = torch.empty((M, N), dtype=torch.int32, device=A.device)
+        # one launch, no int32 matrix; only calls of at most 32 rows (weight-streaming kernel) need the workspace
+        acc = torch.empty((M, N), dtype=torch.int32, device=A.device) \
+            if lib.quik_fused_dequantize_workspace_bytes(M, N) else None
         out = torch.empty((M, N), dtype=torch.float16, device=A.device)
         L.check(lib.quik_asym_fused_dequantize(L.ptr(A), L.ptr(B), L.ptr(scale_row), L.ptr(scale_col),
                                                float(shift_value), L.ptr(zero_row), L.ptr(w_reduced), L.ptr(y), M, N,

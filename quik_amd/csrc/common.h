@@ -15,6 +15,13 @@ int num_cus();       // compute units of the GPU (asked once per process; 256 wh
 
 inline hipStream_t as_stream(void *s) { return reinterpret_cast<hipStream_t>(s); }
 
+// gemm.hip: integer GEMM + the fp16-arithmetic epilogue of the reference's fused ops in one launch (zero_row ==
+// NULL: symmetric form).  Returns kChainNotHandled for shapes it leaves to the two-launch path.
+constexpr int kChainNotHandled = 1;
+int int_gemm_chain(const void *A, const void *B, const void *s_row, const void *s_col, const void *zero_row,
+                   const void *w_red, uint16_t shift_bits, const void *y, int64_t M, int64_t N, int64_t K, int bits,
+                   void *out, hipStream_t st);
+
 // ---- storage types as 16-bit patterns --------------------------------------------------
 // Half values are handled with the native _Float16 type; bfloat16 with explicit bit math
 // so that every rounding is a visible round-to-nearest-even.

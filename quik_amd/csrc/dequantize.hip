@@ -209,13 +209,18 @@ extern "C" int quik_asym_fused_dequantize(const void *A, const void *B, const vo
   if (bits != 4 && bits != 8) return QUIK_ERR_BITS;
   if (M < 0 || N < 0 || K <= 0) return QUIK_ERR_SHAPE;
   if (M == 0 || N == 0) return QUIK_OK;
-  if (!scale_row || !scale_col || !zero_row || !w_reduced || !y || !acc_workspace || !out) return QUIK_ERR_NULL;
-  if (int rc = int_matmul(A, B, acc_workspace, M, N, K, bits, stream)) return rc;
+  if (!scale_row || !scale_col || !zero_row || !w_reduced || !y || !out) return QUIK_ERR_NULL;
+  const _Float16 shift = static_cast<_Float16>(shift_value);
+  const int rc = int_gemm_chain(A, B, scale_row, scale_col, zero_row, w_reduced, __builtin_bit_cast(uint16_t, shift), y,
+                                M, N, K, bits, out, as_stream(stream));
+  if (rc != kChainNotHandled) return rc;
+  // at most 32 rows: product by the weight-streaming kernel into the workspace, epilogue as a second launch
+  if (!acc_workspace) return QUIK_ERR_NULL;
+  if (int rc2 = int_matmul(A, B, acc_workspace, M, N, K, bits, stream)) return rc2;
   hipLaunchKernelGGL(asym_fused_chain_kernel, dim3(grid_for(M * N)), dim3(kThreads), 0, as_stream(stream),
                      acc_workspace, static_cast<const uint16_t *>(scale_row), static_cast<const uint16_t *>(scale_col),
-                     static_cast<_Float16>(shift_value), static_cast<const uint16_t *>(zero_row),
-                     static_cast<const uint16_t *>(w_reduced), static_cast<const uint16_t *>(y), M, N,
-                     static_cast<uint16_t *>(out));
+                     shift, static_cast<const uint16_t *>(zero_row), static_cast<const uint16_t *>(w_reduced),
+                     static_cast<const uint16_t *>(y), M, N, static_cast<uint16_t *>(out));
   return check_launch();
 }
 
@@ -225,7 +230,16 @@ extern "C" int quik_sym_fused_dequantize(const void *A, const void *B, const voi
   if (bits != 4 && bits != 8) return QUIK_ERR_BITS;
   if (M < 0 || N < 0 || K <= 0) return QUIK_ERR_SHAPE;
   if (M == 0 || N == 0) return QUIK_OK;
-  if (!scale_row || !scale_col || !y || !acc_workspace || !out) return QUIK_ERR_NULL;
-  if (int rc = int_matmul(A, B, acc_workspace, M, N, K, bits, stream)) return rc;
+  if (!scale_row || !scale_col || !y || !out) return QUIK_ERR_NULL;
+  const int rc = int_gemm_chain(A, B, scale_row, scale_col, nullptr, nullptr, 0, y, M, N, K, bits, out,
+                                as_stream(stream));
+  if (rc != kChainNotHandled) return rc;
+  if (!acc_workspace) return QUIK_ERR_NULL;
+  if (int rc2 = int_matmul(A, B, acc_workspace, M, N, K, bits, stream)) return rc2;
   return quik_sym_dequantize(acc_workspace, 32, scale_row, scale_col, y, M, N, out, stream);
+}
+
+/* bytes of the int32 workspace the fused dequantize entry points need for this shape (0: none, one launch) */
+extern "C" int64_t quik_fused_dequantize_workspace_bytes(int64_t M, int64_t N) {
+  return (M > 0 && M <= 32 && N > 0) ? M * N * 4 : 0;
 }

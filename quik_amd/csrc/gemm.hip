@@ -292,6 +292,28 @@ int run_i32(const uint8_t *X, const uint8_t *W, int32_t *C, int64_t M, int64_t N
   return launch_i32_split<CfgL, CfgH, MODE>(wide, tail, st);
 }
 
+template <class C, int MODE, bool ASYM>
+int launch_chain(const I32Args &a, const ChainArgs &e, hipStream_t st) {
+  int tiles_m, tiles_n;
+  const int grid = grid_of<C>(a.M, a.N, tiles_m, tiles_n);
+  auto kern = gemm_chain_kernel<C, MODE, ASYM>;
+  if (int rc = prepare(kern, C::SMEM)) return rc;
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(C::kThreads), C::SMEM, st, a, e, tiles_m, tiles_n);
+  return check_launch();
+}
+
+template <int MODE, bool ASYM>
+int run_chain(const I32Args &a, const ChainArgs &e, hipStream_t st) {
+  switch (make_plan(a.M, a.N, a.kbytes % 64 == 0).kind) {
+    case Plan::kSmall: return kChainNotHandled;  // at most 32 rows: the weight-streaming kernel has no such epilogue
+    case Plan::kMid: return launch_chain<CfgM, MODE, ASYM>(a, e, st);
+    case Plan::kNarrow: return launch_chain<CfgN, MODE, ASYM>(a, e, st);
+    case Plan::kMidPlain:
+    case Plan::kLargePlain: return launch_chain<CfgMp, MODE, ASYM>(a, e, st);
+    default: return launch_chain<CfgL, MODE, ASYM>(a, e, st);
+  }
+}
+
 // Tile plan of the 6-bit path (gemm_fp6.h).  Costs in percent of a 256x256 tile, measured at K = 7936, F = 256:
 // a 256x128 tile 59; 128x128 tiles run two to a CU, 66 for a pair, 36 for one that has the CU to itself.
 Plan make_plan6(int64_t M, int64_t N, int64_t min_rows = 33) {
@@ -486,6 +508,23 @@ int run_fused(const FusedArgs &p, hipStream_t st) {
 }
 
 }  // namespace
+
+// Integer GEMM with the fp16-arithmetic epilogue of the reference's fused ops in one launch (see ChainArgs in
+// gemm_kernels.h); kChainNotHandled when the shape belongs to the weight-streaming kernel (at most 32 rows), which
+// has no such epilogue: the caller then runs the product and the epilogue as two launches.
+int int_gemm_chain(const void *A, const void *B, const void *s_row, const void *s_col, const void *zero_row,
+                   const void *w_red, uint16_t shift_bits, const void *y, int64_t M, int64_t N, int64_t K, int bits,
+                   void *out, hipStream_t st) {
+  if (int rc = check_gemm_args(A, B, out, M, N, K, bits)) return rc;
+  I32Args a{static_cast<const uint8_t *>(A), static_cast<const uint8_t *>(B), nullptr, static_cast<int>(M),
+            static_cast<int>(N), static_cast<int>(N), static_cast<int>(bits == 4 ? K / 2 : K)};
+  ChainArgs e{static_cast<const uint16_t *>(s_row), static_cast<const uint16_t *>(s_col),
+              static_cast<const uint16_t *>(zero_row), static_cast<const uint16_t *>(w_red),
+              static_cast<const uint16_t *>(y), static_cast<uint16_t *>(out), static_cast<int>(N), shift_bits};
+  const bool asym = zero_row != nullptr;
+  if (bits == 4) return asym ? run_chain<kInt4, true>(a, e, st) : run_chain<kInt4, false>(a, e, st);
+  return asym ? run_chain<kInt8, true>(a, e, st) : run_chain<kInt8, false>(a, e, st);
+}
 }  // namespace quik
 
 using namespace quik;

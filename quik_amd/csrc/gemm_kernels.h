@@ -476,6 +476,40 @@ struct BlockStore {
     *reinterpret_cast<uint2 *>(stage + (lane & 31) * kRowBytes + (ni * 32 + acc_col(g, lane)) * 2) = make_uint2(lo, hi);
   }
 
+  // the reverse direction: g[row * ld + col] (rows < rows_valid, cols < cols_valid, zeros elsewhere) -> staged block,
+  // as 16-byte pieces of row segments; get() then reads this lane's four consecutive columns (ni, g) of its row
+  static __device__ __forceinline__ void load(uint8_t *stage, int lane, const T *g, int64_t ld, int rows_valid,
+                                              int cols_valid, bool vec) {
+    __builtin_amdgcn_wave_barrier();  // earlier reads of the staging block by other lanes are done (same wave: in order)
+#pragma unroll
+    for (int it = 0; it < 32 / kRowsPerInstr; ++it) {
+      const int r = it * kRowsPerInstr + lane / kLanesPerRow;
+      const int c = (lane % kLanesPerRow) * kElems;
+      v4i piece = v4i{0, 0, 0, 0};
+      if (r < rows_valid) {
+        const T *src = g + int64_t(r) * ld + c;
+        if (vec && c + kElems <= cols_valid) {
+          piece = *reinterpret_cast<const v4i *>(src);
+        } else {
+          T tmp[kElems] = {};
+#pragma unroll
+          for (int e = 0; e < kElems; ++e)
+            if (c + e < cols_valid) tmp[e] = src[e];
+          __builtin_memcpy(&piece, tmp, 16);
+        }
+      }
+      *reinterpret_cast<v4i *>(stage + r * kRowBytes + (lane % kLanesPerRow) * 16) = piece;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+  }
+  static __device__ __forceinline__ void get(const uint8_t *stage, int lane, int ni, int g, T (&v)[4]) {
+    static_assert(sizeof(T) == 2, "16-bit elements");
+    const uint2 w = *reinterpret_cast<const uint2 *>(stage + (lane & 31) * kRowBytes + (ni * 32 + acc_col(g, lane)) * 2);
+    v[0] = static_cast<T>(w.x & 0xFFFFu), v[1] = static_cast<T>(w.x >> 16);
+    v[2] = static_cast<T>(w.y & 0xFFFFu), v[3] = static_cast<T>(w.y >> 16);
+  }
+
   // interior block: the 32 / kRowsPerInstr pieces of a staged block, and their places in global memory
   static constexpr int kIters = 32 / kRowsPerInstr;
   static __device__ __forceinline__ void read_block(const uint8_t *stage, int lane, v4i (&piece)[kIters]) {
@@ -593,6 +627,91 @@ __global__ __launch_bounds__(C::kThreads) void gemm_i32_kernel(I32Args a, int ti
   int tm, tn;
   if (!tile_of_block(blockIdx.x, tiles_m, tiles_n, tm, tn)) return;
   i32_tile<C, MODE>(a, tm, tn, smem);
+}
+
+// ---- the reference's fused GEMM + dequantize ops: exact integer product, fp16-arithmetic epilogue -----------------
+// (reference: src/asymmetric/fused_dequantize.cu:9-119 with include/asymmetric/epilogue/thread/
+// linear_combination_dequant.h:155-162, and src/symmetric/fused_dequantize.cu:9-107 with
+// include/symmetric/epilogue/thread/linear_combination_dequant.h:149-150).  Every operation rounds to fp16:
+//   asymmetric: ((h(acc) * s_col) * s_row + (zero_row + h(shift) * s_row) * w_red) + y
+//   symmetric:  ((h(acc) * s_row) * s_col) + y
+// h(acc): int32 -> fp16, round to nearest even, +-inf above 65519.  One launch: the epilogue runs on the accumulators
+// of the tile (no int32 matrix in memory), y is read and the result written as 16-byte pieces of row segments.
+struct ChainArgs {
+  const uint16_t *s_row, *s_col, *zero_row, *w_red, *y;  // zero_row, w_red: NULL for the symmetric form
+  uint16_t *out;
+  int ldy;          // row stride of y and out in elements
+  uint16_t shift;   // fp16 bit pattern of the shift value (asymmetric)
+};
+
+template <class C, int MODE, bool ASYM>
+__device__ __forceinline__ void chain_tile(const I32Args &a, const ChainArgs &e, int tm, int tn, uint8_t *smem) {
+  const int M = a.M, N = a.N, kbytes = a.kbytes;
+  const int m0 = tm * C::BM, n0 = tn * C::BN;
+  v16i acc[C::MI][C::NI];
+#pragma unroll
+  for (int mi = 0; mi < C::MI; ++mi)
+#pragma unroll
+    for (int ni = 0; ni < C::NI; ++ni)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[mi][ni][v] = 0;
+  run_mainloop<C, MODE>(a.X + int64_t(m0) * kbytes, kbytes, M - m0, a.W + int64_t(n0) * kbytes, kbytes, N - n0, kbytes,
+                        smem, acc);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = wave / C::WAVES_N, wn = wave % C::WAVES_N;
+  constexpr int kShift = MODE == kInt4 ? 8 : 0;
+  using Store = BlockStore<C, uint16_t>;
+  static_assert(Store::kBytes * C::WAVES <= C::SMEM, "staging fits in the (now idle) operand buffers");
+  uint8_t *stage = smem + wave * Store::kBytes;
+  const bool vec = (e.ldy & 7) == 0 && (reinterpret_cast<uintptr_t>(e.out) & 15) == 0 &&
+                   (reinterpret_cast<uintptr_t>(e.y) & 15) == 0;
+  const int nw = n0 + wn * C::WN;
+  auto h = [](uint16_t b) { return __builtin_bit_cast(_Float16, b); };
+  const _Float16 shift = h(e.shift);
+#pragma unroll
+  for (int mi = 0; mi < C::MI; ++mi) {
+    const int mb = m0 + wm * C::WM + mi * 32;
+    if (!(mb < M && nw < N)) continue;  // wave-uniform
+    // y of this 32-row block through the staging area: global -> LDS as row segments, LDS -> this lane's places
+    Store::load(stage, lane, e.y + int64_t(mb) * e.ldy + nw, e.ldy, M - mb, N - nw, vec);
+    const int r = mb + (lane & 31) < M ? mb + (lane & 31) : M - 1;
+    const _Float16 sr = h(e.s_row[r]);
+    _Float16 u0 = static_cast<_Float16>(0);
+    if constexpr (ASYM) u0 = h(e.zero_row[r]) + shift * sr;  // (zero_row + h(shift) * s_row), two roundings
+#pragma unroll
+    for (int ni = 0; ni < C::NI; ++ni)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int c0 = nw + ni * 32 + acc_col(g, lane);
+        uint16_t yv[4], o[4];
+        Store::get(stage, lane, ni, g, yv);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          const int c = c0 + k < N ? c0 + k : N - 1;
+          _Float16 t = static_cast<_Float16>(static_cast<float>(acc[mi][ni][4 * g + k] >> kShift));
+          if constexpr (ASYM) {
+            t = t * h(e.s_col[c]);
+            t = t * sr;
+            t = t + u0 * h(e.w_red[c]);
+          } else {
+            t = t * sr;
+            t = t * h(e.s_col[c]);
+          }
+          t = t + h(yv[k]);
+          o[k] = __builtin_bit_cast(uint16_t, t);
+        }
+        Store::put(stage, lane, ni, g, o);
+      }
+    Store::flush(stage, lane, e.out + int64_t(mb) * e.ldy + nw, e.ldy, M - mb, N - nw, vec);
+  }
+}
+
+template <class C, int MODE, bool ASYM>
+__global__ __launch_bounds__(C::kThreads) void gemm_chain_kernel(I32Args a, ChainArgs e, int tiles_m, int tiles_n) {
+  extern __shared__ __align__(16) uint8_t smem[];
+  int tm, tn;
+  if (!tile_of_block(blockIdx.x, tiles_m, tiles_n, tm, tn)) return;
+  chain_tile<C, MODE, ASYM>(a, e, tm, tn, smem);
 }
 
 // One launch, two tile shapes.  Workgroup ids [lead, lead + wide_blocks) take CW tiles of `wide`,

@@ -79,7 +79,9 @@ def _fused_dequantize(op, bits, A, B, scale_row, scale_col, y):
             raise RuntimeError(f"{op}: expected {name} to have {n} elements but got {t.numel()}")
     lib = L.load()
     with L.device_guard(A.device):
-        acc = torch.empty((M, N), dtype=torch.int32, device=A.device)
+        # one launch, no int32 matrix; only calls of at most 32 rows (weight-streaming kernel) need the workspace
+        acc = torch.empty((M, N), dtype=torch.int32, device=A.device) \
+            if lib.quik_fused_dequantize_workspace_bytes(M, N) else None
         out = torch.empty((M, N), dtype=torch.float16, device=A.device)
         L.check(lib.quik_sym_fused_dequantize(L.ptr(A), L.ptr(B), L.ptr(scale_row), L.ptr(scale_col), L.ptr(y), M, N, K,
                                               bits, L.ptr(acc), L.ptr(out), L.stream()), op)

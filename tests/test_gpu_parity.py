@@ -916,6 +916,48 @@ def test_fused_dequantize_vs_oracle_full_operand_range(bits, spread):
     assert np.array_equal(got[~np.isnan(want)].view(np.uint16), want[~np.isnan(want)].view(np.uint16))
 
 
+@pytest.mark.parametrize("M,N,K", [(33, 40, 64), (100, 130, 96), (257, 300, 512), (300, 8200, 128),
+                                   (2048, 2048 + 136, 256), (1000, 520, 160), (16, 200, 256), (1, 64, 4096)])
+@pytest.mark.parametrize("bits", [4, 8])
+def test_fused_dequantize_is_one_launch_on_every_tile_plan(M, N, K, bits, monkeypatch):
+    """The fused GEMM + dequantize ops run the integer product and the fp16-arithmetic epilogue in ONE launch
+    (src/asymmetric/fused_dequantize.cu:9-119, src/symmetric/fused_dequantize.cu:9-107 of the reference do the
+    same) on every tile shape of the plan, ragged M and N, K that only the plain (non-pipelined) tiles accept; no
+    M x N int32 matrix is allocated.  Calls of at most 32 rows keep the two-launch form (weight-streaming kernel +
+    epilogue kernel).  Bit-exact against the oracle either way."""
+    import quik
+    from quik_amd import _lib as L
+    spread = 8 if bits == 4 else 128
+    a_ref, b_ref, a, b = _fused_operands(bits, M, N, K, spread, M + N + K)
+    rng = np.random.default_rng(M + K)
+    scale_row = rng.uniform(0, 0.1, (M, 1)).astype(np.float16)
+    scale_col = rng.uniform(0, 0.1, (1, N)).astype(np.float16)
+    zero_row = rng.standard_normal((M, 1)).astype(np.float16)
+    w_reduce = rng.standard_normal((1, N)).astype(np.float16)
+    y = rng.standard_normal((M, N)).astype(np.float16)
+    need = L.load().quik_fused_dequantize_workspace_bytes(M, N)
+    assert (need > 0) == (M <= 32)
+    int32_allocs = []
+    real_empty = torch.empty
+
+    def spy(*args, **kw):
+        if kw.get("dtype") == torch.int32:
+            int32_allocs.append(args)
+        return real_empty(*args, **kw)
+    monkeypatch.setattr(torch, "empty", spy)
+    acc = qo.int_matmul(a_ref.cpu().numpy(), b_ref.cpu().numpy())
+    sym = quik.symmetric.int4FusedDequantize if bits == 4 else quik.symmetric.int8FusedDequantize
+    asym = quik.asymmetric.int4FusedDequantize if bits == 4 else quik.asymmetric.int8FusedDequantize
+    got_s = sym(a, b, _t(scale_row), _t(scale_col), _t(y)).cpu().numpy()
+    got_a = asym(a, b, _t(scale_row), _t(scale_col), float(2 ** (bits - 1)), _t(zero_row), _t(w_reduce), _t(y)).cpu().numpy()
+    assert (len(int32_allocs) == 0) == (M > 32)
+    for got, want in ((got_s, qo.sym_dequantize(acc, scale_row, scale_col, y, 32)),
+                      (got_a, qo.asym_fused_dequantize(acc, scale_row, scale_col, float(2 ** (bits - 1)), zero_row,
+                                                       w_reduce, y))):
+        assert np.array_equal(np.isnan(got), np.isnan(want))
+        assert np.array_equal(got[~np.isnan(want)].view(np.uint16), want[~np.isnan(want)].view(np.uint16))
+
+
 # ------------------------------------------------------------------------------ 6-bit matrix-core path
 def _decode_operand6(buf, rows, K, F):
     """Operand buffer of the 6-bit path -> (levels [rows, K], outlier bit patterns [rows, F], level sums [rows]),
