@@ -391,11 +391,10 @@ def main():
     from quik_amd import asymmetric, matmul
     colmap = mod._column_map()
     # the path MixedQLinear.forward takes: tile-ordered operands (4 bits: 6-bit matrix-core GEMM, 8 bits: int8 MFMA)
-    six = mod.fused and not args.int8_mfma and mod._six_bit_ok(M)
-    w6 = mod._weight6() if six else None
-
+    if args.int8_mfma:
+        mod.six_bit_path = False          # row-major operands on the int8 MFMA kernels
+    six = mod._six_bit_ok(M)
     quantize6 = asymmetric.quantize_mapped_fp6 if bits == 4 else asymmetric.quantize_mapped_tile8
-    linear6 = matmul.mixed_linear_fp6 if bits == 4 else matmul.mixed_linear_tile8
 
     def quantize_only():
         if six:
@@ -403,27 +402,27 @@ def main():
         return asymmetric.quantize_mapped(x, colmap, K, F, bits)
 
     def step(ev=None):
+        """One forward of the layer.  Fused (the default): ONE call of the module, mod(x) -> quik_layer_forward, which
+        launches the quantize kernel and the fused GEMM; ev = (event recorded by the library between the two
+        launches, event recorded after the call), both on the launch stream.  --unfused: the reference's op sequence
+        through the stand-alone ops, ev = (before, between, after)."""
+        if mod.fused:
+            if ev is not None:
+                mod.mid_event = ev[0]
+            out = mod(x)[0]
+            if ev is not None:
+                assert mod.mid_event is None, "the forward did not go through the one-call path"
+                ev[1].record()
+            return out
         if ev is not None:
             ev[0].record()
-        if six:
-            x6, meta = quantize6(x, colmap, K, F)
-            if ev is not None:
-                ev[1].record()
-            out = linear6(x6, w6, meta, mod.weights_scales, mod.reduced_w, mod.bias, M, N, K, F, torch.float16)
-            if ev is not None:
-                ev[2].record()
-            return out
         q, meta, fp = asymmetric.quantize_mapped(x, colmap, K, F, bits)
         if ev is not None:
             ev[1].record()
-        if mod.fused:
-            out = matmul.mixed_linear(q, mod.int_weight, meta, mod.weights_scales, mod.reduced_w, fp, mod.fp_weight,
-                                      mod.bias, bits, torch.float16)
-        else:
-            from quik_amd.qlinear import SharedQuantizedInput
-            sh = SharedQuantizedInput(1)
-            sh.qint_x, sh.meta, sh.fp_x = q, meta, fp
-            out = mod._forward_unfused(sh)
+        from quik_amd.qlinear import SharedQuantizedInput
+        sh = SharedQuantizedInput(1)
+        sh.qint_x, sh.meta, sh.fp_x = q, meta, fp
+        out = mod._forward_unfused(sh)
         if ev is not None:
             ev[2].record()
         return out
@@ -434,7 +433,11 @@ def main():
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
-    events = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    n_ev = 2 if mod.fused else 3
+    events = [[torch.cuda.Event(enable_timing=True) for _ in range(n_ev)] for _ in range(args.steps)]
+    for evs in events:                 # an event has a handle only once it has been recorded
+        for e in evs:
+            e.record()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(args.steps):
@@ -442,8 +445,14 @@ def main():
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     ms_step = (t1 - t0) * 1e3 / args.steps
-    q_ms = sorted(e[0].elapsed_time(e[1]) for e in events)
-    g_ms = sorted(e[1].elapsed_time(e[2]) for e in events)
+    if mod.fused:
+        # GEMM launch: between-event -> after-event of the same step; quantize launch: after-event of the previous
+        # step -> between-event (this interval also holds the gap between two forwards)
+        g_ms = sorted(e[0].elapsed_time(e[1]) for e in events)
+        q_ms = sorted(events[i - 1][1].elapsed_time(events[i][0]) for i in range(1, args.steps)) or [0.0]
+    else:
+        q_ms = sorted(e[0].elapsed_time(e[1]) for e in events)
+        g_ms = sorted(e[1].elapsed_time(e[2]) for e in events)
     q_avg, g_avg = sum(q_ms) / len(q_ms), sum(g_ms) / len(g_ms)
 
     # the quantize kernel alone, launched back to back (outside the timed region)
@@ -455,6 +464,18 @@ def main():
     torch.cuda.synchronize()
     q_b2b = e0.elapsed_time(e1) / 50
     traffic = MEASURED_TRAFFIC_BYTES.get(name, {})
+
+    # the same forward without the two event records per step: the figure a caller of the module sees
+    module_ms = None
+    if mod.fused:
+        for _ in range(3):
+            mod(x)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            mod(x)
+        torch.cuda.synchronize()
+        module_ms = (time.perf_counter() - t0) * 1e3 / args.steps
 
     # the same step replayed from a HIP graph (extra figure: what a serving loop that captures the layer sees;
     # for small token counts the eager step is bound by Python launch overhead, not by the kernels)
@@ -547,6 +568,7 @@ def main():
                                f"{', 6-bit matrix-core path' if six and bits == 4 else ', tile-ordered operands' if six else ''}",
                    "M": M, "in_features": n_in, "K": K, "N": N, "F": F, "bits": bits},
         "pct_int8_mfma_peak": round(100.0 * tops / PEAK_INT8_TOPS, 2),
+        "module_forward_ms_per_step": None if module_ms is None else round(module_ms, 4),
         "graph_replay_ms_per_step": None if graph_ms is None else round(graph_ms, 4),
         "cold_ms_per_forward": None if cold_ms is None else round(cold_ms, 4),
         "verified_vs_oracle": None if spot is None else {"tiles": 3, "max_abs_err_over_rms": round(spot, 6),
@@ -558,17 +580,19 @@ def main():
                      "traffic": traffic.get("gemm6" if six else "gemm") if mod.fused else None,
                      "avg_ms": round(g_avg, 4), "median_ms": round(g_ms[len(g_ms) // 2], 4),
                      "algorithmic_ops": int_ops},
-        "roofline_quantize": {"kernel": "asym_quantize_stream_kernel" + (" (tile-ordered operand output)" if six else ""),
+        "roofline_quantize": {"kernel": ("quantize_fp6_wave_kernel (one wave per token row, 6-bit operand output)" if six and bits == 4
+                                         else "asym_quantize_stream_kernel" + (" (tile-ordered operand output)" if six else "")),
                               "bound": "hbm",
                               "achieved": round(quant_gbps, 1),
                               "peak": PEAK_HBM_GBPS, "unit": "GB/s", "frac": round(quant_gbps / PEAK_HBM_GBPS, 4),
                               "traffic": traffic.get("quantize6" if six else "quantize"), "avg_ms": round(q_avg, 5),
                               "median_ms": round(q_ms[len(q_ms) // 2], 5), "algorithmic_bytes": quant_bytes,
                               "back_to_back_ms": round(q_b2b, 5),
-                              "note": "avg_ms: two event records around one ~15 us launch inside the step "
-                                      "(includes several us of event overhead); back_to_back_ms: per launch over "
-                                      "50 consecutive launches after the timed region, input warm in the "
-                                      "Infinity Cache"},
+                              "note": "avg_ms: from the event after the previous forward to the event the library "
+                                      "records between the quantize launch and the GEMM launch (the launch plus the "
+                                      "gap between two forwards); back_to_back_ms: per launch over 50 consecutive "
+                                      "launches after the timed region (bound by the host: ~14 us of Python per "
+                                      "call); kernel-trace durations: profiles/"},
     }
     if not args.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline(name, x_cpu, W_cpu, int_idx, fp_idx)

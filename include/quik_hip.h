@@ -227,6 +227,39 @@ int quik_mixed_linear_fwd_tile8_ws(const void *x8, const void *w8, const void *m
                                    int64_t K, int64_t F, void *out, void *workspace, int64_t workspace_bytes,
                                    void *stream);
 
+/* ---- one call per layer forward -----------------------------------------------------------------------
+ * replaces the op sequence of MixedQLinear.forward, experiments/qlinear.py:80-148 (quantize, integer GEMM,
+ * F.linear on the outlier columns, dequantize), for callers that want one boundary crossing per layer:
+ * at decode sizes the kernels take 20 us and every crossing from an interpreter costs several.
+ * quik_layer describes the layer's buffers once (all device pointers; the same buffers MixedQLinear
+ * registers, qlinear.py:53-78); a forward picks the kernels as MixedQLinear does here: up to
+ * tiled_min_rows - 1 rows the row-major quantize + quik_mixed_linear_fwd (weight-streaming kernel up to 32
+ * rows), from tiled_min_rows rows the tile-ordered paths when tiled_weight is given and the shape allows.
+ *   struct_bytes    sizeof(quik_layer), checked
+ *   bits 4 | 8; dtype QUIK_F16 | QUIK_BF16; symmetric 0 | 1 (fp16 and a streaming column map only)
+ *   colmap          quik_colmap_build(...) for (in_features, num_int, num_fp); colmap_streams: what
+ *                   quik_colmap_streaming returned for it
+ *   int_weight [out, num_int/2] u8 or [out, num_int] i8; weights_scales [out]; reduced_w [out] (NULL when
+ *   symmetric); fp_weight [out, num_fp] (NULL when num_fp == 0); bias [out] or NULL
+ *   tiled_weight    quik_fp6_pack_weight (bits 4) / quik_tile8_pack_weight (bits 8) buffer, or NULL
+ *   tiled_min_rows  33 is what MixedQLinear uses
+ * workspace: quik_layer_workspace_bytes(layer, rows) bytes, 256-byte aligned, holds the quantized activation
+ * between the two launches; splitk_workspace as for the _ws entry points (may be NULL).
+ * mid_event: NULL, or a hipEvent_t that is recorded on the stream between the quantize launch and the
+ * GEMM launch (profiling hook: lets a caller time the two kernels of a one-call forward).
+ * x [rows, in_features] dtype, out [rows, out_features] dtype. */
+typedef struct quik_layer {
+  int32_t struct_bytes, bits, dtype, symmetric;
+  int64_t in_features, num_int, num_fp, out_features;
+  float sym_divisor;
+  int32_t colmap_streams, tiled_min_rows, reserved;
+  const void *colmap, *int_weight, *weights_scales, *reduced_w, *fp_weight, *bias, *tiled_weight;
+} quik_layer;
+int64_t quik_layer_workspace_bytes(const quik_layer *layer, int64_t rows);
+int quik_layer_forward(const quik_layer *layer, const void *x, int64_t rows, void *workspace,
+                       int64_t workspace_bytes, void *splitk_workspace, int64_t splitk_bytes, void *out,
+                       void *mid_event, void *stream);
+
 /* ---- the reference's simulated (fake-quant) activation path ---------------------------------------
  * replaces the tensor-op sequence of ActQuantWrapper.forward, experiments/quant_sim.py:227-256
  * (ActQuantizer.find_params :167-188, asymmetric_quantize :5-7), which the reference uses for its

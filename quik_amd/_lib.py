@@ -46,6 +46,8 @@ SIGNATURES = {
                                             _vp]),
     "quik_mixed_linear_fwd_tile8_ws": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _i64, _vp, _vp, _i64,
                                               _vp]),
+    "quik_layer_workspace_bytes": (_i64, [_vp, _i64]),
+    "quik_layer_forward": (_int, [_vp, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp]),
     "quik_sim_act_fake_quant": (_int, [_vp, _int, _i64, _i64, _vp, _int, _vp, _vp]),
     "quik_mixed_linear_fwd_tile8_noalloc": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _i64, _vp, _vp]),
     "quik_int4_matmul": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
@@ -53,6 +55,17 @@ SIGNATURES = {
     "quik_mixed_linear_fwd": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _i64, _int,
                                      _vp, _vp]),
 }
+
+
+
+class QuikLayer(ctypes.Structure):
+    """struct quik_layer of include/quik_hip.h."""
+    _fields_ = [("struct_bytes", ctypes.c_int32), ("bits", ctypes.c_int32), ("dtype", ctypes.c_int32),
+                ("symmetric", ctypes.c_int32), ("in_features", _i64), ("num_int", _i64), ("num_fp", _i64),
+                ("out_features", _i64), ("sym_divisor", ctypes.c_float), ("colmap_streams", ctypes.c_int32),
+                ("tiled_min_rows", ctypes.c_int32), ("reserved", ctypes.c_int32), ("colmap", _vp), ("int_weight", _vp),
+                ("weights_scales", _vp), ("reduced_w", _vp), ("fp_weight", _vp), ("bias", _vp), ("tiled_weight", _vp)]
+
 
 _lib = None
 

@@ -17,9 +17,12 @@ reference (experiments/qlinear.py:21-199), so `llama_replace_with_kernels`
 """
 from __future__ import annotations
 
+import ctypes
+
 import torch
 from torch import Tensor
 
+from . import _lib as L
 from . import asymmetric, matmul, symmetric
 from ._lib import device_guard
 
@@ -35,6 +38,16 @@ def pack_to_i4(X: Tensor) -> Tensor:
     """Signed int4 codes [R, K] (K even) -> uint8 [R, K/2], even element in the low nibble."""
     u = two_compl(X.to(dtype=torch.int8), 4).to(torch.uint8)
     return u[:, 0::2] | (u[:, 1::2] << 4)
+
+
+class _PerObjectCache(dict):
+    """A cache that copies of its owner do not inherit (it holds ctypes structures with raw pointers)."""
+
+    def __copy__(self):
+        return _PerObjectCache()
+
+    def __deepcopy__(self, memo):
+        return _PerObjectCache()
 
 
 class SharedQuantizedInput:
@@ -73,6 +86,10 @@ class MixedQLinear(torch.nn.Module):
     1 byte per weight).  Both need fp_features % 32 == 0 and ascending int_indices and give the output bits
     of the row-major kernels; `six_bit_path = False` turns them off."""
 
+    # Profiling hook: a torch.cuda.Event (created, i.e. recorded once before) stored here is recorded between the
+    # quantize launch and the GEMM launch of the next forward that goes through the one-call path, then cleared.
+    mid_event = None
+
     six_bit_min_rows = 33    # up to 32 rows the weight-streaming decode kernel on the packed int4 weights is the right one
     tile8_min_rows = 33      # the same switch for 8 bits (the tile-ordered kernel itself takes any row count)
 
@@ -108,6 +125,7 @@ class MixedQLinear(torch.nn.Module):
             self.register_buffer('reduced_w', torch.zeros((1, out_features), dtype=dtype))
         self._colmap = None
         self._colmap_key = None
+        self._descs = _PerObjectCache()
 
     # -- cached column map: rebuilt when the index buffers move or are written in place
     def _column_map(self):
@@ -160,6 +178,61 @@ class MixedQLinear(torch.nn.Module):
             self._streams = flag
         return self._streams
 
+    # -- one library call per forward (quik_layer_forward): the layer's buffers described once
+    def _descriptor(self, tiled):
+        """(ctypes quik_layer, workspace sizes by row count) for this module, with or without the tile-ordered weight
+        copy; cached, rebuilt when a buffer moves or is written in place."""
+        bufs = (self.int_weight, self.weights_scales, self.int_indices, self.fp_indices,
+                self.reduced_w if not self.symmetric else None, self.fp_weight if self.fp_features_num > 0 else None,
+                self.bias)
+        key = tuple((b.data_ptr(), b._version) if b is not None else None for b in bufs)
+        entry = self._descs.get(tiled)
+        if entry is None or entry[0] != key:
+            w6 = self._weight6() if tiled else None
+            colmap = self._column_map()
+            d = L.QuikLayer()
+            d.struct_bytes = ctypes.sizeof(L.QuikLayer)
+            d.bits, d.symmetric = self.bits, int(self.symmetric)
+            d.dtype = L.QUIK_F16 if self.dtype == torch.float16 else L.QUIK_BF16
+            d.in_features, d.num_int, d.num_fp = self.in_features, self.int_features_num, self.fp_features_num
+            d.out_features = self.out_features
+            d.sym_divisor = float(self.sym_divisor)
+            d.colmap_streams = int(self._streams_flag())
+            d.tiled_min_rows = self.six_bit_min_rows if self.bits == 4 else self.tile8_min_rows
+            d.colmap, d.int_weight, d.weights_scales = colmap.data_ptr(), bufs[0].data_ptr(), bufs[1].data_ptr()
+            d.reduced_w = bufs[4].data_ptr() if bufs[4] is not None else None
+            d.fp_weight = bufs[5].data_ptr() if bufs[5] is not None else None
+            d.bias = bufs[6].data_ptr() if bufs[6] is not None and bufs[6].numel() > 0 else None
+            d.tiled_weight = w6.data_ptr() if w6 is not None else None
+            entry = self._descs[tiled] = (key, d, {}, (colmap, w6))   # the tensors the pointers refer to stay alive
+        return entry[1], entry[2]
+
+    def _forward_one_call(self, x2):
+        """quantize + fused GEMM through quik_layer_forward; None when this call is not one it serves."""
+        if x2.dtype != self.dtype or x2.data_ptr() % 16 != 0 or self.dtype not in (torch.float16, torch.bfloat16):
+            return None
+        if self.symmetric and not (self.dtype == torch.float16 and self._streams_flag()):
+            return None
+        rows = x2.shape[0]
+        if rows == 0:
+            return None
+        tiled = self._six_bit_ok(rows)
+        desc, ws_bytes = self._descriptor(tiled)
+        lib = L.load()
+        nbytes = ws_bytes.get(rows)
+        if nbytes is None:
+            nbytes = ws_bytes[rows] = lib.quik_layer_workspace_bytes(ctypes.byref(desc), rows)
+        ws = torch.empty((nbytes,), dtype=torch.uint8, device=x2.device)
+        out = torch.empty((rows, self.out_features), dtype=self.dtype, device=x2.device)
+        sk, sk_bytes = matmul._splitk_workspace(x2.device, rows, self.out_features, self.int_features_num, self.bits) \
+            if tiled else (None, 0)
+        mid = None
+        if self.mid_event is not None:   # profiling hook, see the class comment
+            mid, self.mid_event = self.mid_event.cuda_event, None
+        L.check(lib.quik_layer_forward(ctypes.byref(desc), x2.data_ptr(), rows, ws.data_ptr(), nbytes, L.ptr(sk),
+                                       sk_bytes, out.data_ptr(), mid, L.stream()), "MixedQLinear.forward")
+        return out
+
     def _quantize_input(self, x, shared_input):
         if self.symmetric and x.dtype == torch.float16 and x.data_ptr() % 16 == 0 and self._streams_flag():
             # the op sequence of the next branch in one kernel, same bits
@@ -190,6 +263,11 @@ class MixedQLinear(torch.nn.Module):
         x2 = x.reshape(-1, x.shape[-1])
         if not x2.is_contiguous():
             x2 = x2.contiguous()
+        if self.fused and (self.shared_input is None or self.shared_input.group_size == 1):
+            with device_guard(x.device):
+                output = self._forward_one_call(x2)
+            if output is not None:
+                return output.reshape(*lead, self.out_features)
         shared_input = self.shared_input if self.shared_input is not None else SharedQuantizedInput(1)
         with device_guard(x.device):
             if x2.data_ptr() % 16 == 0 and (not self.symmetric or x2.dtype == torch.float16) \

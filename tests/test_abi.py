@@ -194,3 +194,54 @@ def test_from_float_buffers_on_cpu():
     assert pack_to_i4(torch.tensor([[-8, 7]])).tolist() == [[0x78]]
     with pytest.raises(AssertionError, match="duplication"):
         MixedQLinear.from_float(lin, torch.from_numpy(W), torch.from_numpy(s_w), None, torch.tensor([1, 1]), bits=4)
+
+
+def test_layer_forward_validates_without_gpu():
+    """quik_layer_forward / quik_layer_workspace_bytes check the descriptor, the pointers, their alignment and the
+    workspace size before any HIP call."""
+    from quik_amd import _lib as L
+    lib = L.load()
+    null = ctypes.c_void_p(None)
+    one, odd = ctypes.c_void_p(256), ctypes.c_void_p(264)
+
+    def layer(**kw):
+        d = L.QuikLayer()
+        d.struct_bytes = ctypes.sizeof(L.QuikLayer)
+        d.bits, d.dtype, d.symmetric = 4, L.QUIK_F16, 0
+        d.in_features, d.num_int, d.num_fp, d.out_features = 8192, 7936, 256, 1024
+        d.sym_divisor, d.colmap_streams, d.tiled_min_rows = 4.0, 1, 33
+        d.colmap = d.int_weight = d.weights_scales = d.reduced_w = d.fp_weight = 256
+        for k, v in kw.items():
+            setattr(d, k, v)
+        return d
+
+    fwd = lambda d, x=one, rows=64, ws=one, nb=1 << 30, out=one: lib.quik_layer_forward(
+        ctypes.byref(d), x, rows, ws, nb, null, 0, out, null, null)
+    a256 = lambda v: (v + 255) // 256 * 256
+    # row-major plan: packed codes, (scale, zero) per row, outlier values; every section 256-byte aligned
+    d = layer()
+    assert lib.quik_layer_workspace_bytes(ctypes.byref(d), 20) == a256(20 * 7936 // 2) + a256(20 * 4) + a256(20 * 256 * 2)
+    assert lib.quik_layer_workspace_bytes(ctypes.byref(d), 64) == a256(64 * 7936 // 2) + a256(64 * 4) + a256(64 * 256 * 2)
+    # tile-ordered plan once the layer has a tile-ordered weight copy and enough rows: operand buffer + (scale, zero)
+    t = layer(tiled_weight=256)
+    assert lib.quik_layer_workspace_bytes(ctypes.byref(t), 64) == \
+        a256(lib.quik_fp6_operand_bytes(64, 7936, 256)) + a256(64 * 4)
+    assert lib.quik_layer_workspace_bytes(ctypes.byref(t), 32) == lib.quik_layer_workspace_bytes(ctypes.byref(d), 32)
+    t8 = layer(bits=8, tiled_weight=256, in_features=28672, num_int=28416)
+    assert lib.quik_layer_workspace_bytes(ctypes.byref(t8), 64) == \
+        a256(lib.quik_tile8_operand_bytes(64, 28416, 256)) + a256(64 * 4)
+    assert lib.quik_layer_workspace_bytes(ctypes.byref(layer(struct_bytes=8)), 64) == 0
+    assert lib.quik_layer_workspace_bytes(ctypes.byref(d), 0) == 0
+    assert fwd(layer(struct_bytes=8)) == -2                  # a descriptor of another layout
+    assert fwd(layer(bits=5)) == -2
+    assert fwd(layer(num_fp=255)) == -2                      # num_int + num_fp != in_features
+    assert fwd(d, rows=-1) == -2
+    assert fwd(d, rows=0) == 0                               # empty batch
+    assert fwd(d, x=null) == -5
+    assert fwd(d, out=null) == -5
+    assert fwd(layer(reduced_w=None)) == -5                  # asymmetric needs the reduced weights
+    assert fwd(layer(fp_weight=None)) == -5
+    assert fwd(d, x=ctypes.c_void_p(264)) == -4
+    assert fwd(d, ws=odd) == -4
+    assert fwd(d, nb=1024) == -6                             # workspace too small
+    assert fwd(layer(symmetric=1, dtype=L.QUIK_BF16)) == -3  # symmetric activations are fp16

@@ -1,0 +1,180 @@
+"""quik_layer_forward: one library call per MixedQLinear forward (quantize launch + fused GEMM launch).
+
+The entry point replaces the op sequence of MixedQLinear.forward (experiments/qlinear.py:80-148 of the reference)
+for callers that want one crossing into the library per layer.  Checks:
+  * through the C ABI, with a descriptor and a workspace built by the test, the output bits equal those of the
+    stand-alone entry points called one after the other (which tests/test_gpu_parity.py holds against the oracle);
+  * `MixedQLinear.forward` takes this path by default and gives the bits of the module's op-by-op route;
+  * the oracle's forward on the same inputs, within 1e-2 x output RMS;
+  * the profiling event is recorded between the two launches, on the launch stream.
+"""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import quik_oracle as qo
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _lib():
+    from quik_amd import _lib as L
+    L.load()
+    assert torch.cuda.is_available()
+    yield
+
+
+def _bits(t):
+    return t.detach().contiguous().view(torch.int16)
+
+
+def _layer(rng, N, n_in, F, bits):
+    fi = np.sort(rng.permutation(n_in)[:F]).astype(np.int64)
+    keep = np.ones(n_in, bool)
+    keep[fi] = False
+    ii = np.arange(n_in)[keep]
+    lo, hi = (-8, 8) if bits == 4 else (-127, 128)
+    s_w = rng.uniform(0.001, 0.01, (N, 1)).astype(np.float16)
+    W = np.zeros((N, n_in), np.float16)
+    W[:, ii] = (rng.integers(lo, hi, (N, n_in - F)) * s_w.astype(np.float32)).astype(np.float16)
+    W[:, fi] = (0.02 * rng.standard_normal((N, F))).astype(np.float16)
+    return W, s_w, fi
+
+
+def _module(W, s_w, fi, bits, bias, symm, dtype=torch.float16):
+    from quik_amd.qlinear import MixedQLinear
+    N, n_in = W.shape
+    lin = torch.nn.Linear(n_in, N, bias=bias is not None)
+    if bias is not None:
+        lin.bias.data = torch.from_numpy(bias)
+    mod = MixedQLinear.from_float(lin, torch.from_numpy(W).to(dtype), torch.from_numpy(s_w).to(dtype), None,
+                                  torch.from_numpy(fi) if fi.size else None, symm=symm, bits=bits)
+    return mod.to(DEV)
+
+
+CASES = [
+    # rows, out, in, outliers, bits, symmetric, bias
+    (1, 384, 1024, 64, 4, False, False),      # decode kernel
+    (20, 200, 1056, 32, 4, False, True),
+    (32, 256, 2048 + 256, 256, 8, False, False),
+    (33, 300, 1024 + 64, 64, 4, False, True),  # first row count on the tile-ordered path
+    (200, 520, 4096 + 128, 128, 4, False, False),
+    (260, 300, 1280 + 256, 256, 8, False, True),
+    (48, 256, 1024 + 32, 32, 4, True, False),  # symmetric activations, tile-ordered
+    (8, 256, 1024 + 32, 32, 4, True, True),    # symmetric activations, decode kernel
+    (100, 128, 1000, 40, 4, False, True),      # K % 128 != 0: row-major operands at any row count
+    (64, 128, 512, 0, 4, False, True),         # no outliers
+]
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_module_forward_is_one_call_and_matches_the_op_sequence(case, monkeypatch):
+    M, N, n_in, F, bits, symm, with_bias = case
+    rng = np.random.default_rng(sum(case[:5]) + symm)
+    W, s_w, fi = _layer(rng, N, n_in, F, bits)
+    bias = rng.standard_normal(N).astype(np.float16) if with_bias else None
+    x = rng.standard_normal((M, n_in)).astype(np.float32)
+    x[:, fi] *= 50
+    x = x.astype(np.float16)
+    mod = _module(W, s_w, fi, bits, bias, symm)
+    xt = torch.from_numpy(x).to(DEV)
+
+    from quik_amd import _lib as L
+    calls = []
+    real = L.load().quik_layer_forward
+    monkeypatch.setattr(L.load(), "quik_layer_forward", lambda *a: calls.append(a[2]) or real(*a))
+    out = mod(xt)
+    assert calls == [M]                          # the module went through the one-call entry point
+    assert out.shape == (1, M, N) and out.dtype == torch.float16
+
+    monkeypatch.setattr(type(mod), "_forward_one_call", lambda self, x2: None)
+    ref = mod(xt)                                # the module's op-by-op route: two library calls
+    assert calls == [M]
+    assert torch.equal(_bits(out), _bits(ref))
+
+    omod = qo.from_float(W, s_w, fi, bits, symm=symm)
+    want, _ = qo.mixed_qlinear_forward(x, omod, bits, bias, symm=symm)
+    w64 = want.astype(np.float64)
+    err = np.abs(out[0].float().cpu().numpy().astype(np.float64) - w64).max()
+    assert err <= 1e-2 * np.sqrt((w64 ** 2).mean())
+    assert err <= 4 * np.abs(w64).max() * 2.0 ** -10
+
+
+def test_bfloat16_module_takes_the_one_call_path():
+    M, N, n_in, F, bits = 70, 256, 2048 + 64, 64, 4
+    rng = np.random.default_rng(3)
+    W, s_w, fi = _layer(rng, N, n_in, F, bits)
+    mod = _module(W, s_w, fi, bits, None, False, dtype=torch.bfloat16)
+    x = torch.from_numpy(rng.standard_normal((M, n_in)).astype(np.float32)).to(torch.bfloat16).to(DEV)
+    out = mod(x)
+    assert out.dtype == torch.bfloat16
+    type(mod)._forward_one_call, keep = (lambda self, x2: None), type(mod)._forward_one_call
+    try:
+        ref = mod(x)
+    finally:
+        type(mod)._forward_one_call = keep
+    assert torch.equal(_bits(out), _bits(ref))
+
+
+@pytest.mark.parametrize("M,bits", [(16, 4), (96, 4), (96, 8)])
+def test_layer_forward_through_the_c_abi(M, bits):
+    """Descriptor, workspace and call made by hand, as a C caller would; against the stand-alone entry points."""
+    from quik_amd import _lib as L, asymmetric, matmul
+    lib = L.load()
+    N, n_in, F = 320, 2048 + 64, 64
+    K = n_in - F
+    rng = np.random.default_rng(M + bits)
+    W, s_w, fi = _layer(rng, N, n_in, F, bits)
+    mod = _module(W, s_w, fi, bits, None, False)
+    x = torch.from_numpy(rng.standard_normal((M, n_in)).astype(np.float16)).to(DEV)
+    colmap = asymmetric.build_colmap(mod.int_indices, mod.fp_indices, n_in)
+    assert asymmetric.colmap_streams(colmap, K, F)
+    tiled = M >= 33
+    w_t = None
+    if tiled:
+        w_t = matmul.pack_weight_fp6(mod.int_weight, mod.fp_weight, colmap) if bits == 4 else \
+            matmul.pack_weight_tile8(mod.int_weight, mod.fp_weight)
+
+    d = L.QuikLayer()
+    d.struct_bytes = ctypes.sizeof(L.QuikLayer)
+    d.bits, d.dtype, d.symmetric = bits, L.QUIK_F16, 0
+    d.in_features, d.num_int, d.num_fp, d.out_features = n_in, K, F, N
+    d.sym_divisor, d.colmap_streams, d.tiled_min_rows = 4.0, 1, 33
+    d.colmap, d.int_weight, d.weights_scales = colmap.data_ptr(), mod.int_weight.data_ptr(), mod.weights_scales.data_ptr()
+    d.reduced_w, d.fp_weight = mod.reduced_w.data_ptr(), mod.fp_weight.data_ptr()
+    d.tiled_weight = w_t.data_ptr() if tiled else None
+    nbytes = lib.quik_layer_workspace_bytes(ctypes.byref(d), M)
+    assert nbytes > 0
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=DEV)
+    out = torch.empty(M, N, dtype=torch.float16, device=DEV)
+    before, mid, after = (torch.cuda.Event(enable_timing=True) for _ in range(3))
+    mid.record()                                 # an event has a handle once it has been recorded
+    torch.cuda.synchronize()
+    before.record()
+    rc = lib.quik_layer_forward(ctypes.byref(d), x.data_ptr(), M, ws.data_ptr(), nbytes, None, 0, out.data_ptr(),
+                                mid.cuda_event, L.stream())
+    after.record()
+    assert rc == 0, lib.quik_status_string(rc)
+    torch.cuda.synchronize()
+    # the event sits between the two launches on the launch stream
+    assert before.elapsed_time(mid) > 0 and mid.elapsed_time(after) > 0
+
+    if tiled and bits == 4:
+        q, meta = asymmetric.quantize_mapped_fp6(x, colmap, K, F)
+        ref = matmul.mixed_linear_fp6(q, w_t, meta, mod.weights_scales, mod.reduced_w, None, M, N, K, F, torch.float16)
+    elif tiled:
+        q, meta = asymmetric.quantize_mapped_tile8(x, colmap, K, F)
+        ref = matmul.mixed_linear_tile8(q, w_t, meta, mod.weights_scales, mod.reduced_w, None, M, N, K, F, torch.float16)
+    else:
+        q, meta, fp = asymmetric.quantize_mapped(x, colmap, K, F, bits)
+        ref = matmul.mixed_linear(q, mod.int_weight, meta, mod.weights_scales, mod.reduced_w, fp, mod.fp_weight, None,
+                                  bits, torch.float16)
+    assert torch.equal(_bits(out), _bits(ref))
+    # a workspace one byte short is refused before anything is launched
+    assert lib.quik_layer_forward(ctypes.byref(d), x.data_ptr(), M, ws.data_ptr(), nbytes - 1, None, 0, out.data_ptr(),
+                                  None, L.stream()) == -6
