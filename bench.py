@@ -571,6 +571,9 @@ def main():
         "module_forward_ms_per_step": None if module_ms is None else round(module_ms, 4),
         "graph_replay_ms_per_step": None if graph_ms is None else round(graph_ms, 4),
         "cold_ms_per_forward": None if cold_ms is None else round(cold_ms, 4),
+        # weight storage of this layer on the GPU: the reference's buffers and the tile-ordered copy the prefill GEMM
+        # reads (MixedQLinear.release_row_major_weights() / release_tiled_weights() keep one of them)
+        "resident_weight_bytes": mod.weight_bytes(),
         "verified_vs_oracle": None if spot is None else {"tiles": 3, "max_abs_err_over_rms": round(spot, 6),
                                                          "tolerance": 1e-2},
         "roofline": {"kernel": gemm_kernel,

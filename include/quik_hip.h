@@ -157,7 +157,7 @@ int quik_colmap_streaming(const void *colmap, int64_t cols, int64_t num_int, int
 int quik_asym_quantize_fp6(const void *x, int dtype, int64_t rows, int64_t cols, const void *colmap,
                            int64_t num_int, int64_t num_fp, void *out6, void *meta, void *stream);
 
-/* as quik_mixed_linear_fwd (asymmetric form, bits = 4) on operand buffers */
+/* as quik_mixed_linear_fwd (asymmetric form, bits = 4) on operand buffers; any row count (M >= 1) */
 int quik_mixed_linear_fwd_fp6(const void *x6, const void *w6, const void *meta, const void *s_col,
                               const void *w_reduced, const void *bias, int dtype, int64_t M, int64_t N,
                               int64_t K, int64_t F, void *out, void *stream);
@@ -242,7 +242,10 @@ int quik_mixed_linear_fwd_tile8_ws(const void *x8, const void *w8, const void *m
  *   int_weight [out, num_int/2] u8 or [out, num_int] i8; weights_scales [out]; reduced_w [out] (NULL when
  *   symmetric); fp_weight [out, num_fp] (NULL when num_fp == 0); bias [out] or NULL
  *   tiled_weight    quik_fp6_pack_weight (bits 4) / quik_tile8_pack_weight (bits 8) buffer, or NULL
- *   tiled_min_rows  33 is what MixedQLinear uses
+ *   tiled_min_rows  33 is what MixedQLinear uses.  With 1 every call takes the tile-ordered path and reads
+ *                   only tiled_weight: int_weight and fp_weight may then be NULL, i.e. the layer can live
+ *                   with ONE copy of its weights (0.75 byte per int4 weight, 1 per int8 weight) at the price
+ *                   of slower calls of at most 32 rows (the weight-streaming kernel reads the packed nibbles)
  * workspace: quik_layer_workspace_bytes(layer, rows) bytes, 256-byte aligned, holds the quantized activation
  * between the two launches; splitk_workspace as for the _ws entry points (may be NULL).
  * mid_event: NULL, or a hipEvent_t that is recorded on the stream between the quantize launch and the

@@ -316,7 +316,7 @@ int run_chain(const I32Args &a, const ChainArgs &e, hipStream_t st) {
 
 // Tile plan of the 6-bit path (gemm_fp6.h).  Costs in percent of a 256x256 tile, measured at K = 7936, F = 256:
 // a 256x128 tile 59; 128x128 tiles run two to a CU, 66 for a pair, 36 for one that has the CU to itself.
-Plan make_plan6(int64_t M, int64_t N, int64_t min_rows = 33) {
+Plan make_plan6(int64_t M, int64_t N, int64_t min_rows) {
   if (M < min_rows) return {Plan::kSmall, 0};
   const int64_t tiles_m = (M + 255) / 256;
   const int64_t mid_tiles = ((M + 127) / 128) * ((N + 127) / 128);
@@ -359,6 +359,15 @@ SplitPlan plan_splitk(int64_t M, int64_t N, int64_t steps, int64_t min_steps, in
   return none;
 }
 
+// The arrival counters are zero between launches because every launch that completes returns them there.  After a
+// launch that was refused nothing ran, but the caller may not know how far an earlier one got: clear the counters
+// behind a failed launch so that the next one on this workspace starts clean.
+int splitk_launch_status(void *workspace, hipStream_t st) {
+  const int rc = check_launch();
+  if (rc != QUIK_OK) (void)hipMemsetAsync(workspace, 0, kSplitCounterBytes, st);
+  return rc;
+}
+
 template <bool BF16>
 int launch_fused6_splitk(const Fused6Args &p, const SplitPlan &sp, void *workspace, hipStream_t st) {
   int tiles_m, tiles_n;
@@ -369,7 +378,7 @@ int launch_fused6_splitk(const Fused6Args &p, const SplitPlan &sp, void *workspa
   constexpr int smem = fused6_smem<CfgM>();
   if (int rc = prepare(kern, smem)) return rc;
   hipLaunchKernelGGL(kern, dim3(grid_tiles * sp.splits), dim3(CfgM::kThreads), smem, st, p, tiles_m, tiles_n, sk);
-  return check_launch();
+  return splitk_launch_status(workspace, st);
 }
 
 template <bool BF16>
@@ -382,7 +391,7 @@ int launch_fused8t_splitk(const Fused8Args &p, const SplitPlan &sp, void *worksp
   constexpr int smem = fused8t_smem<CfgM>();
   if (int rc = prepare(kern, smem)) return rc;
   hipLaunchKernelGGL(kern, dim3(grid_tiles * sp.splits), dim3(CfgM::kThreads), smem, st, p, tiles_m, tiles_n, sk);
-  return check_launch();
+  return splitk_launch_status(workspace, st);
 }
 
 template <class C, bool BF16>
@@ -415,11 +424,12 @@ int launch_fused6_split(const Fused6Args &wide, const Fused6Args &tail, hipStrea
 // launch (four waves), or 128x128 tiles.
 template <bool BF16>
 int run_fused6(const Fused6Args &p, hipStream_t st, void *workspace, int64_t workspace_bytes) {
-  const Plan plan = make_plan6(p.M, p.N);
-  if (plan.kind == Plan::kSmall) return QUIK_ERR_SHAPE;  // at most 32 rows: the weight-streaming kernel is the right one
+  // any row count: up to 32 rows the weight-streaming kernel on the packed nibbles reads a third fewer bytes, and
+  // callers that keep both weight copies route such calls there
+  const Plan plan = make_plan6(p.M, p.N, 1);
   if (plan.kind == Plan::kSplit && plan.n_wide >= p.N) return launch_fused6<CfgL8, BF16>(p, st);
   if (plan.kind != Plan::kSplit) {
-    const SplitPlan sp = plan_splitk(p.M, p.N, p.K / 64, kSplitMinSteps6, 33, 3);
+    const SplitPlan sp = plan_splitk(p.M, p.N, p.K / 64, kSplitMinSteps6, 1, 3);
     if (sp.splits > 1 && workspace && workspace_bytes >= sp.bytes) return launch_fused6_splitk<BF16>(p, sp, workspace, st);
     return launch_fused6<CfgM, BF16>(p, st);
   }
@@ -583,7 +593,7 @@ extern "C" int quik_mixed_linear_fwd(const void *qx, const void *qw, const void 
 extern "C" int64_t quik_splitk_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits) {
   if (M <= 0 || N <= 0 || K <= 0 || (bits != 4 && bits != 8)) return 0;
   if (bits == 4 ? K % 128 != 0 : K % 64 != 0) return 0;
-  return (bits == 4 ? plan_splitk(M, N, K / 64, kSplitMinSteps6, 33, 3) : plan_splitk(M, N, K / 32, kSplitMinSteps8, 1, 2)).bytes;
+  return (bits == 4 ? plan_splitk(M, N, K / 64, kSplitMinSteps6, 1, 3) : plan_splitk(M, N, K / 32, kSplitMinSteps8, 1, 2)).bytes;
 }
 
 extern "C" int quik_mixed_linear_fwd_fp6(const void *x6, const void *w6, const void *meta, const void *s_col,
@@ -599,7 +609,6 @@ extern "C" int quik_mixed_linear_fwd_fp6_ws(const void *x6, const void *w6, cons
   if (dtype != QUIK_F16 && dtype != QUIK_BF16) return QUIK_ERR_DTYPE;
   if (M < 0 || N < 0 || K <= 0 || F < 0) return QUIK_ERR_SHAPE;
   if (M == 0 || N == 0) return QUIK_OK;
-  if (M <= 32) return QUIK_ERR_SHAPE;
   if (!x6 || !w6 || !meta || !s_col || !out) return QUIK_ERR_NULL;  // w_reduced == NULL: symmetric activations
   if (K % 128 != 0 || F % 32 != 0) return QUIK_ERR_ALIGN;
   auto misaligned = [](const void *p) { return reinterpret_cast<uintptr_t>(p) % 256 != 0; };

@@ -66,12 +66,14 @@ extern "C" int quik_layer_forward(const quik_layer *layer, const void *x, int64_
   if (!layer_valid(layer)) return QUIK_ERR_SHAPE;
   if (rows < 0) return QUIK_ERR_SHAPE;
   if (rows == 0) return QUIK_OK;
-  if (!x || !workspace || !out || !layer->colmap || !layer->int_weight || !layer->weights_scales) return QUIK_ERR_NULL;
+  if (!x || !workspace || !out || !layer->colmap || !layer->weights_scales) return QUIK_ERR_NULL;
   if (!layer->symmetric && !layer->reduced_w) return QUIK_ERR_NULL;
-  if (layer->num_fp > 0 && !layer->fp_weight) return QUIK_ERR_NULL;
   if (reinterpret_cast<uintptr_t>(x) % 16 != 0 || reinterpret_cast<uintptr_t>(workspace) % 256 != 0) return QUIK_ERR_ALIGN;
   const quik_layer &l = *layer;
   const LayerPlan p = plan_layer(layer, rows);
+  // the row-major weights are read only by calls that do not take the tile-ordered path: a layer whose every call
+  // does (tiled_min_rows <= 1) may leave them NULL
+  if (!p.tiled && (!l.int_weight || (l.num_fp > 0 && !l.fp_weight))) return QUIK_ERR_NULL;
   if (workspace_bytes < p.bytes) return QUIK_ERR_RANGE;
   uint8_t *ws = static_cast<uint8_t *>(workspace);
   void *q = ws + p.off_q, *meta = ws + p.off_meta, *fp_x = l.num_fp > 0 ? ws + p.off_fp : nullptr;

@@ -8,6 +8,8 @@ as a separate op; it computes what experiments/qlinear.py:122-145 computes in th
 """
 from __future__ import annotations
 
+import threading
+
 import torch
 
 from . import _lib as L
@@ -86,13 +88,19 @@ def mixed_linear(qx, int_weight, meta, weights_scales, reduced_w, fp_x, fp_weigh
     return out
 
 
-# K split of the tile-ordered GEMMs (few token rows, few output columns, long K): one zeroed workspace per GPU,
-# shared by all layers (arrival counters, which every launch leaves at zero, and partial sums).  Launches that may
-# overlap on one GPU (several streams) must not share it: set split_k = False there.
+# K split of the tile-ordered GEMMs (few token rows, few output columns, long K) needs a zeroed workspace (arrival
+# counters, which every launch leaves at zero, and partial sums).  Launches that overlap on one GPU must not share
+# one, so there is one per (GPU, stream), made by the first eager call on that stream that can use it, shared by all
+# layers, and one more per GPU for calls recorded into HIP graphs (made together with the GPU's first eager one: a
+# capture cannot allocate).  Graphs that are replayed on different streams at the same time would share that one:
+# set split_k = False while capturing such graphs.  Beyond _MAX_STREAMS streams per GPU further streams run without
+# the K split (same output bits, the unsplit kernel).
 split_k = True
 _SPLITK_BYTES = 4096 + 256 * 128 * 128 * 4   # the largest request: 256 workgroups of one 128x128 tile each
+_MAX_STREAMS = 8
 _splitk_workspaces = {}
 _splitk_needed = {}
+_splitk_lock = threading.Lock()
 
 
 def _splitk_workspace(device, M, N, K, bits):
@@ -104,11 +112,21 @@ def _splitk_workspace(device, M, N, K, bits):
         need = _splitk_needed[key] = L.load().quik_splitk_workspace_bytes(M, N, K, bits)
     if need == 0:
         return None, 0
-    ws = _splitk_workspaces.get(device.index)
+    capturing = torch.cuda.is_current_stream_capturing()
+    slot = (device.index, "graphs" if capturing else torch.cuda.current_stream(device).cuda_stream)
+    ws = _splitk_workspaces.get(slot)
     if ws is None:
-        if torch.cuda.is_current_stream_capturing():   # no allocation that a graph's pool would own
+        if capturing:                                   # no allocation that a graph's pool would own
             return None, 0
-        ws = _splitk_workspaces[device.index] = torch.zeros(_SPLITK_BYTES, dtype=torch.uint8, device=device)
+        with _splitk_lock:
+            ws = _splitk_workspaces.get(slot)
+            if ws is None:
+                if sum(1 for d, _ in _splitk_workspaces if d == device.index) > _MAX_STREAMS:
+                    return None, 0
+                if (device.index, "graphs") not in _splitk_workspaces:
+                    _splitk_workspaces[(device.index, "graphs")] = torch.zeros(_SPLITK_BYTES, dtype=torch.uint8,
+                                                                               device=device)
+                ws = _splitk_workspaces[slot] = torch.zeros(_SPLITK_BYTES, dtype=torch.uint8, device=device)
     return ws, ws.numel()
 
 

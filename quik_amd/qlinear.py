@@ -99,6 +99,7 @@ class MixedQLinear(torch.nn.Module):
         self.six_bit_path = True
         self._w6 = None
         self._w6_key = None
+        self._row_major_released = False
         self._streams = None
         self.fp_features_num = fp_features_num
         self.int_features_num = in_features - fp_features_num
@@ -153,6 +154,8 @@ class MixedQLinear(torch.nn.Module):
         return self._streams_flag()
 
     def _weight6(self):
+        if self._row_major_released:
+            return self._w6
         fp_w = self.fp_weight if self.fp_features_num > 0 else \
             torch.empty((self.out_features, 0), dtype=self.dtype, device=self.int_weight.device)
         key = (self.int_weight.data_ptr(), self.int_weight._version, fp_w.data_ptr(), fp_w._version,
@@ -164,6 +167,45 @@ class MixedQLinear(torch.nn.Module):
                 self._w6 = matmul.pack_weight_tile8(self.int_weight, fp_w)
             self._w6_key = key
         return self._w6
+
+    # -- which copies of the weights stay resident
+    def weight_bytes(self):
+        """Bytes of weight storage this module holds on its device: the reference's buffers (int_weight + fp_weight,
+        qlinear.py:53-78 of the reference) and the tile-ordered copy the prefill GEMMs read (made by the first call
+        that takes that path; 0.75 byte per int4 weight, 1 per int8 weight, outlier columns included)."""
+        fp = self.fp_weight if self.fp_features_num > 0 else None
+        row_major = self.int_weight.numel() * self.int_weight.element_size() + \
+            (fp.numel() * fp.element_size() if fp is not None else 0)
+        tiled = self._w6.numel() * self._w6.element_size() if self._w6 is not None else 0
+        packed = self.out_features * (self.int_features_num * self.bits // 8 +
+                                      self.fp_features_num * self.weights_scales.element_size())
+        return {"row_major": row_major, "tiled": tiled, "reference_layout": packed}
+
+    def release_tiled_weights(self):
+        """Drop the tile-ordered copy and stop using the tile-ordered paths: every call reads the reference's
+        buffers (int8-MFMA GEMM above 32 rows: same output bits, about half the 6-bit path's rate for W4A4)."""
+        if self._row_major_released:
+            raise RuntimeError("the tile-ordered copy is the only one this module holds")
+        self.six_bit_path = False
+        self._w6 = self._w6_key = None
+        self._descs.clear()
+
+    def release_row_major_weights(self):
+        """Keep only the tile-ordered copy: int_weight and fp_weight become empty tensors and EVERY call, down to
+        one row, takes the tile-ordered path (same output bits above 32 rows; up to 32 rows equal within rounding
+        of the fp32 sums, and slower than the weight-streaming kernel, which reads the packed nibbles).  The
+        module can no longer be saved in the reference's checkpoint format or moved to another device."""
+        if not self._six_bit_ok(max(self.six_bit_min_rows, self.tile8_min_rows)):
+            raise RuntimeError("this layer does not take the tile-ordered path (shape, dtype or column map)")
+        w6 = self._weight6()
+        self._row_major_released = True
+        self.six_bit_min_rows = self.tile8_min_rows = 1
+        dev = self.int_weight.device
+        self.int_weight = torch.empty((0,), dtype=self.int_weight.dtype, device=dev)
+        if self.fp_features_num > 0:
+            self.fp_weight = torch.empty((0,), dtype=self.dtype, device=dev)
+        self._descs.clear()
+        assert self._weight6() is w6
 
     def _streams_flag(self):
         """True if the column map selects the streaming quantize kernel (cached; one synchronisation per map)."""
@@ -199,9 +241,10 @@ class MixedQLinear(torch.nn.Module):
             d.sym_divisor = float(self.sym_divisor)
             d.colmap_streams = int(self._streams_flag())
             d.tiled_min_rows = self.six_bit_min_rows if self.bits == 4 else self.tile8_min_rows
-            d.colmap, d.int_weight, d.weights_scales = colmap.data_ptr(), bufs[0].data_ptr(), bufs[1].data_ptr()
+            d.colmap, d.weights_scales = colmap.data_ptr(), bufs[1].data_ptr()
+            d.int_weight = bufs[0].data_ptr() if bufs[0].numel() > 0 else None
             d.reduced_w = bufs[4].data_ptr() if bufs[4] is not None else None
-            d.fp_weight = bufs[5].data_ptr() if bufs[5] is not None else None
+            d.fp_weight = bufs[5].data_ptr() if bufs[5] is not None and bufs[5].numel() > 0 else None
             d.bias = bufs[6].data_ptr() if bufs[6] is not None and bufs[6].numel() > 0 else None
             d.tiled_weight = w6.data_ptr() if w6 is not None else None
             entry = self._descs[tiled] = (key, d, {}, (colmap, w6))   # the tensors the pointers refer to stay alive
@@ -289,6 +332,9 @@ class MixedQLinear(torch.nn.Module):
                                  self.dtype)
                 shared_input.finish()
                 return output.reshape(*lead, self.out_features)
+            if self._row_major_released:
+                raise RuntimeError("this call needs the row-major weights, which release_row_major_weights() dropped "
+                                   "(input dtype / alignment, or fused / six_bit_path switched off)")
             if shared_input.qint_x is None:
                 self._quantize_input(x2, shared_input)
             if self.fused:

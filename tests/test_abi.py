@@ -88,7 +88,7 @@ def test_tile_ordered_entry_points_validate_without_gpu():
     assert lib.quik_sym_quantize_mapped(one, 64, 8190, one, 7934, 256, 4, f(4.0), 0, one, one, one, null) == -2
     assert lib.quik_sym_quantize_mapped(one, 64, 8192, one, 7936, 256, 4, f(4.0), 0, one, one, null, null) == -5
     assert lib.quik_sym_quantize_mapped(one, 64, 8192, one, 7936, 256, 4, f(4.0), 1, odd, one, null, null) == -4
-    assert lib.quik_mixed_linear_fwd_fp6(one, one, one, one, one, null, 0, 32, 256, 7936, 256, one, null) == -2  # decode size
+    assert lib.quik_mixed_linear_fwd_fp6(one, one, one, one, one, null, 0, -1, 256, 7936, 256, one, null) == -2
     assert lib.quik_mixed_linear_fwd_fp6(one, odd, one, one, one, null, 0, 64, 256, 7936, 256, one, null) == -4
     assert lib.quik_mixed_linear_fwd_fp6(one, one, one, one, one, null, 0, 64, 256, 74496 + 128, 256, one, null) == -6
     assert lib.quik_mixed_linear_fwd_tile8(one, one, null, one, one, null, 0, 64, 256, 28416, 256, one, null) == -5
@@ -241,6 +241,8 @@ def test_layer_forward_validates_without_gpu():
     assert fwd(d, out=null) == -5
     assert fwd(layer(reduced_w=None)) == -5                  # asymmetric needs the reduced weights
     assert fwd(layer(fp_weight=None)) == -5
+    assert fwd(layer(int_weight=None)) == -5                 # ... only a layer whose every call is tile-ordered may
+    assert fwd(layer(int_weight=None, tiled_weight=256), rows=20) == -5
     assert fwd(d, x=ctypes.c_void_p(264)) == -4
     assert fwd(d, ws=odd) == -4
     assert fwd(d, nb=1024) == -6                             # workspace too small

@@ -178,3 +178,48 @@ def test_layer_forward_through_the_c_abi(M, bits):
     # a workspace one byte short is refused before anything is launched
     assert lib.quik_layer_forward(ctypes.byref(d), x.data_ptr(), M, ws.data_ptr(), nbytes - 1, None, 0, out.data_ptr(),
                                   None, L.stream()) == -6
+
+
+@pytest.mark.parametrize("bits,symm,n_in,F", [(4, False, 2048 + 64, 64), (8, False, 1280 + 256, 256),
+                                              (4, True, 1024 + 32, 32)])
+def test_one_resident_copy_of_the_weights(bits, symm, n_in, F):
+    """release_row_major_weights(): the module keeps the tile-ordered copy only and serves every row count from
+    it; release_tiled_weights(): the reference's buffers only.  Above 32 rows all three give the same bits; up to
+    32 rows the tile-ordered kernels add the fp32 terms in another order than the weight-streaming kernel:
+    equal within rounding, and within 1e-2 x RMS of the oracle."""
+    N = 384
+    rng = np.random.default_rng(bits + F)
+    W, s_w, fi = _layer(rng, N, n_in, F, bits)
+    bias = rng.standard_normal(N).astype(np.float16)
+    omod = qo.from_float(W, s_w, fi, bits, symm=symm)
+    both = _module(W, s_w, fi, bits, bias, symm)
+    tiled_only = _module(W, s_w, fi, bits, bias, symm)
+    rows_only = _module(W, s_w, fi, bits, bias, symm)
+    rows_only.release_tiled_weights()
+    xs = {}
+    for M in (1, 20, 32, 33, 200):
+        x = rng.standard_normal((M, n_in)).astype(np.float32)
+        x[:, fi] *= 50
+        xs[M] = x.astype(np.float16)
+    ref = {M: both(torch.from_numpy(x).to(DEV)) for M, x in xs.items()}
+    wb = both.weight_bytes()
+    assert wb["row_major"] == wb["reference_layout"] == N * ((n_in - F) * bits // 8 + F * 2)
+    assert wb["tiled"] >= N * ((n_in - F) * (6 if bits == 4 else 8) // 8 + F * 2)
+    tiled_only.release_row_major_weights()
+    wt = tiled_only.weight_bytes()
+    assert wt["row_major"] == 0 and wt["tiled"] == wb["tiled"]
+    assert rows_only.weight_bytes()["tiled"] == 0
+    for M, x in xs.items():
+        xt = torch.from_numpy(x).to(DEV)
+        got_t, got_r = tiled_only(xt), rows_only(xt)
+        assert rows_only._w6 is None
+        assert torch.equal(_bits(got_r), _bits(ref[M]))
+        want, _ = qo.mixed_qlinear_forward(x, omod, bits, bias, symm=symm)
+        w64 = want.astype(np.float64)
+        if M > 32:
+            assert torch.equal(_bits(got_t), _bits(ref[M]))
+        err = np.abs(got_t[0].float().cpu().numpy().astype(np.float64) - w64).max()
+        assert err <= 1e-2 * np.sqrt((w64 ** 2).mean())
+        assert err <= 4 * np.abs(w64).max() * 2.0 ** -10
+    with pytest.raises(RuntimeError):
+        tiled_only.release_tiled_weights()

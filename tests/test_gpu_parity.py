@@ -1252,8 +1252,16 @@ def test_split_k_gives_the_same_bits(case):
     nan_rows = np.isnan(x[:, ii].astype(np.float32)).any(1) if symm else np.zeros(M, bool)
     for g in got:
         assert np.array_equal(g[0][~nan_rows], want[0][~nan_rows])
-    ws = matmul._splitk_workspaces[torch.cuda.current_device()]
+    ws = matmul._splitk_workspaces[(torch.cuda.current_device(), torch.cuda.current_stream().cuda_stream)]
     assert int(ws[:4096].view(torch.int32).abs().sum()) == 0               # counters are back at zero
+    # a second stream gets a workspace of its own (launches on two streams may overlap), same bits
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        other = _bits(mod(xt))
+        assert matmul._splitk_workspaces[(torch.cuda.current_device(), side.cuda_stream)] is not ws
+    side.synchronize()
+    assert np.array_equal(other[0][~nan_rows], want[0][~nan_rows])
 
 
 @pytest.mark.parametrize("M,tiled", [(16, False), (24, True), (32, False), (32, True), (33, True)])
