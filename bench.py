@@ -342,6 +342,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="llama2-70b.gate_proj", choices=sorted(WORKLOADS) + sorted(BLOCK_WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--event-every", type=int, default=1,
+                    help="record the HIP events that time the two kernels on every N-th timed step (default: every step)")
     ap.add_argument("--no-verify", action="store_true", help="skip the spot check of the output against the CPU oracle")
     ap.add_argument("--unfused", action="store_true", help="run the reference's three-op sequence instead")
     ap.add_argument("--int8-mfma", action="store_true",
@@ -403,19 +405,19 @@ def main():
 
     def step(ev=None):
         """One forward of the layer.  Fused (the default): ONE call of the module, mod(x) -> quik_layer_forward, which
-        launches the quantize kernel and the fused GEMM; ev = (event recorded by the library between the two
-        launches, event recorded after the call), both on the launch stream.  --unfused: the reference's op sequence
-        through the stand-alone ops, ev = (before, between, after)."""
+        launches the quantize kernel and the fused GEMM.  --unfused: the reference's op sequence through the stand-alone
+        ops.  ev = (before, between, after): events on the launch stream; in the fused form the library records the
+        middle one between its two launches."""
+        if ev is not None:
+            ev[0].record()
         if mod.fused:
             if ev is not None:
-                mod.mid_event = ev[0]
+                mod.mid_event = ev[1]
             out = mod(x)[0]
             if ev is not None:
                 assert mod.mid_event is None, "the forward did not go through the one-call path"
-                ev[1].record()
+                ev[2].record()
             return out
-        if ev is not None:
-            ev[0].record()
         q, meta, fp = asymmetric.quantize_mapped(x, colmap, K, F, bits)
         if ev is not None:
             ev[1].record()
@@ -433,26 +435,23 @@ def main():
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
-    n_ev = 2 if mod.fused else 3
-    events = [[torch.cuda.Event(enable_timing=True) for _ in range(n_ev)] for _ in range(args.steps)]
-    for evs in events:                 # an event has a handle only once it has been recorded
+    # Kernel durations from HIP events inside the timed region (three per step: before, between the two launches,
+    # after; an event record between two launches costs 3 - 4 us on the GPU's timeline, which ms_per_step includes;
+    # --event-every N records them on every N-th step only).
+    every = max(1, args.event_every)
+    events = {i: [torch.cuda.Event(enable_timing=True) for _ in range(3)] for i in range(0, args.steps, every)}
+    for evs in events.values():        # an event has a handle only once it has been recorded
         for e in evs:
             e.record()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(args.steps):
-        step(events[i])
+        step(events.get(i))
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     ms_step = (t1 - t0) * 1e3 / args.steps
-    if mod.fused:
-        # GEMM launch: between-event -> after-event of the same step; quantize launch: after-event of the previous
-        # step -> between-event (this interval also holds the gap between two forwards)
-        g_ms = sorted(e[0].elapsed_time(e[1]) for e in events)
-        q_ms = sorted(events[i - 1][1].elapsed_time(events[i][0]) for i in range(1, args.steps)) or [0.0]
-    else:
-        q_ms = sorted(e[0].elapsed_time(e[1]) for e in events)
-        g_ms = sorted(e[1].elapsed_time(e[2]) for e in events)
+    q_ms = sorted(e[0].elapsed_time(e[1]) for e in events.values())
+    g_ms = sorted(e[1].elapsed_time(e[2]) for e in events.values())
     q_avg, g_avg = sum(q_ms) / len(q_ms), sum(g_ms) / len(g_ms)
 
     # the quantize kernel alone, launched back to back (outside the timed region)
@@ -582,7 +581,7 @@ def main():
                      "frac_of_int8_peak": round(gemm_tops / PEAK_INT8_TOPS, 4),
                      "traffic": traffic.get("gemm6" if six else "gemm") if mod.fused else None,
                      "avg_ms": round(g_avg, 4), "median_ms": round(g_ms[len(g_ms) // 2], 4),
-                     "algorithmic_ops": int_ops},
+                     "timed_launches": len(g_ms), "algorithmic_ops": int_ops},
         "roofline_quantize": {"kernel": ("quantize_fp6_wave_kernel (one wave per token row, 6-bit operand output)" if six and bits == 4
                                          else "asym_quantize_stream_kernel" + (" (tile-ordered operand output)" if six else "")),
                               "bound": "hbm",
@@ -591,9 +590,9 @@ def main():
                               "traffic": traffic.get("quantize6" if six else "quantize"), "avg_ms": round(q_avg, 5),
                               "median_ms": round(q_ms[len(q_ms) // 2], 5), "algorithmic_bytes": quant_bytes,
                               "back_to_back_ms": round(q_b2b, 5),
-                              "note": "avg_ms: from the event after the previous forward to the event the library "
-                                      "records between the quantize launch and the GEMM launch (the launch plus the "
-                                      "gap between two forwards); back_to_back_ms: per launch over 50 consecutive "
+                              "note": "avg_ms: from an event in front of the forward to the event the library records "
+                                      "between the quantize launch and the GEMM launch (the launch plus the cost of "
+                                      "one event record, several us); back_to_back_ms: per launch over 50 consecutive "
                                       "launches after the timed region (bound by the host: ~14 us of Python per "
                                       "call); kernel-trace durations: profiles/"},
     }
