@@ -115,7 +115,8 @@ __device__ __forceinline__ float wave_min(float v) {
 // as inline assembly so that the outstanding-load count stays under this file's control: the
 // loop waits with vmcnt(loads per stage), leaving the newest stage in flight across the barrier.
 // (s_nop 0: one wait state between the scalar write of m0 and the copy that reads it, which the compiler
-// keeps for its own LDS copies on this generation and cannot see inside an asm statement.)
+// keeps for its own LDS copies on this generation and cannot see inside an asm statement.  m0 is declared
+// clobbered; the "memory" clobber orders the statement against the compiler's own LDS and global accesses.)
 __device__ __forceinline__ void dma_load16(const uint8_t *sbase, uint32_t voff, uint32_t lds_addr) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(sbase) : "memory", "m0");
 }

@@ -34,6 +34,9 @@ typedef int v8i __attribute__((ext_vector_type(8)));
 
 // One wave-wide copy global -> LDS (see dma_load16) whose instruction offset moves both addresses: the three
 // kilobytes of a block unit are copied with one source pointer and one LDS base.
+// (Hazards: one wait state between the scalar write of m0 and the copy that reads it, the s_nop 0; m0 is in the
+// clobber list, so the compiler does not keep a value of its own in it across the statement; the "memory" clobber
+// keeps LDS accesses of the compiler on their side of the copy, and completion is awaited through vmcnt.)
 template <int OFFSET>
 __device__ __forceinline__ void dma_load16k(const uint8_t *sbase, uint32_t voff, uint32_t lds_addr) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 offset:%3"
@@ -125,7 +128,7 @@ struct Fp6Pipe {
       const int jj = j < MI ? j : j - MI;
       tail[j] = (j < MI ? (wm * C::WM / 64) * 3072 : W_OFF + (wn * C::WN / 64) * 3072) + (jj >> 1) * 3072 + 2048 +
                 h * 512 + ((jj & 1) * 32 + r) * 8;
-      asm volatile("" : "+v"(tail[j]));  // unrelated values as far as the compiler can tell
+      asm volatile("" : "+v"(tail[j]));  // unrelated values as far as the compiler can tell (empty statement: no hazard)
     }
 #pragma unroll
     for (int q = 0; q < 3; ++q) {
@@ -419,9 +422,12 @@ struct SplitK {
 __device__ __forceinline__ void splitk_store4(int32_t *p, v4i v) {
   asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 2" : : "v"(p), "v"(v) : "memory");
 }
+// (a wait only: no register or wait-state hazard; "memory" keeps the compiler from moving stores across it)
 __device__ __forceinline__ void splitk_stores_done() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 // eight 16-byte loads, STRIDE int32 apart, and the wait for them in one statement: the compiler sees the
-// registers only once they hold the data
+// registers only once they hold the data (hazards: the outputs are early-clobber, so no load's destination
+// overlaps an address register that a later load of the statement still reads; the statement ends with
+// vmcnt(0), so nothing it started is in flight when the compiler's instructions resume)
 template <int STRIDE>
 __device__ __forceinline__ void splitk_load8(const int32_t *p, v4i *r) {
   asm volatile(

@@ -756,6 +756,10 @@ struct FusedArgs {
 // registers (the only ones VALU instructions can touch).  Spelled out so that the conversion
 // between the two MFMA phases streams through a handful of vector registers; left to itself the
 // register allocator copies all 256 accumulators out at once and spills.
+// (Hazards: a read that follows an MFMA writing the same accumulator needs that MFMA's passes to have finished;
+// the callers put 2 x s_nop 15 between the last MFMA and the first read, more than the 18 wait states the
+// longest MFMA used here asks for.  Between VALU instructions and these moves the hardware interlocks, as for any
+// VALU pair; the compiler schedules its own MFMAs after an agpr_write through the register dependence.)
 __device__ __forceinline__ float agpr_read(float a) {
   float v;
   asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(a));

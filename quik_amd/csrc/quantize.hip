@@ -364,6 +364,8 @@ struct __attribute__((packed, aligned(1))) Bytes8 {
 // The code is (level - 2^(BITS-1)) mod 256; for BITS == 4 only its low nibble is meaningful.
 // SYM (fp16 only): symmetric codes, rne(fp16(x / scale)) kept modulo 256 without a clamp (reference:
 // src/symmetric/symmetric.cu:6-61; NaN -> 0, +-infinity saturate as __half2int_rn does before the low bits are cut).
+// (The v_fma_mix pairs below are plain VALU instructions; their output is early-clobber because the second
+// instruction of a pair reads the inputs after the first has written its half: no wait-state hazard.)
 template <int BITS, bool BF16, bool SLOW, bool SYM = false>
 __device__ __forceinline__ uint32_t code_pair(uint32_t w, const RowQuant<BF16> &rq) {
   constexpr float kMaxQ = static_cast<float>((1 << BITS) - 1);
@@ -749,6 +751,8 @@ __global__ __launch_bounds__(TPR) void asym_quantize_stream_kernel(
 
 // Packed fp16 min / max as single instructions.  (The compiler's own minnum / maxnum first quiet a possible
 // signalling NaN with an extra v_pk_max x, x whenever it cannot prove that the operand is not one.)
+// (Plain VALU instructions on the statement's own operands, not volatile: no wait-state hazard, and the compiler
+// is free to schedule or drop them like any other arithmetic.)
 __device__ __forceinline__ uint32_t pk_min_f16(uint32_t a, uint32_t b) {
   uint32_t r;
   asm("v_pk_min_f16 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
@@ -769,6 +773,8 @@ __device__ __forceinline__ uint32_t pk_max_f16(uint32_t a, uint32_t b) {
 //   tests/test_quotient_levels.py enumerates them).
 //   symmetric: t = fp16(f32(x) * rcp) with |t| <= 4.2 (scale = fp16(max|x| / 4), at most 3 % below the quotient
 //   for the smallest scale); t + 1544 holds rne(t) + 8 in its low mantissa bits.
+// (The two v_fma_mix instructions write the low and the high half of one register: the output is early-clobber
+// because the second one still reads the inputs after the first has written; VALU to VALU, no wait states needed.)
 template <bool SYM, class RQ>
 __device__ __forceinline__ uint32_t level_pair_fast(uint32_t w, const RQ &rq) {
   uint32_t d = w, tb;
@@ -1019,7 +1025,7 @@ __global__ __launch_bounds__(64) void quantize_fp6_wave_kernel(
     const int64_t row = row_of(w);
     if (row < rows) process(row, row_img);
     if (w + gridDim.x < items) {
-      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // this row's LDS reads are done before the image is overwritten
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // this row's LDS reads are done before the image is overwritten (a wait only: no hazard)
       issue(clamped(row_of(w + gridDim.x)));
     }
   }
