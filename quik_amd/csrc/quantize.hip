@@ -846,14 +846,22 @@ __global__ __launch_bounds__(64) void quantize_fp6_wave_kernel(
     const uint32_t a_hi = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(a >> 32)));
     const uint32_t a_lo = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(a & 0xFFFFFFFFu)));
     const uint8_t *rp = reinterpret_cast<const uint8_t *>((static_cast<uint64_t>(a_hi) << 32) | a_lo);
-    // kilobyte q = 4 j + t of the row: this lane copies group 64 q + 4 (lane % 16) + lane / 16 to slot 64 q + lane
+    // kilobyte q of the row: this lane copies group 64 q + 4 (lane % 16) + lane / 16 to slot 64 q + lane.
+    // The kilobytes are requested in an order that starts at a row-dependent one and wraps around: all waves of
+    // the launch issue their copies at about the same time, and with every row starting at its kilobyte 0 (rows
+    // are a multiple of 1 KB apart) the requests in flight at any moment would share their low address bits and
+    // crowd onto a few memory channels (measured with the input in HBM: 15.8 -> 14.0 us for 2048 x 8192).
     const int g_in = 4 * (lane & 15) + (lane >> 4), g_last = (cols >> 3) - 1;
+    const int nkb = 4 * J;
+    const int rot = __builtin_amdgcn_readfirstlane(static_cast<int>((row * 5) % nkb));
     for_j([&](int j) {
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
-        const int g = 64 * (4 * j + t) + g_in;
+        int q = 4 * j + t + rot;
+        q = q >= nkb ? q - nkb : q;
+        const int g = 64 * q + g_in;
         const uint32_t voff = static_cast<uint32_t>(g < g_last ? g : g_last) * 16u;  // past the row: any valid group
-        dma_load16(rp, voff, lds0 + (4 * j + t) * 1024);
+        dma_load16(rp, voff, lds0 + q * 1024);
       }
     });
   };
