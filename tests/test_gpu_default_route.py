@@ -33,7 +33,7 @@ def _bits(t):
     return t.detach().contiguous().view(torch.int16)
 
 
-def make_full_size_layer(M, n_in, N, F, bits, symm, kind, seed):
+def make_full_size_layer(M, n_in, N, F, bits, symm, kind, seed, dtype=torch.float16):
     """Inputs of the measurement protocol, made on the device: x ~ N(0, 1) (or Student-t, 3 degrees of freedom) with
     the outlier columns scaled up, W = codes x per-row scale on the integer columns, N(0, 0.02) on the outlier
     columns.  Returns the module (through from_float), x and the float weight matrix / scales / outlier indices."""
@@ -47,20 +47,20 @@ def make_full_size_layer(M, n_in, N, F, bits, symm, kind, seed):
         x = x / torch.sqrt(chi2 / 3)
     fi = torch.randperm(n_in, generator=g, device=DEV)[:F]
     x[:, fi] *= 20 if kind == "student" else 50
-    x = x.clamp(-6e4, 6e4).half()
+    x = x.clamp(-6e4, 6e4).to(dtype)
     keep = torch.ones(n_in, dtype=torch.bool, device=DEV)
     keep[fi] = False
     ii = torch.arange(n_in, device=DEV)[keep]
     K = n_in - F
     lo, hi = (-8, 8) if bits == 4 else (-127, 128)
-    s_w = (torch.rand(N, 1, generator=g, device=DEV) * 0.009 + 0.001).half()
-    W = torch.empty(N, n_in, dtype=torch.float16, device=DEV)
+    s_w = (torch.rand(N, 1, generator=g, device=DEV) * 0.009 + 0.001).to(dtype)
+    W = torch.empty(N, n_in, dtype=dtype, device=DEV)
     for s in range(0, N, 4096):
         e = min(N, s + 4096)
         codes = torch.randint(lo, hi, (e - s, K), generator=g, device=DEV).float()
-        W[s:e, ii] = (codes * s_w[s:e].float()).half()
-        W[s:e, fi] = (0.02 * torch.randn(e - s, F, generator=g, device=DEV)).half()
-    lin = torch.nn.Linear(n_in, N, bias=False, dtype=torch.float16, device="meta")
+        W[s:e, ii] = (codes * s_w[s:e].float()).to(dtype)      # the codes survive the rounding of the product
+        W[s:e, fi] = (0.02 * torch.randn(e - s, F, generator=g, device=DEV)).to(dtype)
+    lin = torch.nn.Linear(n_in, N, bias=False, dtype=dtype, device="meta")
     mod = MixedQLinear.from_float(lin, W, s_w.cpu(), None, fi.cpu(), symm=symm, bits=bits).to(DEV)
     return mod, x, W, s_w, fi
 
@@ -68,12 +68,21 @@ def make_full_size_layer(M, n_in, N, F, bits, symm, kind, seed):
 def check_against_oracle(out, x, W, s_w, fi, bits, symm, tiles):
     """out [M, N] (device) against the oracle's forward on row / column index sets `tiles`."""
     fin = fi.cpu().numpy()
+    bf16 = out.dtype == torch.bfloat16
+    dt = qo.BF16 if bf16 else qo.F16
+    host = (lambda t: t.float().cpu().numpy()) if bf16 else (lambda t: t.cpu().numpy())
     for rows, cols in tiles:
-        omod = qo.from_float(W[cols].cpu().numpy(), s_w[cols].cpu().numpy(), fin, bits, symm=symm)
-        want, _ = qo.mixed_qlinear_forward(x[rows].cpu().numpy(), omod, bits, None, symm=symm)
+        omod = qo.from_float(host(W[cols]), host(s_w[cols]), fin, bits, symm=symm, dtype=dt)
+        want, inter = qo.mixed_qlinear_forward(host(x[rows]), omod, bits, None, symm=symm, dtype=dt)
         got = out[rows][:, cols].float().cpu().numpy().astype(np.float64)
         w64 = want.astype(np.float64)
         assert np.isfinite(w64).all()
+        if bf16:
+            # one bf16 ulp of the output exceeds 1e-2 x RMS for the larger outputs, and the oracle (like the
+            # reference) rounds the outlier product to bf16 before the final sum: one ulp of each
+            y64 = np.abs(np.asarray(inter["fp_result"], np.float64))
+            assert (np.abs(got - w64) <= (np.abs(w64) + y64) * 2.0 ** -7).all(), (rows[0], cols[0])
+            continue
         err = np.abs(got - w64).max()
         assert err <= 1e-2 * np.sqrt((w64 ** 2).mean()), (err, rows[0], cols[0])
         assert err <= 4 * np.abs(w64).max() * 2.0 ** -10, (err, rows[0], cols[0])
@@ -107,17 +116,21 @@ DEFAULT_ROUTE = [
     (128, 13824, 5120, 256, 8, False, "student"),   # Llama-2-13B down_proj, 128 tokens: K split
     (128, 5120, 5120, 256, 4, False, "student"),    # Llama-2-13B q/k/v/o, 128 tokens
     (64, 28672, 8192, 256, 8, False, "x50"),        # Llama-2-70B down_proj, 64 single-token rows: K split
+    (2049, 8192, 28672, 256, 4, False, "x50"),      # Llama-2-70B gate/up, one row more than the tiles hold: ragged last row block
+    (2048, 8192, 28672, 256, 4, False, "x50", torch.bfloat16),     # Llama-2-70B gate/up, bf16 activations and weights
+    (2048, 13824, 5120, 256, 8, False, "student", torch.bfloat16),  # Llama-2-13B down_proj, W8A8, bf16
 ]
 
 
 @pytest.mark.parametrize("case", DEFAULT_ROUTE)
 def test_default_route_at_benchmark_shapes(case):
-    M, n_in, N, F, bits, symm, kind = case
-    mod, x, W, s_w, fi = make_full_size_layer(M, n_in, N, F, bits, symm, kind, seed=sum(case[:5]) + symm)
+    M, n_in, N, F, bits, symm, kind = case[:7]
+    dtype = case[7] if len(case) > 7 else torch.float16
+    mod, x, W, s_w, fi = make_full_size_layer(M, n_in, N, F, bits, symm, kind, seed=sum(case[:5]) + symm, dtype=dtype)
     assert mod._six_bit_ok(M)                      # the shape is one the tile-ordered path takes
     out = mod(x)
     assert mod._w6 is not None                     # ... and it did run
-    assert out.shape == (1, M, N) and out.dtype == torch.float16
+    assert out.shape == (1, M, N) and out.dtype == dtype
     out = out[0]
     assert torch.isfinite(out).all()
     mod.six_bit_path = False
