@@ -585,7 +585,7 @@ __device__ __forceinline__ void fused6_tile(const Fused6Args &p, int tm, int tn,
   pipe.template run_f16<BF16>(acc);
   pipe.drain();
 
-  // out = storage(acc + (zs * w_red + bias)), written through a staging area in the (now idle) ring: all MI row
+  // out = storage(acc + fma(zs, w_red, bias)), written through a staging area in the (now idle) ring: all MI row
   // blocks of the wave are staged, then read back as whole row segments, then stored, so the LDS round trip and
   // the store issue are paid once per tile and not once per row block.  The per-column vectors are read once;
   // the fragment registers are free by now.
@@ -611,10 +611,10 @@ __device__ __forceinline__ void fused6_tile(const Fused6Args &p, int tm, int tn,
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         Store::put_pairs(stage + mi * Store::kBytes, lane, ni, g,
-                         pack2_from_f32<BF16>(acc[mi][ni][4 * g] + (zs * wr[ni][g].x + bs[ni][g].x),
-                                              acc[mi][ni][4 * g + 1] + (zs * wr[ni][g].y + bs[ni][g].y)),
-                         pack2_from_f32<BF16>(acc[mi][ni][4 * g + 2] + (zs * wr[ni][g].z + bs[ni][g].z),
-                                              acc[mi][ni][4 * g + 3] + (zs * wr[ni][g].w + bs[ni][g].w)));
+                         pack2_from_f32<BF16>(acc[mi][ni][4 * g] + __builtin_fmaf(zs, wr[ni][g].x, bs[ni][g].x),
+                                              acc[mi][ni][4 * g + 1] + __builtin_fmaf(zs, wr[ni][g].y, bs[ni][g].y)),
+                         pack2_from_f32<BF16>(acc[mi][ni][4 * g + 2] + __builtin_fmaf(zs, wr[ni][g].z, bs[ni][g].z),
+                                              acc[mi][ni][4 * g + 3] + __builtin_fmaf(zs, wr[ni][g].w, bs[ni][g].w)));
       }
   }
   if (vec && p.M - mw >= C::WM && p.N - nw >= C::WN) {  // interior (wave-uniform): straight-line code

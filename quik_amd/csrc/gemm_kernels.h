@@ -874,7 +874,7 @@ __device__ __forceinline__ void fused_tile(const FusedArgs &p, int tm, int tn, u
                                              int64_t(p.F) * 2, p.N - n0, p.F * 2, smem, accf);
     }
   }
-  // out = storage(accf + (zs * w_red + bias)), written through the staging area
+  // out = storage(accf + fma(zs, w_red, bias)), written through the staging area
   using Store = BlockStore<C, uint16_t>;
   static_assert(Store::kBytes * C::WAVES <= C::SMEM, "staging fits in the (now idle) operand buffers");
   uint8_t *stage = smem + wave * Store::kBytes;
@@ -892,10 +892,10 @@ __device__ __forceinline__ void fused_tile(const FusedArgs &p, int tm, int tn, u
         const float4 wr = *reinterpret_cast<const float4 *>(tv.wred + c);
         const float4 bs = *reinterpret_cast<const float4 *>(tv.bias + c);
         Store::put_pairs(stage, lane, ni, g,
-                         pack2_from_f32<BF16>(accf[mi][ni][4 * g] + (zs * wr.x + bs.x),
-                                              accf[mi][ni][4 * g + 1] + (zs * wr.y + bs.y)),
-                         pack2_from_f32<BF16>(accf[mi][ni][4 * g + 2] + (zs * wr.z + bs.z),
-                                              accf[mi][ni][4 * g + 3] + (zs * wr.w + bs.w)));
+                         pack2_from_f32<BF16>(accf[mi][ni][4 * g] + __builtin_fmaf(zs, wr.x, bs.x),
+                                              accf[mi][ni][4 * g + 1] + __builtin_fmaf(zs, wr.y, bs.y)),
+                         pack2_from_f32<BF16>(accf[mi][ni][4 * g + 2] + __builtin_fmaf(zs, wr.z, bs.z),
+                                              accf[mi][ni][4 * g + 3] + __builtin_fmaf(zs, wr.w, bs.w)));
       }
     if (mb < p.M && nw < p.N) Store::flush(stage, lane, p.out + int64_t(mb) * p.ldo + nw, p.ldo, p.M - mb, p.N - nw, vec);
     __builtin_amdgcn_sched_barrier(0);

@@ -336,7 +336,7 @@ __device__ __forceinline__ void fused8t_tile(const Fused8Args &p, int tm, int tn
   pipe.template run<BF16 ? kBF16 : kF16, false>(pipe.steps0, pipe.steps, f0, f1, acc);
   pipe.drain();
 
-  // out = storage(acc + (zs * w_red + bias)): all row blocks of the wave staged in the (now idle) ring, read back
+  // out = storage(acc + fma(zs, w_red, bias)): all row blocks of the wave staged in the (now idle) ring, read back
   // as whole row segments, stored
   using Store = BlockStore<C, uint16_t>;
   static_assert(Store::kBytes * C::MI * C::WAVES <= tile8_vectors_offset<C>(), "staging ends before the vectors");
@@ -360,10 +360,10 @@ __device__ __forceinline__ void fused8t_tile(const Fused8Args &p, int tm, int tn
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         Store::put_pairs(stage + mi * Store::kBytes, lane, ni, g,
-                         pack2_from_f32<BF16>(acc[mi][ni][4 * g] + (zs * wr[ni][g].x + bs[ni][g].x),
-                                              acc[mi][ni][4 * g + 1] + (zs * wr[ni][g].y + bs[ni][g].y)),
-                         pack2_from_f32<BF16>(acc[mi][ni][4 * g + 2] + (zs * wr[ni][g].z + bs[ni][g].z),
-                                              acc[mi][ni][4 * g + 3] + (zs * wr[ni][g].w + bs[ni][g].w)));
+                         pack2_from_f32<BF16>(acc[mi][ni][4 * g] + __builtin_fmaf(zs, wr[ni][g].x, bs[ni][g].x),
+                                              acc[mi][ni][4 * g + 1] + __builtin_fmaf(zs, wr[ni][g].y, bs[ni][g].y)),
+                         pack2_from_f32<BF16>(acc[mi][ni][4 * g + 2] + __builtin_fmaf(zs, wr[ni][g].z, bs[ni][g].z),
+                                              acc[mi][ni][4 * g + 3] + __builtin_fmaf(zs, wr[ni][g].w, bs[ni][g].w)));
       }
   }
   if (vec && p.M - mw >= C::WM && p.N - nw >= C::WN) {  // interior (wave-uniform): straight-line code
