@@ -835,29 +835,38 @@ __device__ __forceinline__ void fused_tile(const FusedArgs &p, int tm, int tn, u
     } else {
       mainloop_plain<C, MODE>(qx, p.kbytes, p.M - m0, qw, p.kbytes, p.N - n0, p.kbytes, smem, acc);
     }
-    // acc -> f32(acc) * (s_row * s_col), in place.  The int4 accumulators carry a factor 256;
+    // acc -> f32(acc) * (s_row * s_col) + (zs * w_red + bias), in place.  The int4 accumulators carry a factor 256;
     // it is removed by scaling s_row with 2^-8 instead of shifting: both are exact, so
-    // f32(256 a) * ((s_row 2^-8) s_col) rounds to the same float as f32(a) * (s_row s_col).
-    float srow[C::MI];
+    // f32(256 a) * ((s_row 2^-8) s_col) rounds to the same float as f32(a) * (s_row s_col).  The zero-point and
+    // bias term is the addend of the multiply: the epilogue only converts and stores.
+    float srow[C::MI], zsr[C::MI];
 #pragma unroll
-    for (int mi = 0; mi < C::MI; ++mi)
+    for (int mi = 0; mi < C::MI; ++mi) {
       srow[mi] = tv.srow[wm * C::WM + mi * 32 + (lane & 31)] * (MODE == kInt4 ? 0.00390625f : 1.0f);
+      zsr[mi] = tv.zs[wm * C::WM + mi * 32 + (lane & 31)];
+    }
     // one 32x32 block (a 16-register accumulator tuple) at a time
     asm volatile("s_nop 15\n\ts_nop 15");  // the last MFMA results are architecturally visible to the reads below
 #pragma unroll
     for (int ni = 0; ni < C::NI; ++ni) {
-      float scv[16];
+      float scv[16], wrv[16], bsv[16];
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        const float4 sc = *reinterpret_cast<const float4 *>(tv.scol + wn * C::WN + ni * 32 + acc_col(g, lane));
+        const int c = wn * C::WN + ni * 32 + acc_col(g, lane);
+        const float4 sc = *reinterpret_cast<const float4 *>(tv.scol + c);
+        const float4 wr = *reinterpret_cast<const float4 *>(tv.wred + c);
+        const float4 bs = *reinterpret_cast<const float4 *>(tv.bias + c);
         scv[4 * g] = sc.x, scv[4 * g + 1] = sc.y, scv[4 * g + 2] = sc.z, scv[4 * g + 3] = sc.w;
+        wrv[4 * g] = wr.x, wrv[4 * g + 1] = wr.y, wrv[4 * g + 2] = wr.z, wrv[4 * g + 3] = wr.w;
+        bsv[4 * g] = bs.x, bsv[4 * g + 1] = bs.y, bsv[4 * g + 2] = bs.z, bsv[4 * g + 3] = bs.w;
       }
 #pragma unroll
       for (int mi = 0; mi < C::MI; ++mi) {
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
           const float raw = agpr_read(acc[mi][ni][v]);
-          accf[mi][ni][v] = agpr_write(static_cast<float>(__float_as_int(raw)) * (srow[mi] * scv[v]));
+          accf[mi][ni][v] = agpr_write(__builtin_fmaf(static_cast<float>(__float_as_int(raw)), srow[mi] * scv[v],
+                                                      __builtin_fmaf(zsr[mi], wrv[v], bsv[v])));
         }
       }
     }
@@ -874,7 +883,7 @@ __device__ __forceinline__ void fused_tile(const FusedArgs &p, int tm, int tn, u
                                              int64_t(p.F) * 2, p.N - n0, p.F * 2, smem, accf);
     }
   }
-  // out = storage(accf + fma(zs, w_red, bias)), written through the staging area
+  // out = storage(accf), written through the staging area
   using Store = BlockStore<C, uint16_t>;
   static_assert(Store::kBytes * C::WAVES <= C::SMEM, "staging fits in the (now idle) operand buffers");
   uint8_t *stage = smem + wave * Store::kBytes;
@@ -883,20 +892,12 @@ __device__ __forceinline__ void fused_tile(const FusedArgs &p, int tm, int tn, u
 #pragma unroll
   for (int mi = 0; mi < C::MI; ++mi) {
     const int mb = m0 + wm * C::WM + mi * 32;
-    const float zs = tv.zs[wm * C::WM + mi * 32 + (lane & 31)];
 #pragma unroll
     for (int ni = 0; ni < C::NI; ++ni)
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const int c = wn * C::WN + ni * 32 + acc_col(g, lane);
-        const float4 wr = *reinterpret_cast<const float4 *>(tv.wred + c);
-        const float4 bs = *reinterpret_cast<const float4 *>(tv.bias + c);
-        Store::put_pairs(stage, lane, ni, g,
-                         pack2_from_f32<BF16>(accf[mi][ni][4 * g] + __builtin_fmaf(zs, wr.x, bs.x),
-                                              accf[mi][ni][4 * g + 1] + __builtin_fmaf(zs, wr.y, bs.y)),
-                         pack2_from_f32<BF16>(accf[mi][ni][4 * g + 2] + __builtin_fmaf(zs, wr.z, bs.z),
-                                              accf[mi][ni][4 * g + 3] + __builtin_fmaf(zs, wr.w, bs.w)));
-      }
+      for (int g = 0; g < 4; ++g)
+        Store::put_pairs(stage, lane, ni, g, pack2_from_f32<BF16>(accf[mi][ni][4 * g], accf[mi][ni][4 * g + 1]),
+                         pack2_from_f32<BF16>(accf[mi][ni][4 * g + 2], accf[mi][ni][4 * g + 3]));
     if (mb < p.M && nw < p.N) Store::flush(stage, lane, p.out + int64_t(mb) * p.ldo + nw, p.ldo, p.M - mb, p.N - nw, vec);
     __builtin_amdgcn_sched_barrier(0);
   }

@@ -310,25 +310,35 @@ __device__ __forceinline__ void fused8t_tile(const Fused8Args &p, int tm, int tn
     }
   }
 
-  // acc -> f32(acc) * (s_row * s_col), in place, one 32x32 block at a time
-  float srow[C::MI];
+  // acc -> f32(acc) * (s_row * s_col) + (zs * w_red + bias), in place, one 32x32 block at a time (the zero-point and
+  // bias term is the addend of the multiply: the epilogue only converts and stores)
+  float srow[C::MI], zsr[C::MI];
 #pragma unroll
-  for (int mi = 0; mi < C::MI; ++mi) srow[mi] = tv.srow[wm * C::WM + mi * 32 + (lane & 31)];
+  for (int mi = 0; mi < C::MI; ++mi) {
+    srow[mi] = tv.srow[wm * C::WM + mi * 32 + (lane & 31)];
+    zsr[mi] = tv.zs[wm * C::WM + mi * 32 + (lane & 31)];
+  }
   asm volatile("s_nop 15\n\ts_nop 15");  // the last MFMA results are architecturally visible to the reads below
 #pragma unroll
   for (int ni = 0; ni < C::NI; ++ni) {
-    float scv[16];
+    float scv[16], wrv[16], bsv[16];
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
-      const float4 sc = *reinterpret_cast<const float4 *>(tv.scol + wn * C::WN + ni * 32 + acc_col(g, lane));
+      const int c = wn * C::WN + ni * 32 + acc_col(g, lane);
+      const float4 sc = *reinterpret_cast<const float4 *>(tv.scol + c);
+      const float4 wr = *reinterpret_cast<const float4 *>(tv.wred + c);
+      const float4 bs = *reinterpret_cast<const float4 *>(tv.bias + c);
       scv[4 * g] = sc.x, scv[4 * g + 1] = sc.y, scv[4 * g + 2] = sc.z, scv[4 * g + 3] = sc.w;
+      wrv[4 * g] = wr.x, wrv[4 * g + 1] = wr.y, wrv[4 * g + 2] = wr.z, wrv[4 * g + 3] = wr.w;
+      bsv[4 * g] = bs.x, bsv[4 * g + 1] = bs.y, bsv[4 * g + 2] = bs.z, bsv[4 * g + 3] = bs.w;
     }
 #pragma unroll
     for (int mi = 0; mi < C::MI; ++mi) {
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         const float raw = agpr_read(acc[mi][ni][v]);
-        acc[mi][ni][v] = agpr_write(static_cast<float>(__float_as_int(raw)) * (srow[mi] * scv[v]));
+        acc[mi][ni][v] = agpr_write(__builtin_fmaf(static_cast<float>(__float_as_int(raw)), srow[mi] * scv[v],
+                                                   __builtin_fmaf(zsr[mi], wrv[v], bsv[v])));
       }
     }
   }
@@ -336,36 +346,22 @@ __device__ __forceinline__ void fused8t_tile(const Fused8Args &p, int tm, int tn
   pipe.template run<BF16 ? kBF16 : kF16, false>(pipe.steps0, pipe.steps, f0, f1, acc);
   pipe.drain();
 
-  // out = storage(acc + fma(zs, w_red, bias)): all row blocks of the wave staged in the (now idle) ring, read back
+  // out = storage(acc): all row blocks of the wave staged in the (now idle) ring, read back
   // as whole row segments, stored
   using Store = BlockStore<C, uint16_t>;
   static_assert(Store::kBytes * C::MI * C::WAVES <= tile8_vectors_offset<C>(), "staging ends before the vectors");
   uint8_t *stage = smem + wave * (Store::kBytes * C::MI);
   const bool vec = (p.ldo & 7) == 0 && (reinterpret_cast<uintptr_t>(p.out) & 15) == 0;
   const int nw = n0 + wn * C::WN, mw = m0 + wm * C::WM;
-  float4 wr[C::NI][4], bs[C::NI][4];
 #pragma unroll
-  for (int ni = 0; ni < C::NI; ++ni)
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const int c = wn * C::WN + ni * 32 + acc_col(g, lane);
-      wr[ni][g] = *reinterpret_cast<const float4 *>(tv.wred + c);
-      bs[ni][g] = *reinterpret_cast<const float4 *>(tv.bias + c);
-    }
-#pragma unroll
-  for (int mi = 0; mi < C::MI; ++mi) {
-    const float zs = tv.zs[wm * C::WM + mi * 32 + (lane & 31)];
+  for (int mi = 0; mi < C::MI; ++mi)
 #pragma unroll
     for (int ni = 0; ni < C::NI; ++ni)
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
+      for (int g = 0; g < 4; ++g)
         Store::put_pairs(stage + mi * Store::kBytes, lane, ni, g,
-                         pack2_from_f32<BF16>(acc[mi][ni][4 * g] + __builtin_fmaf(zs, wr[ni][g].x, bs[ni][g].x),
-                                              acc[mi][ni][4 * g + 1] + __builtin_fmaf(zs, wr[ni][g].y, bs[ni][g].y)),
-                         pack2_from_f32<BF16>(acc[mi][ni][4 * g + 2] + __builtin_fmaf(zs, wr[ni][g].z, bs[ni][g].z),
-                                              acc[mi][ni][4 * g + 3] + __builtin_fmaf(zs, wr[ni][g].w, bs[ni][g].w)));
-      }
-  }
+                         pack2_from_f32<BF16>(acc[mi][ni][4 * g], acc[mi][ni][4 * g + 1]),
+                         pack2_from_f32<BF16>(acc[mi][ni][4 * g + 2], acc[mi][ni][4 * g + 3]));
   if (vec && p.M - mw >= C::WM && p.N - nw >= C::WN) {  // interior (wave-uniform): straight-line code
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
