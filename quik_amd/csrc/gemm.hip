@@ -17,6 +17,7 @@ using CfgL = Cfg<256, 256, 2, 2, 2>;   // prefill: 128x128 per wave, 256 accumul
 using CfgH = Cfg<256, 128, 2, 2, 2>;   // half-width tile that evens out the last round
 using CfgM = Cfg<128, 128, 2, 2, 2>;   // mid-size problems, two workgroups per CU
 using CfgN = Cfg<128, 64, 2, 2, 2>;    // few tiles: narrower ones put more CUs to work, three workgroups per CU
+using CfgN6 = Cfg<128, 64, 2, 2, 2>;   // 6-bit path, 86 .. ~150 tiles of 128x128 and no K split: twice as many workgroups
 using CfgL8 = Cfg<256, 256, 2, 4, 2>;  // 6-bit path, launches of 256x256 tiles only: two waves per SIMD (1-5 % faster than CfgL)
 using CfgLp = Cfg<256, 256, 2, 2, 0>;  // plain fallbacks
 using CfgMp = Cfg<128, 128, 2, 2, 0>;
@@ -431,6 +432,11 @@ int run_fused6(const Fused6Args &p, hipStream_t st, void *workspace, int64_t wor
   if (plan.kind != Plan::kSplit) {
     const SplitPlan sp = plan_splitk(p.M, p.N, p.K / 64, kSplitMinSteps6, 1, 3);
     if (sp.splits > 1 && workspace && workspace_bytes >= sp.bytes) return launch_fused6_splitk<BF16>(p, sp, workspace, st);
+    // too few 128x128 tiles for the CUs and no K split (it takes three workgroups per tile to pay): 128x64 tiles
+    const int64_t mid_tiles = ((p.M + 127) / 128) * ((p.N + 127) / 128);
+    // (up to 0.62 tiles per CU: measured 6 - 12 % less time on 13B gate_proj at 128 tokens, 70B k_proj and the
+    // 512 x 4096 x 4096 configuration; with 0.88 tiles per CU, 70B gate_proj at 64 tokens, 11 % more)
+    if (mid_tiles * 8 <= int64_t(num_cus()) * 5) return launch_fused6<CfgN6, BF16>(p, st);
     return launch_fused6<CfgM, BF16>(p, st);
   }
   Fused6Args wide = p, tail = p;

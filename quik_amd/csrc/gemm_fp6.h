@@ -46,7 +46,10 @@ __device__ __forceinline__ void dma_load16k(const uint8_t *sbase, uint32_t voff,
 template <class C>
 struct Fp6Pipe {
   static constexpr int MI = C::MI, NI = C::NI, NS = 6, NF = MI + NI;
-  static_assert(C::WM % 64 == 0 && C::WN % 64 == 0, "a wave's rows start at a 64-row block");
+  // a wave's fragments start at a 64-row block of the operand, or the wave has a single 32-row fragment (then it may
+  // be the second half of a block)
+  static_assert(C::WM % 64 == 0 || C::MI == 1, "a wave's token rows");
+  static_assert(C::WN % 64 == 0 || C::NI == 1, "a wave's weight rows");
   static_assert(C::WAVES == 4 || C::WAVES == 8, "copy assignment below");
   // LDS slot of one step: the 3 KB units of the tile's X blocks, then of its W blocks, as they are in memory
   static constexpr int W_OFF = C::BM * 48;
@@ -56,11 +59,11 @@ struct Fp6Pipe {
   // Every wave copies one whole block from its source A (X block w, or W block w - XB when the tile has
   // fewer than 4 X blocks), and NB further kilobytes from its source B:
   //   256x256: W block w (3);  256x128: W block w % 2, pieces w / 2 and w / 2 + 1 (piece 1 is copied twice);
-  //   128x128: none.
+  //   128x128: none;  128x64: none (two waves copy the one W block: the same bytes to the same place).
   static constexpr int XB = C::BM / 64, WB = C::BN / 64;
   // (eight waves, 256x256: one block per wave, no source B)
   static constexpr int NB = C::WAVES == 8 ? 0 : XB + WB == 8 ? 3 : XB + WB == 6 ? 2 : 0;
-  static_assert((XB == 4 && (WB == 4 || WB == 2)) || (XB == 2 && WB == 2), "supported tile shapes");
+  static_assert((XB == 4 && (WB == 4 || WB == 2)) || (XB == 2 && (WB == 2 || WB == 1)), "supported tile shapes");
   static_assert(C::WAVES == 4 || XB + WB == 8, "eight waves copy eight blocks");
   static constexpr int P = 3 + NB;  // copies per wave and step
   static_assert(3 * P <= 63, "three steps in flight must fit the vmcnt counter");
@@ -100,7 +103,7 @@ struct Fp6Pipe {
     };
     {
       const bool is_x = wave < XB;
-      const int blk = is_x ? wave : wave - XB;
+      const int blk = is_x ? wave : (wave - XB) % WB;
       pa = block_ptr(is_x, blk);
       da = (is_x ? 0 : W_OFF) + blk * 3072;
     }
@@ -121,13 +124,17 @@ struct Fp6Pipe {
     left = steps;
     const int r = lane & 31, h = lane >> 5;
     const int slot16 = (h ^ ((r >> 3) & 1)) << 4;
-    x_head = (wm * C::WM / 64) * 3072 + r * 32 + slot16;
-    w_head = W_OFF + (wn * C::WN / 64) * 3072 + r * 32 + slot16;
+    // first 32-row fragment of the wave in each operand: block fx0 / 2 (fw0 / 2), half fx0 % 2 (odd only for waves of
+    // a single fragment)
+    const int fx0 = wm * C::WM / 32, fw0 = wn * C::WN / 32;
+    x_head = (fx0 >> 1) * 3072 + (fx0 & 1) * 1024 + r * 32 + slot16;
+    w_head = W_OFF + (fw0 >> 1) * 3072 + (fw0 & 1) * 1024 + r * 32 + slot16;
 #pragma unroll
     for (int j = 0; j < NF; ++j) {
       const int jj = j < MI ? j : j - MI;
-      tail[j] = (j < MI ? (wm * C::WM / 64) * 3072 : W_OFF + (wn * C::WN / 64) * 3072) + (jj >> 1) * 3072 + 2048 +
-                h * 512 + ((jj & 1) * 32 + r) * 8;
+      const int f0 = j < MI ? fx0 : fw0;
+      tail[j] = (j < MI ? 0 : W_OFF) + (f0 >> 1) * 3072 + (jj >> 1) * 3072 + 2048 + h * 512 +
+                ((((f0 & 1) + jj) & 1) * 32 + r) * 8;
       asm volatile("" : "+v"(tail[j]));  // unrelated values as far as the compiler can tell (empty statement: no hazard)
     }
 #pragma unroll
@@ -263,10 +270,12 @@ struct Fp6Pipe {
       constexpr int r_lo = G * NF / P, r_hi = (G + 1) * NF / P, m_lo = G * MM / P, m_hi = (G + 1) * MM / P;
       chunk_reads6<RS, r_lo, r_hi>(nh, nt);
       chunk_mfmas6<m_lo, m_hi>(ch, ct, acc);
+      if constexpr (m_hi > m_lo) {
 #pragma unroll
-      for (int i = m_lo; i < m_hi; ++i) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, (2 * (r_hi - r_lo) + (m_hi - m_lo) - 1) / (m_hi - m_lo), 0);
+        for (int i = m_lo; i < m_hi; ++i) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, (2 * (r_hi - r_lo) + (m_hi - m_lo) - 1) / (m_hi - m_lo), 0);
+        }
       }
       __builtin_amdgcn_sched_barrier(0);
       issue_one<G, FS>();
@@ -299,10 +308,12 @@ struct Fp6Pipe {
       constexpr int r_lo = G * NF / P, r_hi = (G + 1) * NF / P, m_lo = G * MM / P, m_hi = (G + 1) * MM / P;
       chunk_reads16<r_lo, r_hi>(nf);
       chunk_mfmas16<BF16, m_lo, m_hi>(cf, acc);
+      if constexpr (m_hi > m_lo) {
 #pragma unroll
-      for (int i = m_lo; i < m_hi; ++i) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, ((r_hi - r_lo) + (m_hi - m_lo) - 1) / (m_hi - m_lo), 0);
+        for (int i = m_lo; i < m_hi; ++i) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, ((r_hi - r_lo) + (m_hi - m_lo) - 1) / (m_hi - m_lo), 0);
+        }
       }
       __builtin_amdgcn_sched_barrier(0);
       issue_one<G>();
