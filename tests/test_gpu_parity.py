@@ -1262,6 +1262,7 @@ def test_split_k_gives_the_same_bits(case):
         assert matmul._splitk_workspaces[(torch.cuda.current_device(), side.cuda_stream)] is not ws
     side.synchronize()
     assert np.array_equal(other[0][~nan_rows], want[0][~nan_rows])
+    del matmul._splitk_workspaces[(torch.cuda.current_device(), side.cuda_stream)]   # (the number per GPU is bounded)
 
 
 @pytest.mark.parametrize("M,tiled", [(16, False), (24, True), (32, False), (32, True), (33, True)])
