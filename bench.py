@@ -58,6 +58,12 @@ PEAK_HBM_GBPS = 8000.0    # MI355X HBM3E, published
 # scaled by what the same counter reads for a plain 256 MiB copy): offline figures, kept per workload;
 # the summaries with the commands are profiles/*__llama2-70b.gate_proj*.md and profiles/copy_calibration__256MiB.md
 # (gemm6 / quantize6: the kernels of the 6-bit matrix-core path, the default; gemm / quantize: --int8-mfma)
+# Average duration of the quantize launch by `rocprofv3 --kernel-trace --stats` over this file's default command
+# line (--steps 20 --warmup 5), offline like the traffic figures: the HIP-event interval around a 15 us launch
+# also holds one event record (3 - 4 us) and the gap to the launch in front of it.
+QUANTIZE_KERNEL_TRACE_MS = {
+    "llama2-70b.gate_proj": 0.01482,   # profiles/quantize_fp6_wave_kernel__llama2-70b.gate_proj.md, run (a)
+}
 MEASURED_TRAFFIC_BYTES = {
     "llama2-70b.gate_proj": {"gemm": 831.3e6, "quantize": 43.0e6, "gemm6": 767.8e6, "quantize6": 47.1e6},
 }
@@ -590,6 +596,10 @@ def main():
                               "traffic": traffic.get("quantize6" if six else "quantize"), "avg_ms": round(q_avg, 5),
                               "median_ms": round(q_ms[len(q_ms) // 2], 5), "algorithmic_bytes": quant_bytes,
                               "back_to_back_ms": round(q_b2b, 5),
+                              "kernel_trace_avg_ms": QUANTIZE_KERNEL_TRACE_MS.get(name) if six and bits == 4 else None,
+                              "frac_by_kernel_trace": round(quant_bytes / (QUANTIZE_KERNEL_TRACE_MS[name] * 1e-3) / 1e9
+                                                            / PEAK_HBM_GBPS, 4)
+                              if six and bits == 4 and name in QUANTIZE_KERNEL_TRACE_MS else None,
                               "note": "avg_ms: from an event in front of the forward to the event the library records "
                                       "between the quantize launch and the GEMM launch (the launch plus the cost of "
                                       "one event record, several us); back_to_back_ms: per launch over 50 consecutive "
