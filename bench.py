@@ -409,12 +409,13 @@ def main():
             return quantize6(x, colmap, K, F)
         return asymmetric.quantize_mapped(x, colmap, K, F, bits)
 
-    def step(ev=None):
+    def step(ev=None, before=True):
         """One forward of the layer.  Fused (the default): ONE call of the module, mod(x) -> quik_layer_forward, which
         launches the quantize kernel and the fused GEMM.  --unfused: the reference's op sequence through the stand-alone
         ops.  ev = (before, between, after): events on the launch stream; in the fused form the library records the
-        middle one between its two launches."""
-        if ev is not None:
+        middle one between its two launches.  before=False: the step in front of this one recorded its `after` event,
+        which then serves as this step's `before` (one event record per step less)."""
+        if ev is not None and before:
             ev[0].record()
         if mod.fused:
             if ev is not None:
@@ -441,9 +442,10 @@ def main():
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
-    # Kernel durations from HIP events inside the timed region (three per step: before, between the two launches,
-    # after; an event record between two launches costs 3 - 4 us on the GPU's timeline, which ms_per_step includes;
-    # --event-every N records them on every N-th step only).
+    # Kernel durations from HIP events inside the timed region: between the two launches (recorded by the library) and
+    # after the forward; the event after one forward is the event before the next.  An event record between two
+    # launches costs 3 - 4 us on the GPU's timeline, which ms_per_step includes (--event-every N records them on
+    # every N-th step only).
     every = max(1, args.event_every)
     events = {i: [torch.cuda.Event(enable_timing=True) for _ in range(3)] for i in range(0, args.steps, every)}
     for evs in events.values():        # an event has a handle only once it has been recorded
@@ -452,11 +454,11 @@ def main():
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(args.steps):
-        step(events.get(i))
+        step(events.get(i), before=(i - 1) not in events)
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     ms_step = (t1 - t0) * 1e3 / args.steps
-    q_ms = sorted(e[0].elapsed_time(e[1]) for e in events.values())
+    q_ms = sorted((events[i - 1][2] if (i - 1) in events else e[0]).elapsed_time(e[1]) for i, e in events.items())
     g_ms = sorted(e[1].elapsed_time(e[2]) for e in events.values())
     q_avg, g_avg = sum(q_ms) / len(q_ms), sum(g_ms) / len(g_ms)
 
@@ -600,9 +602,9 @@ def main():
                               "frac_by_kernel_trace": round(quant_bytes / (QUANTIZE_KERNEL_TRACE_MS[name] * 1e-3) / 1e9
                                                             / PEAK_HBM_GBPS, 4)
                               if six and bits == 4 and name in QUANTIZE_KERNEL_TRACE_MS else None,
-                              "note": "avg_ms: from an event in front of the forward to the event the library records "
-                                      "between the quantize launch and the GEMM launch (the launch plus the cost of "
-                                      "one event record, several us); back_to_back_ms: per launch over 50 consecutive "
+                              "note": "avg_ms: from the event behind the previous forward to the event the library "
+                                      "records between the quantize launch and the GEMM launch (the launch plus the "
+                                      "cost of one event record, several us); back_to_back_ms: per launch over 50 consecutive "
                                       "launches after the timed region (bound by the host: ~14 us of Python per "
                                       "call); kernel-trace durations: profiles/"},
     }
