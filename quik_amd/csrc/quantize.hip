@@ -908,10 +908,18 @@ __global__ __launch_bounds__(64) void quantize_fp6_wave_kernel(
     float mn = inf, mx = -inf;
     uint32_t pmn_b = 0x7C007C00u, pmx_b = 0xFC00FC00u;  // +inf / -inf in both halves
     u2 amax = u2{0, 0};
+    // up to four fragments per lane stay in registers from the first pass to the second (64 registers): the second
+    // pass then has no LDS round trip in front of its arithmetic
+    constexpr bool kKeep = JT > 0 && JT <= 4;
+    uint4 kept[kKeep ? JT : 1][4];
     for_j([&](int j) {
       if (lane + 64 * j < frags) {
         uint4 v[4];
         load_fragment(j, v);
+        if constexpr (kKeep) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) kept[j][i] = v[i];
+        }
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const uint32_t w[4] = {v[i].x, v[i].y, v[i].z, v[i].w};
@@ -964,7 +972,12 @@ __global__ __launch_bounds__(64) void quantize_fp6_wave_kernel(
         const int f = lane + 64 * j;
         if (f < frags) {
           uint4 v[4];
-          load_fragment(j, v);
+          if constexpr (kKeep) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) v[i] = kept[j][i];
+          } else {
+            load_fragment(j, v);
+          }
           uint32_t b[8];  // 32 levels, one per byte
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
