@@ -55,17 +55,19 @@ PEAK_FP6_TOPS = 10100.0   # MI355X dense fp6 / fp4 MFMA, published
 PEAK_HBM_GBPS = 8000.0    # MI355X HBM3E, published
 
 # HBM/fabric bytes per launch from rocprofv3 counter runs of this file (FETCH_SIZE and WRITE_SIZE, each
-# scaled by what the same counter reads for a plain 256 MiB copy): offline figures, kept per workload;
-# the summaries with the commands are profiles/*__llama2-70b.gate_proj*.md and profiles/copy_calibration__256MiB.md
-# (gemm6 / quantize6: the kernels of the 6-bit matrix-core path, the default; gemm / quantize: --int8-mfma)
-# Average duration of the quantize launch by `rocprofv3 --kernel-trace --stats` over this file's default command
-# line (--steps 20 --warmup 5), offline like the traffic figures: the HIP-event interval around a 15 us launch
-# also holds one event record (3 - 4 us) and the gap to the launch in front of it.
-QUANTIZE_KERNEL_TRACE_MS = {
-    "llama2-70b.gate_proj": 0.01513,   # profiles/quantize_fp6_wave_kernel__llama2-70b.gate_proj.md, run (a)
-}
+# scaled by what the same counter reads for a plain 256 MiB copy).  OFFLINE figures: they come from the profiler
+# summaries named beside them, not from the run that prints them, and are labelled so in the JSON line
+# (`traffic_source`).  (gemm6 / quantize6: the kernels of the 6-bit matrix-core path, the default; gemm / quantize:
+# --int8-mfma)
 MEASURED_TRAFFIC_BYTES = {
     "llama2-70b.gate_proj": {"gemm": 831.3e6, "quantize": 43.0e6, "gemm6": 767.1e6, "quantize6": 47.1e6},
+}
+TRAFFIC_SOURCE = {
+    "gemm6": "offline: profiles/gemm_fused6_split_kernel__llama2-70b.gate_proj.md (rocprofv3 --pmc FETCH_SIZE / "
+             "WRITE_SIZE, scaled by profiles/copy_calibration__256MiB.md)",
+    "quantize6": "offline: profiles/quantize_fp6_wave_kernel__llama2-70b.gate_proj.md",
+    "gemm": "offline: profiles/gemm_fused_split_kernel__llama2-70b.gate_proj.md",
+    "quantize": "offline: profiles/asym_quantize_stream_kernel__llama2-70b.gate_proj.md",
 }
 
 
@@ -117,6 +119,20 @@ def verify_spot_tile(name, out, x_cpu, W_cpu, fp_idx, mod, rows=48, cols=64):
         assert rel <= 1e-2, f"bench.py: output differs from the oracle on tile ({r0}, {c0}): {rel:.3e} x RMS"
         worst = max(worst, rel)
     return worst
+
+
+def spread(block_ms, int_ops):
+    """Per-step times of the timed blocks (the first one is the block `value` comes from) -> median, mean and
+    1.96 sigma (the reference's confidence interval, experiments/layer_benchmark.py:29-31), in ms and TOPS."""
+    import statistics
+    n = len(block_ms)
+    mean = sum(block_ms) / n
+    sd = statistics.stdev(block_ms) if n > 1 else 0.0
+    med = statistics.median(block_ms)
+    tops = lambda ms: round(int_ops / (ms * 1e-3) / 1e12, 1)
+    return {"blocks": n, "ms_per_step_each": [round(b, 4) for b in block_ms], "median_ms": round(med, 4),
+            "mean_ms": round(mean, 4), "ci95_ms": round(1.96 * sd, 4), "median_tops": tops(med), "mean_tops": tops(mean),
+            "pct_int8_mfma_peak_median": round(100.0 * int_ops / (med * 1e-3) / 1e12 / PEAK_INT8_TOPS, 2)}
 
 
 def cpu_baseline(name, x, W, int_idx, fp_idx, budget_s=25.0):
@@ -347,6 +363,10 @@ def main():
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="llama2-70b.gate_proj", choices=sorted(WORKLOADS) + sorted(BLOCK_WORKLOADS))
+    ap.add_argument("--repeats", type=int, default=5,
+                    help="further timed blocks of --steps forwards each, run after the block that gives `value` "
+                         "(the reference's protocol repeats its timed block and reports mean +- 1.96 sigma, "
+                         "experiments/layer_benchmark.py:19-31); their spread is printed as `repeats` (0: none)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--event-every", type=int, default=1,
                     help="record the HIP events that time the two kernels on every N-th timed step (default: every step)")
@@ -484,6 +504,20 @@ def main():
         torch.cuda.synchronize()
         module_ms = (time.perf_counter() - t0) * 1e3 / args.steps
 
+    # Spread of the headline: `value` comes from the one timed block above (exactly --steps forwards after --warmup
+    # warm-up forwards).  The same block (with its event records) is timed --repeats more times, back to back, as the
+    # reference's layer benchmark repeats its timed block; median, mean and 1.96 sigma of the per-step time over ALL
+    # blocks, the first included, go into `repeats`.  On this part the first block after an idle period runs in the
+    # window in which the power management has just pulled the clock down, so it is usually the slowest.
+    block_ms = [ms_step]
+    for _ in range(max(0, args.repeats)):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(args.steps):
+            step(events.get(i), before=(i - 1) not in events)
+        torch.cuda.synchronize()
+        block_ms.append((time.perf_counter() - t0) * 1e3 / args.steps)
+
     # the same step replayed from a HIP graph (extra figure: what a serving loop that captures the layer sees;
     # for small token counts the eager step is bound by Python launch overhead, not by the kernels)
     graph_ms = None
@@ -575,6 +609,7 @@ def main():
                                f"{', 6-bit matrix-core path' if six and bits == 4 else ', tile-ordered operands' if six else ''}",
                    "M": M, "in_features": n_in, "K": K, "N": N, "F": F, "bits": bits},
         "pct_int8_mfma_peak": round(100.0 * tops / PEAK_INT8_TOPS, 2),
+        "repeats": spread(block_ms, int_ops),
         "module_forward_ms_per_step": None if module_ms is None else round(module_ms, 4),
         "graph_replay_ms_per_step": None if graph_ms is None else round(graph_ms, 4),
         "cold_ms_per_forward": None if cold_ms is None else round(cold_ms, 4),
@@ -588,6 +623,8 @@ def main():
                      "unit": "TOP/s", "frac": round(gemm_tops / peak, 4),
                      "frac_of_int8_peak": round(gemm_tops / PEAK_INT8_TOPS, 4),
                      "traffic": traffic.get("gemm6" if six else "gemm") if mod.fused else None,
+                     "traffic_source": TRAFFIC_SOURCE["gemm6" if six else "gemm"]
+                     if mod.fused and traffic.get("gemm6" if six else "gemm") else None,
                      "avg_ms": round(g_avg, 4), "median_ms": round(g_ms[len(g_ms) // 2], 4),
                      "timed_launches": len(g_ms), "algorithmic_ops": int_ops},
         "roofline_quantize": {"kernel": ("quantize_fp6_wave_kernel (one wave per token row, 6-bit operand output)" if six and bits == 4
@@ -595,18 +632,17 @@ def main():
                               "bound": "hbm",
                               "achieved": round(quant_gbps, 1),
                               "peak": PEAK_HBM_GBPS, "unit": "GB/s", "frac": round(quant_gbps / PEAK_HBM_GBPS, 4),
-                              "traffic": traffic.get("quantize6" if six else "quantize"), "avg_ms": round(q_avg, 5),
+                              "traffic": traffic.get("quantize6" if six else "quantize"),
+                              "traffic_source": TRAFFIC_SOURCE["quantize6" if six else "quantize"]
+                              if traffic.get("quantize6" if six else "quantize") else None,
+                              "avg_ms": round(q_avg, 5),
                               "median_ms": round(q_ms[len(q_ms) // 2], 5), "algorithmic_bytes": quant_bytes,
                               "back_to_back_ms": round(q_b2b, 5),
-                              "kernel_trace_avg_ms": QUANTIZE_KERNEL_TRACE_MS.get(name) if six and bits == 4 else None,
-                              "frac_by_kernel_trace": round(quant_bytes / (QUANTIZE_KERNEL_TRACE_MS[name] * 1e-3) / 1e9
-                                                            / PEAK_HBM_GBPS, 4)
-                              if six and bits == 4 and name in QUANTIZE_KERNEL_TRACE_MS else None,
                               "note": "avg_ms: from the event behind the previous forward to the event the library "
                                       "records between the quantize launch and the GEMM launch (the launch plus the "
                                       "cost of one event record, several us); back_to_back_ms: per launch over 50 consecutive "
                                       "launches after the timed region (bound by the host: ~14 us of Python per "
-                                      "call); kernel-trace durations: profiles/"},
+                                      "call); kernel-trace durations of the launch alone: profiles/"},
     }
     if not args.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline(name, x_cpu, W_cpu, int_idx, fp_idx)

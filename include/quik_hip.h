@@ -27,7 +27,11 @@ typedef enum quik_status {
   QUIK_ERR_ALIGN = -4,     /* K or a pointer violates the alignment the op needs */
   QUIK_ERR_NULL = -5,      /* required pointer is NULL */
   QUIK_ERR_RANGE = -6,     /* size beyond what the kernel supports */
-  QUIK_ERR_LAUNCH = -7     /* HIP reported a launch error; hipGetLastError text via quik_last_hip_error() */
+  QUIK_ERR_LAUNCH = -7,    /* HIP reported a launch error; hipGetLastError text via quik_last_hip_error() */
+  QUIK_ERR_COLMAP = -8     /* the column map does not select the streaming quantize kernel (or has no in-place
+                              order) and this entry point has no other path; also: the map's flags are not known
+                              to the host yet and the stream is being captured (call quik_colmap_streaming once
+                              per map outside the capture).  Nothing was launched. */
 } quik_status;
 
 typedef enum quik_dtype { QUIK_F16 = 0, QUIK_BF16 = 1 } quik_dtype;
@@ -147,8 +151,12 @@ int64_t quik_fp6_operand_bytes(int64_t rows, int64_t K, int64_t F);
 int quik_fp6_pack_weight(const uint8_t *qw, const void *fp_w, int64_t N, int64_t K, int64_t F,
                          const void *colmap, void *out, void *stream);
 
-/* 1 if the column map selects the streaming quantize kernel (ascending int_indices, ...), 0 if not,
- * negative on error; copies one word from the device and synchronises the stream: call once per layer */
+/* 1 if the column map selects the streaming quantize kernel (ascending int_indices that, with fp_indices,
+ * partition the columns; cols % 8 == 0; cols <= 32768), 0 if not, negative on error.  The first call for a map
+ * copies one word from the device and synchronises the stream; the library remembers the answer per (address,
+ * shape) until quik_colmap_build writes to that address again.  The entry points that need such a map
+ * (quik_asym_quantize_fp6, quik_asym_quantize_tile8, quik_sym_quantize_mapped, quik_fp6_pack_weight) make the
+ * same look-up themselves and return QUIK_ERR_COLMAP, launching nothing, for a map that does not qualify. */
 int quik_colmap_streaming(const void *colmap, int64_t cols, int64_t num_int, int64_t num_fp, void *stream);
 
 /* as quik_asym_quantize with bits = 4, but codes and outlier values go to an operand buffer

@@ -15,6 +15,20 @@ int num_cus();       // compute units of the GPU (asked once per process; 256 wh
 
 inline hipStream_t as_stream(void *s) { return reinterpret_cast<hipStream_t>(s); }
 
+// runtime.hip: flags word of a column map (colmap.h: bit 0 = streams, bit 1 = in-place order), copied from the
+// device once per (address, shape) and remembered; colmap_forget drops what is known about an address.
+// QUIK_ERR_COLMAP when the word is not known yet and `st` is being captured (no synchronisation possible there).
+constexpr uint32_t kColmapStreams = 1u, kColmapInPlace = 2u;
+int colmap_flags(const void *colmap, int64_t cols, int64_t num_int, int64_t num_fp, hipStream_t st, uint32_t *flags);
+void colmap_forget(const void *colmap);
+// QUIK_OK when the column map has all bits of `need` set, QUIK_ERR_COLMAP when not (or an error of colmap_flags)
+inline int colmap_require(const void *colmap, int64_t cols, int64_t num_int, int64_t num_fp, hipStream_t st,
+                          uint32_t need) {
+  uint32_t flags = 0;
+  if (int rc = colmap_flags(colmap, cols, num_int, num_fp, st, &flags)) return rc;
+  return (flags & need) == need ? QUIK_OK : QUIK_ERR_COLMAP;
+}
+
 // gemm.hip: integer GEMM + the fp16-arithmetic epilogue of the reference's fused ops in one launch (zero_row ==
 // NULL: symmetric form).  Returns kChainNotHandled for shapes it leaves to the two-launch path.
 constexpr int kChainNotHandled = 1;

@@ -108,6 +108,7 @@ extern "C" int quik_fp6_pack_weight(const uint8_t *qw, const void *fp_w, int64_t
       reinterpret_cast<uintptr_t>(fp_w) % 16 != 0 || reinterpret_cast<uintptr_t>(colmap) % 16 != 0)
     return QUIK_ERR_ALIGN;
   if (N > (1 << 30) || K > 74496 || K + F > kStreamMaxCols) return QUIK_ERR_RANGE;
+  if (int rc = colmap_require(colmap, K + F, K, F, as_stream(stream), kColmapStreams | kColmapInPlace)) return rc;
   const ColmapLayout cl = colmap_layout(K + F, K, F);
   const uint8_t *cm = static_cast<const uint8_t *>(colmap);
   hipLaunchKernelGGL(pack_weight_kernel, dim3(static_cast<unsigned>(N)), dim3(kThreads), static_cast<size_t>(K / 2),

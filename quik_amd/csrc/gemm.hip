@@ -23,6 +23,13 @@ using CfgLp = Cfg<256, 256, 2, 2, 0>;  // plain fallbacks
 using CfgMp = Cfg<128, 128, 2, 2, 0>;
 
 constexpr int kMaxCUs = 256;  // MI355X; sizes the static K-split scratch array
+
+// Zero-fill of a few words by a kernel: the arrival counters of the K split are cleared with it, not with
+// hipMemsetAsync, because the caller's stream may be under capture and a memset node in a captured graph is not
+// reliable on replays.
+__global__ __launch_bounds__(256) void clear_words_kernel(uint32_t *p, int words) {
+  for (int i = blockIdx.x * 256 + threadIdx.x; i < words; i += gridDim.x * 256) p[i] = 0u;
+}
 constexpr int kLdsBytes = 160 * 1024;  // per CU, and the most one workgroup may ask for
 
 // Kernels that ask for more than 48 KB of dynamic LDS need the attribute raised once per device; the (kernel,
@@ -146,7 +153,9 @@ template <int MODE, bool BF16, bool FUSED, int WAVES, bool XLDS>
 int launch_decode_w(const FusedArgs &p, int32_t *C, int ldc, hipStream_t st) {
   auto kern = gemm_decode_kernel<MODE, BF16, FUSED, WAVES, XLDS>;
   const int smem = decode_smem<WAVES, FUSED, XLDS>() + (XLDS ? static_cast<int>(decode_x_lds_bytes(p.M, p.kbytes)) : 0);
-  if (int rc = prepare(kern, smem)) return rc;
+  // XLDS: the LDS size varies from call to call with the row count, and prepare() sets the attribute once per
+  // kernel and device: set it to the most any call may ask for
+  if (int rc = prepare(kern, XLDS ? kLdsBytes : smem)) return rc;
   // persistent workgroups: as many as are resident at once (8 waves per CU at this register count; the LDS copy
   // of the token rows leaves room for one workgroup)
   // Every workgroup walks the same number of slabs (one more or less): with 896 slabs, 224 workgroups of 4 slabs
@@ -365,7 +374,11 @@ SplitPlan plan_splitk(int64_t M, int64_t N, int64_t steps, int64_t min_steps, in
 // behind a failed launch so that the next one on this workspace starts clean.
 int splitk_launch_status(void *workspace, hipStream_t st) {
   const int rc = check_launch();
-  if (rc != QUIK_OK) (void)hipMemsetAsync(workspace, 0, kSplitCounterBytes, st);
+  if (rc != QUIK_OK) {
+    hipLaunchKernelGGL(clear_words_kernel, dim3(static_cast<unsigned>(kSplitCounterBytes / 4 / 256)), dim3(256), 0, st,
+                       static_cast<uint32_t *>(workspace), static_cast<int>(kSplitCounterBytes / 4));
+    (void)hipGetLastError();  // the status reported is that of the launch that failed
+  }
   return rc;
 }
 
@@ -723,12 +736,8 @@ int scratch_of_current_device(uint8_t **out) {
   return QUIK_OK;
 }
 
-// The arrival counters must be zero when a launch starts.  Launches leave them at zero, but a launch that failed
-// half way would not, and this array outlives every caller: clear them in front of each launch that uses them,
-// with a kernel (a memset node in a captured graph is not reliable on replays).
-__global__ __launch_bounds__(256) void clear_words_kernel(uint32_t *p, int words) {
-  for (int i = blockIdx.x * 256 + threadIdx.x; i < words; i += gridDim.x * 256) p[i] = 0u;
-}
+// (the counters of `scratch` are cleared with clear_words_kernel in front of each launch that uses them: launches
+// leave them at zero, but a launch that failed half way would not, and this array outlives every caller)
 }  // namespace
 }  // namespace quik
 

@@ -72,8 +72,16 @@ __global__ __launch_bounds__(1024) void colmap_build_kernel(const int64_t *__res
     atomicOr(&mask[c >> 5], 1u << (c & 31));
   }
   __syncthreads();
+  // the two lists must not share a column (the streaming kernels take the integer columns as the complement of
+  // the outlier mask, the gather kernels take them from src_col: they agree only for a partition)
+  for (int64_t j = threadIdx.x; j < num_int; j += blockDim.x) {
+    const int64_t c = int_idx[j];
+    if (c >= 0 && c < cols && ((mask[c >> 5] >> (c & 31)) & 1u)) ascending = 0;
+  }
+  __syncthreads();
   const bool stream_shape = cols <= kStreamMaxCols && cols % 8 == 0;
-  // duplicates between the two index lists would make the popcount prefix wrong: require a partition
+  // ascending int_indices (strictly, in range, none of them an outlier column) and num_fp distinct outlier
+  // columns, num_int + num_fp == cols: a partition
   uint32_t total = 0, total_dirty = 0;
   if (threadIdx.x == 0) {
     for (int64_t w = 0; w < words; ++w) {
@@ -742,7 +750,7 @@ __global__ __launch_bounds__(TPR) void asym_quantize_stream_kernel(
   } else if constexpr (!SYM) {
     // Tile-ordered output exists on the streaming path only: a column map that does not stream (any other index
     // order) must not reach the row-major gather code with an operand buffer as `dst` and no `fp_x`.  Nothing is
-    // written then; the host wrappers refuse such a column map before launching.
+    // written then; the entry points refuse such a column map before launching.
     if (vec_out >= 2) return;
     gather_rows<IdxT, BITS, BF16, TPR>(x, rows, cols, src_col, fp_col, mask, num_int, num_fp, dst, meta, fp_x, 1,
                                        row_s, red);
@@ -816,7 +824,7 @@ __global__ __launch_bounds__(64) void quantize_fp6_wave_kernel(
     uint8_t *__restrict__ dst, uint16_t *__restrict__ meta, float sym_divisor) {
   static_assert(!(BF16 && SYM), "symmetric activations are fp16");
   extern __shared__ __align__(16) uint8_t row_img[];
-  if (!(flags[0] & 2u)) return;  // the column map has no in-place order: nothing is written (the host refuses first)
+  if (!(flags[0] & 2u)) return;  // no in-place order: nothing to write (the entry points refuse such a map before launching)
   const int lane = threadIdx.x;
   const int frags_all = cols >> 5, frags = num_int >> 5, nchunk = num_fp >> 3;
   const int J = JT > 0 ? JT : (frags_all + 63) >> 6;
@@ -1328,6 +1336,7 @@ extern "C" int quik_colmap_build(const int64_t *int_indices, int64_t num_int, co
   if (cols <= 0 || num_int < 0 || num_fp < 0 || num_int + num_fp != cols) return QUIK_ERR_SHAPE;
   if (!colmap || (num_int > 0 && !int_indices) || (num_fp > 0 && !fp_indices)) return QUIK_ERR_NULL;
   if (cols > (int64_t(1) << 31)) return QUIK_ERR_RANGE;
+  colmap_forget(colmap);  // whatever was known about a map at this address is void
   const ColmapLayout l = colmap_layout(cols, num_int, num_fp);
   uint8_t *cm = static_cast<uint8_t *>(colmap);
   uint32_t *mask = reinterpret_cast<uint32_t *>(cm + l.off_mask);
@@ -1382,16 +1391,9 @@ extern "C" int quik_asym_quantize(const void *x, int dtype, int64_t rows, int64_
 
 extern "C" int quik_colmap_streaming(const void *colmap, int64_t cols, int64_t num_int, int64_t num_fp, void *stream) {
   if (!colmap || cols <= 0 || num_int < 0 || num_fp < 0 || num_int + num_fp != cols) return QUIK_ERR_SHAPE;
-  const ColmapLayout l = colmap_layout(cols, num_int, num_fp);
   uint32_t flags = 0;
-  hipStream_t st = as_stream(stream);
-  if (hipMemcpyAsync(&flags, static_cast<const uint8_t *>(colmap) + l.off_flags, sizeof(flags), hipMemcpyDeviceToHost,
-                     st) != hipSuccess ||
-      hipStreamSynchronize(st) != hipSuccess) {
-    set_last_hip_error(hipGetLastError());
-    return QUIK_ERR_LAUNCH;
-  }
-  return (flags & 1u) ? 1 : 0;
+  if (int rc = colmap_flags(colmap, cols, num_int, num_fp, as_stream(stream), &flags)) return rc;
+  return (flags & kColmapStreams) ? 1 : 0;
 }
 
 extern "C" int quik_asym_quantize_fp6(const void *x, int dtype, int64_t rows, int64_t cols, const void *colmap,
@@ -1402,6 +1404,7 @@ extern "C" int quik_asym_quantize_fp6(const void *x, int dtype, int64_t rows, in
   if (rows == 0) return QUIK_OK;
   if (!x || !colmap || !out6 || !meta) return QUIK_ERR_NULL;
   if (reinterpret_cast<uintptr_t>(x) % 16 != 0 || reinterpret_cast<uintptr_t>(out6) % 256 != 0) return QUIK_ERR_ALIGN;
+  if (int rc = colmap_require(colmap, cols, num_int, num_fp, as_stream(stream), kColmapStreams | kColmapInPlace)) return rc;
   const ColmapLayout l = colmap_layout(cols, num_int, num_fp);
   const uint8_t *cm = static_cast<const uint8_t *>(colmap);
   hipStream_t st = as_stream(stream);
@@ -1417,6 +1420,7 @@ extern "C" int quik_asym_quantize_tile8(const void *x, int dtype, int64_t rows, 
   if (rows == 0) return QUIK_OK;
   if (!x || !colmap || !out8 || !meta) return QUIK_ERR_NULL;
   if (reinterpret_cast<uintptr_t>(x) % 16 != 0 || reinterpret_cast<uintptr_t>(out8) % 256 != 0) return QUIK_ERR_ALIGN;
+  if (int rc = colmap_require(colmap, cols, num_int, num_fp, as_stream(stream), kColmapStreams)) return rc;
   const ColmapLayout l = colmap_layout(cols, num_int, num_fp);
   const uint8_t *cm = static_cast<const uint8_t *>(colmap);
   hipStream_t st = as_stream(stream);
@@ -1437,6 +1441,9 @@ extern "C" int quik_sym_quantize_mapped(const void *x, int64_t rows, int64_t col
   if (!x || !colmap || !dst || !scale || (!tiled && num_fp > 0 && !fp_x)) return QUIK_ERR_NULL;
   if (reinterpret_cast<uintptr_t>(x) % 16 != 0 || reinterpret_cast<uintptr_t>(dst) % (tiled ? 256 : 1) != 0)
     return QUIK_ERR_ALIGN;
+  if (int rc = colmap_require(colmap, cols, num_int, num_fp, as_stream(stream),
+                              kColmapStreams | (bits == 4 && tiled ? kColmapInPlace : 0u)))
+    return rc;
   const ColmapLayout l = colmap_layout(cols, num_int, num_fp);
   const uint8_t *cm = static_cast<const uint8_t *>(colmap);
   hipStream_t st = as_stream(stream);

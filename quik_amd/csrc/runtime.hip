@@ -1,8 +1,11 @@
 // Status strings and the last-HIP-error slot of libquik_hip.so.
+#include "colmap.h"
 #include "common.h"
 
 #include <atomic>
 #include <cstring>
+#include <mutex>
+#include <unordered_map>
 
 namespace quik {
 namespace {
@@ -29,6 +32,63 @@ int num_cus() {
   return n;
 }
 
+// ---- flags of the column maps this process has used -----------------------------------------------------------
+// The flags word of a column map (colmap.h) lives on the device.  Entry points that have no kernel path for a map
+// without the streaming flag (or without the in-place order) must refuse such a map instead of launching a kernel
+// that writes nothing, so they need the word on the host: it is copied once per (address, shape), with one stream
+// synchronisation, and remembered.  quik_colmap_build forgets the address it writes to, so an address that is
+// reused for another map is read again; a map must therefore be used at the address it was built at (a copy to
+// another address is simply read once more; overwriting a known map by other means than quik_colmap_build is not
+// supported).  A stream that is being captured cannot be synchronised: a map whose flags are not known yet is
+// refused there (QUIK_ERR_COLMAP); call quik_colmap_streaming once per map outside the capture.
+namespace {
+struct ColmapFlags {
+  int64_t cols, num_int, num_fp;
+  uint32_t flags;
+};
+std::mutex g_colmap_mutex;
+std::unordered_map<const void *, ColmapFlags> g_colmap_flags;
+constexpr size_t kMaxKnownColmaps = 1 << 16;
+}  // namespace
+
+void colmap_forget(const void *colmap) {
+  std::lock_guard<std::mutex> lock(g_colmap_mutex);
+  g_colmap_flags.erase(colmap);
+}
+
+int colmap_flags(const void *colmap, int64_t cols, int64_t num_int, int64_t num_fp, hipStream_t st, uint32_t *flags) {
+  {
+    std::lock_guard<std::mutex> lock(g_colmap_mutex);
+    auto it = g_colmap_flags.find(colmap);
+    if (it != g_colmap_flags.end() && it->second.cols == cols && it->second.num_int == num_int &&
+        it->second.num_fp == num_fp) {
+      *flags = it->second.flags;
+      return QUIK_OK;
+    }
+  }
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(st, &capture) != hipSuccess) {
+    set_last_hip_error(hipGetLastError());
+    return QUIK_ERR_LAUNCH;
+  }
+  if (capture != hipStreamCaptureStatusNone) return QUIK_ERR_COLMAP;
+  const ColmapLayout l = colmap_layout(cols, num_int, num_fp);
+  uint32_t word = 0;
+  if (hipMemcpyAsync(&word, static_cast<const uint8_t *>(colmap) + l.off_flags, sizeof(word), hipMemcpyDeviceToHost,
+                     st) != hipSuccess ||
+      hipStreamSynchronize(st) != hipSuccess) {
+    set_last_hip_error(hipGetLastError());
+    return QUIK_ERR_LAUNCH;
+  }
+  {
+    std::lock_guard<std::mutex> lock(g_colmap_mutex);
+    if (g_colmap_flags.size() >= kMaxKnownColmaps) g_colmap_flags.clear();
+    g_colmap_flags[colmap] = ColmapFlags{cols, num_int, num_fp, word};
+  }
+  *flags = word;
+  return QUIK_OK;
+}
+
 int check_launch() {
   hipError_t e = hipGetLastError();
   if (e == hipSuccess) return QUIK_OK;
@@ -47,6 +107,9 @@ extern "C" const char *quik_status_string(int status) {
     case QUIK_ERR_NULL: return "required pointer is null";
     case QUIK_ERR_RANGE: return "size beyond what the kernel supports";
     case QUIK_ERR_LAUNCH: return "HIP launch failed";
+    case QUIK_ERR_COLMAP:
+      return "the column map does not select the streaming quantize kernel (ascending int_indices that partition "
+             "the columns with fp_indices), or its flags are not known yet inside a stream capture";
     default: return "unknown status";
   }
 }

@@ -227,7 +227,9 @@ class MixedQLinear(torch.nn.Module):
         bufs = (self.int_weight, self.weights_scales, self.int_indices, self.fp_indices,
                 self.reduced_w if not self.symmetric else None, self.fp_weight if self.fp_features_num > 0 else None,
                 self.bias)
-        key = tuple((b.data_ptr(), b._version) if b is not None else None for b in bufs)
+        # (the scalar switches below are baked into the descriptor too: changing one after a forward rebuilds it)
+        key = tuple((b.data_ptr(), b._version) if b is not None else None for b in bufs) + \
+            (self.six_bit_min_rows, self.tile8_min_rows, float(self.sym_divisor), bool(self.six_bit_path))
         entry = self._descs.get(tiled)
         if entry is None or entry[0] != key:
             w6 = self._weight6() if tiled else None

@@ -119,6 +119,8 @@ DEFAULT_ROUTE = [
     (2049, 8192, 28672, 256, 4, False, "x50"),      # Llama-2-70B gate/up, one row more than the tiles hold: ragged last row block
     (2048, 8192, 28672, 256, 4, False, "x50", torch.bfloat16),     # Llama-2-70B gate/up, bf16 activations and weights
     (2048, 13824, 5120, 256, 8, False, "student", torch.bfloat16),  # Llama-2-13B down_proj, W8A8, bf16
+    (512, 4096, 4096, 128, 4, False, "x50"),        # the single-layer configuration of the CPU simulated path: 512 tokens, 128 outliers
+    (512, 4096, 4096, 128, 4, True, "x50"),         # ... symmetric activations
 ]
 
 

@@ -1390,12 +1390,54 @@ def test_tile_ordered_ops_refuse_a_column_map_that_does_not_stream():
         asymmetric.quantize_mapped(xt, cm_ok.view(torch.int8), K, F, 4)
     with pytest.raises(RuntimeError, match="CUDA"):
         asymmetric.quantize_mapped_fp6(xt, cm_ok.cpu(), K, F)
-    # the C entry point itself, called with such a map, writes nothing (and does not fault)
+    # the C entry points themselves refuse such a map (QUIK_ERR_COLMAP = -8) and launch nothing
     from quik_amd import _lib as L
     lib = L.load()
-    nbytes = lib.quik_fp6_operand_bytes(M, K, F)
-    buf = torch.full((nbytes,), 0x5A, dtype=torch.uint8, device=DEV)
-    meta6 = torch.zeros(2 * M, dtype=torch.float16, device=DEV)
-    rc = lib.quik_asym_quantize_fp6(L.ptr(xt), L.QUIK_F16, M, n_in, L.ptr(cm), K, F, L.ptr(buf), L.ptr(meta6), L.stream())
+    ERR_COLMAP = -8
+    assert b"column map" in lib.quik_status_string(ERR_COLMAP)
+
+    def c_calls(colmap):
+        """return codes of the four entry points that exist on the streaming kernel only; none may write"""
+        nbytes = lib.quik_fp6_operand_bytes(M, K, F)
+        buf = torch.full((max(nbytes, lib.quik_tile8_operand_bytes(M, K, F)),), 0x5A, dtype=torch.uint8, device=DEV)
+        meta6 = torch.zeros(2 * M, dtype=torch.float16, device=DEV)
+        qw = torch.zeros((M, K // 2), dtype=torch.uint8, device=DEV)
+        fpw = torch.zeros((M, F), dtype=torch.float16, device=DEV)
+        rcs = [lib.quik_asym_quantize_fp6(L.ptr(xt), L.QUIK_F16, M, n_in, L.ptr(colmap), K, F, L.ptr(buf), L.ptr(meta6), L.stream()),
+               lib.quik_asym_quantize_tile8(L.ptr(xt), L.QUIK_F16, M, n_in, L.ptr(colmap), K, F, L.ptr(buf), L.ptr(meta6), L.stream()),
+               lib.quik_sym_quantize_mapped(L.ptr(xt), M, n_in, L.ptr(colmap), K, F, 4, 4.0, 1, L.ptr(buf), L.ptr(meta6), None, L.stream()),
+               lib.quik_fp6_pack_weight(L.ptr(qw), L.ptr(fpw), M, K, F, L.ptr(colmap), L.ptr(buf), L.stream())]
+        torch.cuda.synchronize()
+        assert bool((buf == 0x5A).all()) and bool((meta6 == 0).all())
+        return rcs
+
+    assert c_calls(cm) == [ERR_COLMAP] * 4
+    # ascending int_indices that overlap fp_indices (same counts, but no partition): refused as well, although the
+    # ascending order and the number of distinct outlier columns alone would pass
+    ii_bad = ii2.copy()                              # ascending (from _split)
+    pos = int(np.searchsorted(ii_bad, fi2.max()))    # the integer column just below the largest outlier column ...
+    assert pos > 0
+    ii_bad[pos - 1] = fi2.max()                      # ... is replaced by that outlier column: still ascending
+    assert np.all(np.diff(ii_bad) > 0) and np.intersect1d(ii_bad, fi2).size == 1
+    cm_overlap = asymmetric.build_colmap(_t(ii_bad), _t(fi2), n_in)
+    assert not asymmetric.colmap_streams(cm_overlap, K, F)
+    assert c_calls(cm_overlap) == [ERR_COLMAP] * 4
+    # the library forgets what it knew about an address when a new map is built there
+    assert asymmetric.colmap_streams(cm_ok, K, F)
+    rc = lib.quik_colmap_build(L.ptr(_t(ii)), K, L.ptr(_t(fi)), F, n_in, L.ptr(cm_ok), L.stream())
+    assert rc == 0 and lib.quik_colmap_streaming(L.ptr(cm_ok), n_in, K, F, L.stream()) == 0
+    # one call per layer forward: a descriptor that claims a streaming map for one that is not gets the same refusal
+    desc = L.QuikLayer()
+    import ctypes
+    desc.struct_bytes = ctypes.sizeof(L.QuikLayer)
+    desc.bits, desc.dtype, desc.symmetric = 4, L.QUIK_F16, 0
+    desc.in_features, desc.num_int, desc.num_fp, desc.out_features = n_in, K, F, 64
+    desc.colmap_streams, desc.tiled_min_rows = 1, 1
+    junk = torch.zeros(1 << 20, dtype=torch.uint8, device=DEV)
+    desc.colmap, desc.weights_scales, desc.reduced_w, desc.tiled_weight = L.ptr(cm), L.ptr(junk), L.ptr(junk), L.ptr(junk)
+    nws = lib.quik_layer_workspace_bytes(ctypes.byref(desc), M)
+    ws = torch.zeros(nws, dtype=torch.uint8, device=DEV)
+    out = torch.full((M, 64), 7.0, dtype=torch.float16, device=DEV)
+    rc = lib.quik_layer_forward(ctypes.byref(desc), L.ptr(xt), M, L.ptr(ws), nws, None, 0, L.ptr(out), None, L.stream())
     torch.cuda.synchronize()
-    assert rc == 0 and bool((buf == 0x5A).all()) and bool((meta6 == 0).all())
+    assert rc == ERR_COLMAP and bool((out == 7.0).all())
