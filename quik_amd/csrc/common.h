@@ -122,6 +122,20 @@ __device__ __forceinline__ float wave_min(float v) {
   return fminf(fminf(r0, r1), fminf(r2, r3));
 }
 
+// integer sum over the wave (every lane active), same scheme
+template <int CTRL>
+__device__ __forceinline__ int dpp_move_i(int v) {
+  return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, false);
+}
+__device__ __forceinline__ int wave_sum(int v) {
+  v += dpp_move_i<kDppSwap1>(v);
+  v += dpp_move_i<kDppSwap2>(v);
+  v += dpp_move_i<kDppHalfMirror>(v);
+  v += dpp_move_i<kDppMirror>(v);
+  return __builtin_amdgcn_readlane(v, 0) + __builtin_amdgcn_readlane(v, 16) + __builtin_amdgcn_readlane(v, 32) +
+         __builtin_amdgcn_readlane(v, 48);
+}
+
 // ---- direct global -> LDS copies ---------------------------------------------------------
 // One wave-wide 64 x 16-byte copy global -> LDS: lane i reads 16 bytes at sbase + voff_i and
 // they land at LDS address m0 + 16 i.  sbase (scalar) and m0 are wave-uniform, so advancing K

@@ -451,7 +451,7 @@ __device__ __forceinline__ uint2 group_codes(const uint4 &v, const RowQuant<BF16
 // One row is handled by the TPR threads of one workgroup (a multiple of 64, at most 256; the
 // launches use 256), which walks over rows blockIdx.x, blockIdx.x + gridDim.x, ...
 // SYM: symmetric activations (scale = fp16(max |x| / sym_divisor), one scale per row in meta[row]); fp16 only.
-template <int BITS, bool BF16, int NV, int TPR, bool SYM = false>
+template <int BITS, bool BF16, int NV, int TPR, bool SYM = false, bool PF = false>
 __device__ __forceinline__ void stream_rows(const uint16_t *__restrict__ x, int64_t rows, int64_t cols,
                                             const uint32_t *__restrict__ grp, const uint32_t *__restrict__ dirty,
                                             const uint16_t *__restrict__ dirty_grp, int ndirty,
@@ -473,7 +473,7 @@ __device__ __forceinline__ void stream_rows(const uint16_t *__restrict__ x, int6
   for (int i = 0; i < NV; ++i) g[i] = tid + i * TPR < nvec ? grp[tid + i * TPR] : 0xFFFFFFFFu;
   // row-invariant tables of this lane's first ND dirty groups and outliers, kept in registers so
   // that the per-row loops below wait on no global load
-  constexpr int ND = 256 / TPR;
+  constexpr int ND = TPR >= 256 ? 1 : 256 / TPR;
   uint32_t my_dirty[ND], my_dgrp[ND], my_fpcol[ND];
 #pragma unroll
   for (int k = 0; k < ND; ++k) {
@@ -613,18 +613,19 @@ __device__ __forceinline__ void stream_rows(const uint16_t *__restrict__ x, int6
     mn = wave_min(mn);
     mx = wave_max(mx);
     if constexpr (TPR > 64) {
-      float *r = red + parity * 8;  // two sets: the next row's writes cannot overtake this row's reads
+      constexpr int NW = TPR / 64;
+      float *r = red + parity * 2 * NW;  // two sets: the next row's writes cannot overtake this row's reads
       if ((tid & 63) == 0) {
         r[tid >> 6] = mn;
-        r[4 + (tid >> 6)] = mx;
+        r[NW + (tid >> 6)] = mx;
       }
       __syncthreads();
       mn = r[0];
-      mx = r[4];
+      mx = r[NW];
 #pragma unroll
-      for (int w = 1; w < TPR / 64; ++w) {
+      for (int w = 1; w < NW; ++w) {
         mn = fminf(mn, r[w]);
-        mx = fmaxf(mx, r[4 + w]);
+        mx = fmaxf(mx, r[NW + w]);
       }
     }
 
@@ -690,7 +691,7 @@ __device__ __forceinline__ void stream_rows(const uint16_t *__restrict__ x, int6
     }
   };
 
-  // No software prefetch: the launch makes one workgroup per row (up to the grid limit), several of
+  // Without PF: no software prefetch; the launch makes one workgroup per row (up to the grid limit), several of
   // them are resident per CU, and their phases drift apart, so loads, arithmetic and stores of
   // different rows overlap.
   // Tile-ordered output: a cache line of the operand buffer takes pieces of 4 (heads) or 16 (tails) consecutive rows.
@@ -699,22 +700,56 @@ __device__ __forceinline__ void stream_rows(const uint16_t *__restrict__ x, int6
   const int64_t per_xcd = (rows + 7) >> 3;
   const int64_t items = to8 ? per_xcd * 8 : rows;
   int parity = 0;
-  for (int64_t w = blockIdx.x; w < items; w += gridDim.x) {
-    const int64_t row = to8 ? (w & 7) * per_xcd + (w >> 3) : w;
-    if (row >= rows) continue;
-    parity ^= 1;
-    uint4 cur[NV], dv[ND];
-    uint16_t fpv[ND];
-    load_row(row, cur);
+  auto row_of = [&](int64_t w) -> int64_t {
+    const int64_t r = to8 ? (w & 7) * per_xcd + (w >> 3) : w;
+    return w < items && r < rows ? r : -1;
+  };
+  auto load_all = [&](int64_t row, uint4 (&v)[NV], uint4 (&dvv)[ND], uint16_t (&fv)[ND]) {
+    load_row(row, v);
     const uint4 *xv = reinterpret_cast<const uint4 *>(x + row * cols);
 #pragma unroll
     for (int k = 0; k < ND; ++k) {
-      dv[k] = make_uint4(0, 0, 0, 0);
-      fpv[k] = 0;
-      if (tid + k * TPR < ndirty) dv[k] = xv[my_dgrp[k]];
-      if (tid + k * TPR < num_fp) fpv[k] = x[row * cols + my_fpcol[k]];
+      dvv[k] = make_uint4(0, 0, 0, 0);
+      fv[k] = 0;
+      if (tid + k * TPR < ndirty) dvv[k] = xv[my_dgrp[k]];
+      if (tid + k * TPR < num_fp) fv[k] = x[row * cols + my_fpcol[k]];
     }
-    process(row, cur, dv, fpv, parity);
+  };
+  if constexpr (PF) {
+    // Long rows leave room for two workgroups per CU only (registers), so the launch is persistent (a few rows per
+    // workgroup) and the next row's loads are issued before the current row's arithmetic: the memory pipeline has
+    // work while the workgroup reduces, quantises and stores.
+    uint4 cur[NV], nxt[NV], dv[ND], dvn[ND];
+    uint16_t fpv[ND], fpvn[ND];
+    int64_t w = blockIdx.x;
+    int64_t row = row_of(w);
+    if (row >= 0) load_all(row, cur, dv, fpv);
+    for (; w < items; w += gridDim.x) {
+      const int64_t row2 = row_of(w + gridDim.x);
+      if (row2 >= 0) load_all(row2, nxt, dvn, fpvn);
+      if (row >= 0) {
+        parity ^= 1;
+        process(row, cur, dv, fpv, parity);
+      }
+#pragma unroll
+      for (int i = 0; i < NV; ++i) cur[i] = nxt[i];
+#pragma unroll
+      for (int k = 0; k < ND; ++k) {
+        dv[k] = dvn[k];
+        fpv[k] = fpvn[k];
+      }
+      row = row2;
+    }
+  } else {
+    for (int64_t w = blockIdx.x; w < items; w += gridDim.x) {
+      const int64_t row = row_of(w);
+      if (row < 0) continue;
+      parity ^= 1;
+      uint4 cur[NV], dv[ND];
+      uint16_t fpv[ND];
+      load_all(row, cur, dv, fpv);
+      process(row, cur, dv, fpv, parity);
+    }
   }
 }
 
@@ -732,7 +767,7 @@ __global__ __launch_bounds__(kThreads) void asym_quantize_kernel(
 // Shapes that may stream: the column map's flag (known only on the device) picks the path.
 // Dynamic LDS: the row (gather path) or one byte per code (streaming path), whichever is larger.
 // SYM: symmetric activations; exists on the streaming path only (the host checks the column map's flag first).
-template <typename IdxT, int BITS, bool BF16, int NV, int TPR, bool SYM = false>
+template <typename IdxT, int BITS, bool BF16, int NV, int TPR, bool SYM = false, bool PF = false>
 __global__ __launch_bounds__(TPR) void asym_quantize_stream_kernel(
     const uint16_t *__restrict__ x, int64_t rows, int64_t cols, const IdxT *__restrict__ src_col,
     const IdxT *__restrict__ fp_col, const uint32_t *__restrict__ mask, const uint32_t *__restrict__ grp,
@@ -741,10 +776,10 @@ __global__ __launch_bounds__(TPR) void asym_quantize_stream_kernel(
     uint16_t *__restrict__ fp_x, int vec_out, float sym_divisor) {
   static_assert(sizeof(IdxT) == 2, "streaming needs cols <= 32768");
   extern __shared__ __align__(16) uint16_t row_s[];
-  __shared__ float red[16];
+  __shared__ float red[64];
   if (flags[0] & 1u) {
     uint8_t *codes_s = reinterpret_cast<uint8_t *>(row_s);
-    stream_rows<BITS, BF16, NV, TPR, SYM>(x, rows, cols, grp, dirty, dirty_grp, static_cast<int>(flags[1]),
+    stream_rows<BITS, BF16, NV, TPR, SYM, PF>(x, rows, cols, grp, dirty, dirty_grp, static_cast<int>(flags[1]),
                                           reinterpret_cast<const uint16_t *>(fp_col), num_int, num_fp, dst, meta, fp_x,
                                           codes_s, red, vec_out, sym_divisor);
   } else if constexpr (!SYM) {
@@ -817,17 +852,23 @@ __device__ __forceinline__ uint32_t level_pair_fast(uint32_t w, const RQ &rq) {
 // A workgroup (= wave) walks over rows w, w + grid, ...; up to eight of them share a CU (two per SIMD),
 // so one wave's arithmetic covers the other's transfer and LDS waits.  JT > 0: fragments per lane known at
 // compile time (rows up to 10240 columns); 0: a run-time loop over them.
-template <bool BF16, bool SYM, int JT>
-__global__ __launch_bounds__(64) void quantize_fp6_wave_kernel(
+template <bool BF16, bool SYM, int JT, int W>
+__global__ __launch_bounds__(64 * W) void quantize_fp6_wave_kernel(
     const uint16_t *__restrict__ x, int64_t rows, int cols, const uint32_t *__restrict__ patch,
     const uint16_t *__restrict__ fp_col, const uint32_t *__restrict__ flags, int num_int, int num_fp,
     uint8_t *__restrict__ dst, uint16_t *__restrict__ meta, float sym_divisor) {
   static_assert(!(BF16 && SYM), "symmetric activations are fp16");
-  extern __shared__ __align__(16) uint8_t row_img[];
+  constexpr int kTogether = 2;  // waves that issue their copies at the same time (measured: 1, 2, 4 and all 8)
+  extern __shared__ __align__(16) uint8_t images[];
+  __shared__ int turn_s;
   if (!(flags[0] & 2u)) return;  // no in-place order: nothing to write (the entry points refuse such a map before launching)
-  const int lane = threadIdx.x;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
   const int frags_all = cols >> 5, frags = num_int >> 5, nchunk = num_fp >> 3;
   const int J = JT > 0 ? JT : (frags_all + 63) >> 6;
+  uint8_t *row_img = images + wave * (J * 4096);
+  if (threadIdx.x == 0) turn_s = 0;
+  __syncthreads();
   const int nholes = static_cast<int>(flags[2]);
   const Fp6Layout l6 = fp6_layout(rows, num_int, num_fp);
   const uint32_t lds0 = lds_address(row_img);
@@ -973,6 +1014,11 @@ __global__ __launch_bounds__(64) void quantize_fp6_wave_kernel(
       }
     }
     // ---- pass 2: fragment -> 32 levels -> 24 bytes
+    // (store addresses: the row's part is wave-uniform, the fragment's part is the unit 3072 (f / 2) and its half)
+    const int64_t rb = (row >> 6) * l6.block_bytes;
+    uint8_t *head_row = dst + rb + ((row >> 5) & 1) * 1024 + (row & 31) * 32;
+    uint8_t *tail_row = dst + rb + 2048 + (row & 63) * 8;
+    const uint32_t swap16 = static_cast<uint32_t>((row >> 3) & 1) << 4;
     int sum = 0;
     auto quantise = [&](auto slow_c) {
       constexpr bool SLOW = decltype(slow_c)::value;
@@ -1004,7 +1050,9 @@ __global__ __launch_bounds__(64) void quantize_fp6_wave_kernel(
           for (int i = 0; i < 8; ++i) sum = __builtin_amdgcn_udot4(b[i], 0x01010101u, sum, false);
           uint32_t o[6];
           fp6_pack_fragment(b, o);
-          fp6_store_fragment(dst, l6, row, f, o);
+          const uint32_t unit = static_cast<uint32_t>(f >> 1) * 3072u, h = static_cast<uint32_t>(f & 1);
+          *reinterpret_cast<uint4 *>(head_row + unit + ((h << 4) ^ swap16)) = make_uint4(o[0], o[1], o[2], o[3]);
+          *reinterpret_cast<uint2 *>(tail_row + unit + h * 512u) = make_uint2(o[4], o[5]);
         }
       });
     };
@@ -1013,20 +1061,36 @@ __global__ __launch_bounds__(64) void quantize_fp6_wave_kernel(
     } else {
       quantise(std::false_type{});
     }
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+    sum = wave_sum(sum);
     if (lane == 0) reinterpret_cast<int32_t *>(dst + l6.sums_off)[row] = sum;
   };
 
-  // Workgroup w takes row (w % 8) * rows / 8 + w / 8 (a cache line of the operand buffer takes pieces of 4 (heads) or
-  // 16 (tails) consecutive rows; workgroups are dealt round-robin to the 8 XCDs, so rows that share lines run on
-  // the same XCD at about the same time and meet in its L2), then every gridDim.x-th further item.
-  const int64_t per_xcd = (rows + 7) >> 3, items = per_xcd * 8;
-  auto row_of = [&](int64_t w) { return (w & 7) * per_xcd + (w >> 3); };
-  auto clamped = [&](int64_t r) { return r < rows ? r : rows - 1; };
-  int64_t w = blockIdx.x;
-  if (w >= items) return;
-  issue(clamped(row_of(w)));
+  // Workgroup g takes the rows (g % 8) * rows / 8 + (g / 8) * W + wave (a cache line of the operand buffer takes
+  // pieces of 4 (heads) or 16 (tails) consecutive rows; workgroups are dealt round-robin to the 8 XCDs, so rows that
+  // share lines run on the same XCD at about the same time and meet in its L2), then every gridDim.x-th further group.
+  //
+  // The waves of a workgroup issue their copies kTogether at a time, in the order of a counter in LDS: the memory
+  // system serves a CU's requests about in the order they arrive, so the rows land in that order and a wave does
+  // its arithmetic while the later rows are still in flight.  (With all waves issuing at once the requests
+  // interleave, all rows land together at the end of the transfer, and transfer and arithmetic add up instead of
+  // overlapping.)  Every wave takes every one of its turns, with or without a row, so the counter always advances.
+  const int64_t per_xcd = (rows + 7) >> 3, groups_per_xcd = (per_xcd + W - 1) / W, groups = groups_per_xcd * 8;
+  auto row_of = [&](int64_t g) -> int64_t {
+    const int64_t i = (g >> 3) * W + wave;
+    const int64_t r = (g & 7) * per_xcd + i;
+    return i < per_xcd && r < rows ? r : -1;
+  };
+  volatile int *turn_v = &turn_s;
+  auto take_turn = [&](int t, int64_t row) {
+    const int need = t / kTogether * kTogether;  // all waves of the earlier sets have issued
+    while (__builtin_amdgcn_readfirstlane(*turn_v) < need) __builtin_amdgcn_s_sleep(1);
+    if (row >= 0) issue(row);
+    if (lane == 0) __hip_atomic_fetch_add(&turn_s, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+  };
+  int64_t g = blockIdx.x;
+  if (g >= groups) return;
+  int t = wave;
+  take_turn(t, row_of(g));
   // Row-invariant addresses in registers: this lane's first four patches and its first chunk of 8 outliers.  The
   // loads are unconditional (clamped indices, one 16-byte load for the eight outlier columns) and come after the
   // first row's copies, so they are all in flight together and behind the row, not in front of it.
@@ -1049,13 +1113,14 @@ __global__ __launch_bounds__(64) void quantize_fp6_wave_kernel(
       o_addr[2 * k + 1] = img_of_col(ow[k] >> 16);
     }
   }
-  for (; w < items; w += gridDim.x) {
+  for (; g < groups; g += gridDim.x) {
     __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));  // this row's image has landed
-    const int64_t row = row_of(w);
-    if (row < rows) process(row, row_img);
-    if (w + gridDim.x < items) {
+    const int64_t row = row_of(g);
+    if (row >= 0) process(row, row_img);
+    if (g + gridDim.x < groups) {
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // this row's LDS reads are done before the image is overwritten (a wait only: no hazard)
-      issue(clamped(row_of(w + gridDim.x)));
+      t += W;
+      take_turn(t, row_of(g + gridDim.x));
     }
   }
 }
@@ -1193,12 +1258,13 @@ int grid_for(int64_t work_items, int64_t per_block) {
 
 constexpr int64_t kMaxLdsRowBytes = 128 * 1024;  // of the 160 KB per CU
 
-template <typename IdxT, int BITS, bool BF16, int NV, int TPR, bool SYM = false>
+template <typename IdxT, int BITS, bool BF16, int NV, int TPR, bool SYM = false, bool PF = false>
 int launch_stream(const void *x, int64_t rows, int64_t cols, const uint8_t *cm, const ColmapLayout &l, int64_t num_int,
                   int64_t num_fp, void *dst, void *meta, void *fp_x, hipStream_t st, bool tiled,
                   float sym_divisor = 1.0f) {
-  auto kern = asym_quantize_stream_kernel<IdxT, BITS, BF16, NV, TPR, SYM>;
-  const int64_t lds = align16(cols * 2);  // >= align16(num_int)
+  auto kern = asym_quantize_stream_kernel<IdxT, BITS, BF16, NV, TPR, SYM, PF>;
+  // the row (gather path) or one byte per code (streaming path); a tile-ordered launch only ever streams
+  const int64_t lds = tiled ? align16(num_int) : align16(cols * 2);
   if (lds > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
@@ -1208,7 +1274,8 @@ int launch_stream(const void *x, int64_t rows, int64_t cols, const uint8_t *cm, 
     }
   }
   const int64_t items = tiled ? (rows + 7) / 8 * 8 : rows;
-  const int grid = static_cast<int>(items < (int64_t(1) << 30) ? items : (int64_t(1) << 30));
+  int grid = static_cast<int>(items < (int64_t(1) << 30) ? items : (int64_t(1) << 30));
+  if (PF && grid > 2 * num_cus()) grid = 2 * num_cus();  // persistent: the workgroups that are resident at once
   // tiled: dst is an operand buffer in tile order (6-bit levels for 4 bits, int8 for 8 bits)
   const int vec_out = tiled ? (BITS == 4 ? 2 : 3) : (num_int % 16 == 0 && reinterpret_cast<uintptr_t>(dst) % 16 == 0);
   hipLaunchKernelGGL(kern, dim3(grid), dim3(TPR), static_cast<size_t>(lds), st,
@@ -1251,6 +1318,14 @@ int launch_asym(const void *x, int64_t rows, int64_t cols, const uint8_t *cm, co
     const int64_t groups = cols / 8;
 #define QUIK_STREAM(NV) \
   return launch_stream<IdxT, BITS, BF16, NV, kThreads>(x, rows, cols, cm, l, num_int, num_fp, dst, meta, fp_x, st, tiled)
+    // rows beyond 16384 columns with tile-ordered int8 output (Llama-2-70B down_proj): 180 registers per lane leave
+    // room for two workgroups per CU, so the launch is persistent and prefetches the next row (measured at 2048 x
+    // 28672: 67 -> 61 us inside the forward; at 2048 x 11008, where three workgroups fit, it is slower)
+    if constexpr (BITS == 8) {
+      if (tiled && groups > 2048)
+        return launch_stream<IdxT, BITS, BF16, 16, kThreads, false, true>(x, rows, cols, cm, l, num_int, num_fp, dst, meta,
+                                                                          fp_x, st, tiled);
+    }
     if (groups <= 512) QUIK_STREAM(2);
     if (groups <= 1024) QUIK_STREAM(4);
     if (groups <= 2048) QUIK_STREAM(8);
@@ -1289,12 +1364,10 @@ template <bool BF16, bool SYM>
 int launch_fp6_wave(const void *x, int64_t rows, int64_t cols, const uint8_t *cm, const ColmapLayout &l, int64_t num_int,
                     int64_t num_fp, void *dst, void *meta, hipStream_t st, float sym_divisor = 1.0f) {
   const int J = static_cast<int>((cols / 32 + 63) / 64);
-  const int64_t items = (rows + 7) / 8 * 8;
-  // as many waves per CU as their row images fit (160 KB of LDS), at most 8: two waves per SIMD cover each other's
-  // waits (measured at 2048 x 8192: 12.9 us against 14.0 us for one wave per SIMD with two images each)
-  const int per_cu = 160 / (J * 4) < 8 ? 160 / (J * 4) : 8;
-  auto go = [&](auto kern) {
-    const int lds = J * 4096;  // one row image
+  // one workgroup per CU: as many waves as their row images fit (160 KB of LDS), at most 8 (two per SIMD)
+  const int per_cu = 156 / (J * 4) < 8 ? 156 / (J * 4) : 8;
+  auto go = [&](auto kern, int W) {
+    const int lds = W * J * 4096;  // one row image per wave
     if (lds > 48 * 1024) {
       hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
       if (e != hipSuccess) {
@@ -1302,9 +1375,10 @@ int launch_fp6_wave(const void *x, int64_t rows, int64_t cols, const uint8_t *cm
         return static_cast<int>(QUIK_ERR_LAUNCH);
       }
     }
-    const int64_t resident = int64_t(num_cus()) * per_cu / 8 * 8;
-    const int grid = static_cast<int>(items < resident ? items : resident);
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(64), static_cast<size_t>(lds), st, static_cast<const uint16_t *>(x), rows,
+    const int64_t per_xcd = (rows + 7) / 8, groups = (per_xcd + W - 1) / W * 8;
+    const int64_t resident = int64_t(num_cus()) * (per_cu / W) / 8 * 8;
+    const int grid = static_cast<int>(groups < resident ? groups : resident);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * W), static_cast<size_t>(lds), st, static_cast<const uint16_t *>(x), rows,
                        static_cast<int>(cols), reinterpret_cast<const uint32_t *>(cm + l.off_patch),
                        reinterpret_cast<const uint16_t *>(cm + l.off_fp), reinterpret_cast<const uint32_t *>(cm + l.off_flags),
                        static_cast<int>(num_int), static_cast<int>(num_fp), static_cast<uint8_t *>(dst),
@@ -1312,14 +1386,17 @@ int launch_fp6_wave(const void *x, int64_t rows, int64_t cols, const uint8_t *cm
     return check_launch();
   };
   switch (J) {  // fragments per lane known at compile time: the loops over them unroll
-    case 1: return go(quantize_fp6_wave_kernel<BF16, SYM, 1>);
-    case 2: return go(quantize_fp6_wave_kernel<BF16, SYM, 2>);
-    case 3: return go(quantize_fp6_wave_kernel<BF16, SYM, 3>);
-    case 4: return go(quantize_fp6_wave_kernel<BF16, SYM, 4>);
-    case 5: return go(quantize_fp6_wave_kernel<BF16, SYM, 5>);
+    case 1: return go(quantize_fp6_wave_kernel<BF16, SYM, 1, 8>, 8);
+    case 2: return go(quantize_fp6_wave_kernel<BF16, SYM, 2, 8>, 8);
+    case 3: return go(quantize_fp6_wave_kernel<BF16, SYM, 3, 8>, 8);
+    case 4: return go(quantize_fp6_wave_kernel<BF16, SYM, 4, 8>, 8);
+    case 5: return go(quantize_fp6_wave_kernel<BF16, SYM, 5, 7>, 7);
     default: break;
   }
-  return go(quantize_fp6_wave_kernel<BF16, SYM, 0>);
+  // longer rows: as many waves as fit one CU's LDS, at least one (rows up to 32768 columns: 64 KB per image)
+  if (per_cu >= 4) return go(quantize_fp6_wave_kernel<BF16, SYM, 0, 4>, 4);
+  if (per_cu >= 2) return go(quantize_fp6_wave_kernel<BF16, SYM, 0, 2>, 2);
+  return go(quantize_fp6_wave_kernel<BF16, SYM, 0, 1>, 1);
 }
 }  // namespace
 }  // namespace quik
