@@ -18,6 +18,7 @@ reference (experiments/qlinear.py:21-199), so `llama_replace_with_kernels`
 from __future__ import annotations
 
 import ctypes
+import weakref
 
 import torch
 from torch import Tensor
@@ -52,7 +53,15 @@ class _PerObjectCache(dict):
 
 class SharedQuantizedInput:
     """Quantized activation shared by the layers of one group (q/k/v, gate/up): the first
-    member quantizes, the others reuse, the last one clears (qlinear.py:21-37)."""
+    member quantizes, the others reuse, the last one clears (qlinear.py:21-37).
+
+    The reference shares only the quantized activation and still runs one GEMM per member.  Here the members
+    register with the group when they are built; when the first member of a complete, compatible group is called
+    (same input size, outlier columns, bits, symmetry, dtype, bias or no bias), the group runs ONE quantize and
+    ONE GEMM over the members' weights concatenated along the output dimension, hands the caller its columns of
+    the result and keeps the other members' columns until they are called (they then compute nothing), as the
+    shared quantized activation is kept in the reference.  The per-column arithmetic is the members', so every
+    output has the bits the member alone would give.  `MixedQLinear.fuse_shared_groups = False` switches this off."""
 
     def __init__(self, group_size):
         self.qint_x = None
@@ -62,6 +71,21 @@ class SharedQuantizedInput:
         self.x6 = None  # activation as a tile-ordered operand buffer (codes and outlier values), see MixedQLinear
         self.group_size = group_size
         self.cur_group_elem = 0
+        self._members = []      # weak references, in the order the members were built
+        self._fused = None      # the concatenated layer (built by the first call), or False: this group cannot be fused
+        self._fused_key = None
+        self._outs = None       # column views of the group's result, one per member, until the last member was called
+
+    def __getstate__(self):     # (weak references and device tensors of a forward in flight do not travel)
+        state = dict(self.__dict__)
+        state.update(_members=[], _fused=None, _fused_key=None, _outs=None, qint_x=None, fp_x=None, qscale_x=None,
+                     meta=None, x6=None, cur_group_elem=0)
+        return state
+
+    def register(self, module):
+        self._members = [r for r in self._members if r() is not None and r() is not module]
+        self._members.append(weakref.ref(module))
+        self._fused = None
 
     def finish(self):
         self.cur_group_elem += 1
@@ -71,7 +95,99 @@ class SharedQuantizedInput:
             self.meta = None
             self.fp_x = None
             self.x6 = None
+            self._outs = None
             self.cur_group_elem = 0
+
+    def _members_key(self, mods):
+        return tuple((id(m), m.int_weight.data_ptr(), m.int_weight._version, m.weights_scales.data_ptr(),
+                      m.int_indices._version, m.fp_indices._version, bool(m.six_bit_path), m.six_bit_min_rows,
+                      m.tile8_min_rows) for m in mods)
+
+    def _fused_layer(self):
+        """The members' weights as one MixedQLinear (None when the group is not complete or not compatible).  Built
+        once; afterwards the members' buffers are row slices of the concatenated buffers, so the group holds one
+        copy of the reference's buffers, and the tile-ordered copy exists once, for the whole group."""
+        mods = [r() for r in self._members]
+        if len(mods) != self.group_size or any(m is None for m in mods) or self.group_size < 2:
+            return None
+        if self._fused is not None and self._fused is not False and self._fused_key == self._members_key(mods):
+            return self._fused
+        if self._fused is False and self._fused_key == self._members_key(mods):
+            return None
+        first = mods[0]
+        ok = all(m.fused and not m._row_major_released and m.int_features_num > 0 and m.int_weight.is_cuda and
+                 m.int_weight.device == first.int_weight.device and m.in_features == first.in_features and
+                 m.bits == first.bits and m.symmetric == first.symmetric and m.dtype == first.dtype and
+                 m.fp_features_num == first.fp_features_num and (m.bias is None) == (first.bias is None) and
+                 m.sym_divisor == first.sym_divisor and m.six_bit_path == first.six_bit_path and
+                 m.six_bit_min_rows == first.six_bit_min_rows and m.tile8_min_rows == first.tile8_min_rows
+                 for m in mods)
+        ok = ok and all(torch.equal(m.fp_indices, first.fp_indices) and torch.equal(m.int_indices, first.int_indices)
+                        for m in mods[1:])
+        if not ok:
+            self._fused, self._fused_key = False, self._members_key(mods)
+            return None
+        fused = _concatenate_layers(mods)
+        fused.six_bit_path = first.six_bit_path
+        fused.six_bit_min_rows, fused.tile8_min_rows = first.six_bit_min_rows, first.tile8_min_rows
+        fused.sym_divisor = first.sym_divisor
+        # the members' buffers become row slices (contiguous) of the concatenated ones: no second copy
+        lo = 0
+        for m in mods:
+            hi = lo + m.out_features
+            m.int_weight = fused.int_weight[lo:hi]
+            m.weights_scales = fused.weights_scales[lo:hi]
+            if m.fp_features_num > 0:
+                m.fp_weight = fused.fp_weight[lo:hi]
+            if not m.symmetric:
+                m.reduced_w = fused.reduced_w[:, lo:hi]
+            if m.bias is not None:
+                m.bias = fused.bias[lo:hi]
+            m._w6 = m._w6_key = None      # a member's own tile-ordered copy is not read while the group serves it
+            m._descs.clear()
+            lo = hi
+        self._fused, self._fused_key = fused, self._members_key(mods)
+        self._split = [m.out_features for m in mods]
+        return fused
+
+    def group_forward(self, member, x2):
+        """Output [rows, member.out_features] of `member` for the 2-D input x2 through the fused group, or None when
+        this call is not served that way (the caller then takes the member's own path)."""
+        if self.cur_group_elem == 0:
+            self._outs = None
+            fused = self._fused_layer()
+            if fused is None:
+                return None
+            with device_guard(x2.device):
+                whole = fused._forward_one_call(x2)
+            if whole is None:
+                return None
+            mods = [r() for r in self._members]
+            self._outs = {id(m): o for m, o in zip(mods, whole.split(self._split, dim=-1))}
+        if self._outs is None or id(member) not in self._outs:
+            return None
+        out = self._outs[id(member)]
+        self.finish()
+        return out
+
+
+def _concatenate_layers(layers):
+    """MixedQLinear whose output columns are those of `layers` (same input, outlier columns, bits, symmetry and
+    dtype), one after the other."""
+    first = layers[0]
+    total = sum(m.out_features for m in layers)
+    fused = MixedQLinear(first.in_features, total, None, fp_features_num=first.fp_features_num,
+                         symm=first.symmetric, bits=first.bits, dtype=first.dtype, fused=True, allocate=False)
+    fused.int_weight = torch.cat([m.int_weight for m in layers], dim=0).contiguous()
+    fused.weights_scales = torch.cat([m.weights_scales for m in layers], dim=0).contiguous()
+    fused.int_indices = first.int_indices.clone()
+    fused.fp_indices = first.fp_indices.clone()
+    if first.fp_features_num > 0:
+        fused.fp_weight = torch.cat([m.fp_weight for m in layers], dim=0).contiguous()
+    if not first.symmetric:
+        fused.reduced_w = torch.cat([m.reduced_w for m in layers], dim=1).contiguous()
+    fused.bias = None if first.bias is None else torch.cat([m.bias for m in layers], dim=0).contiguous()
+    return fused
 
 
 class MixedQLinear(torch.nn.Module):
@@ -92,9 +208,11 @@ class MixedQLinear(torch.nn.Module):
 
     six_bit_min_rows = 33    # up to 32 rows the weight-streaming decode kernel on the packed int4 weights is the right one
     tile8_min_rows = 33      # the same switch for 8 bits (the tile-ordered kernel itself takes any row count)
+    fuse_shared_groups = True   # members of a SharedQuantizedInput group run as one quantize + one GEMM (see there)
 
     def __init__(self, in_features, out_features, shared_input=None,
-                 fp_features_num=0, symm=False, bits=4, dtype=torch.float16, fused=True):
+                 fp_features_num=0, symm=False, bits=4, dtype=torch.float16, fused=True, allocate=True):
+        """allocate=False: the buffers are registered empty (the caller assigns them); otherwise as in the reference."""
         super().__init__()
         self.six_bit_path = True
         self._w6 = None
@@ -111,22 +229,24 @@ class MixedQLinear(torch.nn.Module):
         self.dtype = dtype
         self.fused = fused
         self.sym_divisor = 1 << ((bits - 1) - 1)
-        self.register_buffer('weights_scales', torch.zeros((out_features, 1), dtype=dtype))
+        rows = out_features if allocate else 0
+        self.register_buffer('weights_scales', torch.zeros((rows, 1), dtype=dtype))
         if bits == 4:
-            self.register_buffer('int_weight', torch.zeros((out_features, self.int_features_num // 2),
-                                                           dtype=torch.uint8))
+            self.register_buffer('int_weight', torch.zeros((rows, self.int_features_num // 2), dtype=torch.uint8))
         else:
-            self.register_buffer('int_weight', torch.zeros((out_features, self.int_features_num), dtype=torch.int8))
-        self.register_buffer('bias', torch.zeros((out_features,), dtype=dtype))
-        self.register_buffer('int_indices', torch.zeros((self.int_features_num,), dtype=torch.long))
-        self.register_buffer('fp_indices', torch.zeros((fp_features_num,), dtype=torch.long))
+            self.register_buffer('int_weight', torch.zeros((rows, self.int_features_num), dtype=torch.int8))
+        self.register_buffer('bias', torch.zeros((rows,), dtype=dtype))
+        self.register_buffer('int_indices', torch.zeros((self.int_features_num if allocate else 0,), dtype=torch.long))
+        self.register_buffer('fp_indices', torch.zeros((fp_features_num if allocate else 0,), dtype=torch.long))
         if fp_features_num > 0:
-            self.register_buffer('fp_weight', torch.zeros((out_features, fp_features_num), dtype=dtype))
+            self.register_buffer('fp_weight', torch.zeros((rows, fp_features_num), dtype=dtype))
         if not symm:
-            self.register_buffer('reduced_w', torch.zeros((1, out_features), dtype=dtype))
+            self.register_buffer('reduced_w', torch.zeros((1, rows), dtype=dtype))
         self._colmap = None
         self._colmap_key = None
         self._descs = _PerObjectCache()
+        if shared_input is not None and hasattr(shared_input, "register"):
+            shared_input.register(self)
 
     # -- cached column map: rebuilt when the index buffers move or are written in place
     def _column_map(self):
@@ -313,6 +433,11 @@ class MixedQLinear(torch.nn.Module):
                 output = self._forward_one_call(x2)
             if output is not None:
                 return output.reshape(*lead, self.out_features)
+        if self.fused and self.fuse_shared_groups and self.shared_input is not None and \
+                self.shared_input.group_size > 1 and hasattr(self.shared_input, "group_forward"):
+            output = self.shared_input.group_forward(self, x2)    # one quantize + one GEMM for the whole group
+            if output is not None:
+                return output.reshape(*lead, self.out_features)
         shared_input = self.shared_input if self.shared_input is not None else SharedQuantizedInput(1)
         with device_guard(x.device):
             if x2.data_ptr() % 16 == 0 and (not self.symmetric or x2.dtype == torch.float16) \
@@ -441,21 +566,7 @@ class FusedMixedQLinearGroup(torch.nn.Module):
                 raise ValueError("FusedMixedQLinearGroup: members must agree in input size, outlier columns, "
                                  "bits, symmetry, dtype and presence of a bias")
         self.split_sizes = [m.out_features for m in layers]
-        total = sum(self.split_sizes)
-        fused = MixedQLinear(first.in_features, total, None, fp_features_num=first.fp_features_num,
-                             symm=first.symmetric, bits=first.bits, dtype=first.dtype, fused=True)
-        dev = first.int_weight.device
-        fused = fused.to(dev)
-        fused.int_weight = torch.cat([m.int_weight for m in layers], dim=0).contiguous()
-        fused.weights_scales = torch.cat([m.weights_scales for m in layers], dim=0).contiguous()
-        fused.int_indices = first.int_indices.clone()
-        fused.fp_indices = first.fp_indices.clone()
-        if first.fp_features_num > 0:
-            fused.fp_weight = torch.cat([m.fp_weight for m in layers], dim=0).contiguous()
-        if not first.symmetric:
-            fused.reduced_w = torch.cat([m.reduced_w for m in layers], dim=1).contiguous()
-        fused.bias = None if first.bias is None else torch.cat([m.bias for m in layers], dim=0).contiguous()
-        self.fused = fused
+        self.fused = _concatenate_layers(layers)
 
     def forward(self, x):
         return self.fused(x).split(self.split_sizes, dim=-1)

@@ -225,3 +225,103 @@ def test_one_resident_copy_of_the_weights(bits, symm, n_in, F):
         assert err <= 4 * np.abs(w64).max() * 2.0 ** -10
     with pytest.raises(RuntimeError):
         tiled_only.release_tiled_weights()
+
+
+# ------------------------------------------------------------------------------ shared-input groups
+@pytest.mark.parametrize("rows,bits,symm,bias", [(200, 4, False, False), (16, 4, False, True), (72, 4, True, False),
+                                                 (130, 8, False, False), (1, 8, False, False)])
+def test_shared_input_group_is_one_quantize_and_one_gemm(rows, bits, symm, bias, monkeypatch):
+    """Layers wired as the reference wires q/k/v (experiments/llama.py:402-437: one SharedQuantizedInput(3), every
+    member built by from_float with it) run as ONE library call for the whole group; each member's output has the
+    bits the member gives on its own, and equals the oracle's forward within the stated tolerance."""
+    from quik_amd import _lib as L
+    from quik_amd.qlinear import MixedQLinear, SharedQuantizedInput
+    rng = np.random.default_rng(rows + bits)
+    n_in, F = 1024 + 64, 64
+    sizes = [512, 128, 192]                  # q wider than k / v, as with grouped-query attention
+    fi = np.sort(rng.permutation(n_in)[:F]).astype(np.int64)
+    shared = SharedQuantizedInput(len(sizes))
+    members, alone, parts = [], [], []
+    for N in sizes:
+        W, s_w, _ = _layer(rng, N, n_in, F, bits)
+        # the outlier columns of a group are the same for every member (they come from the shared input's statistics)
+        keep = np.ones(n_in, bool)
+        keep[fi] = False
+        lo, hi = (-8, 8) if bits == 4 else (-127, 128)
+        W = np.zeros((N, n_in), np.float16)
+        W[:, keep] = (rng.integers(lo, hi, (N, n_in - F)) * s_w.astype(np.float32)).astype(np.float16)
+        W[:, fi] = (0.02 * rng.standard_normal((N, F))).astype(np.float16)
+        b = (0.1 * rng.standard_normal(N)).astype(np.float16) if bias else None
+        lin = torch.nn.Linear(n_in, N, bias=bias)
+        if bias:
+            lin.bias.data = torch.from_numpy(b)
+        mk = lambda sh: MixedQLinear.from_float(lin, torch.from_numpy(W), torch.from_numpy(s_w), sh,
+                                                torch.from_numpy(fi), symm=symm, bits=bits).to(DEV)
+        members.append(mk(shared))
+        alone.append(mk(None))
+        parts.append((W, s_w, b))
+    x = rng.standard_normal((rows, n_in)).astype(np.float32)
+    x[:, fi] *= 50
+    xt = torch.from_numpy(x.astype(np.float16)).to(DEV)
+
+    lib = L.load()
+    calls = []
+    real = lib.quik_layer_forward
+
+    class Spy:
+        def __getattr__(self, name):
+            if name == "quik_layer_forward":
+                def counted(*a):
+                    calls.append(a[2])
+                    return real(*a)
+                return counted
+            return getattr(lib, name)
+    monkeypatch.setattr(L, "load", lambda: Spy())
+    for rep in range(2):                      # the second pass reuses the fused weights
+        calls.clear()
+        outs = [m(xt) for m in members]       # the call order of the reference's decoder layer: one after the other
+        torch.cuda.synchronize()
+        assert calls == [rows]                # one quantize + one GEMM for the three layers
+        assert shared.cur_group_elem == 0 and shared._outs is None
+    monkeypatch.undo()
+    for m, a, o, (W, s_w, b) in zip(members, alone, outs, parts):
+        assert o.shape == (1, rows, m.out_features)
+        want_bits = a(xt)
+        assert torch.equal(_bits(o), _bits(want_bits))
+        omod = qo.from_float(W, s_w, fi, bits, symm=symm)
+        want, _ = qo.mixed_qlinear_forward(x.astype(np.float16), omod, bits, b, symm=symm)
+        got = o[0].float().cpu().numpy().astype(np.float64)
+        w64 = want.astype(np.float64)
+        assert np.abs(got - w64).max() <= 1e-2 * np.sqrt((w64 ** 2).mean())
+    # the members' buffers are slices of the group's: one copy of the weights, and the state dict is the members' own
+    assert members[1].int_weight.data_ptr() == shared._fused.int_weight[sizes[0]:].data_ptr()
+    for m, a in zip(members, alone):
+        sd_m, sd_a = m.state_dict(), a.state_dict()
+        assert sorted(sd_m) == sorted(sd_a)
+        assert all(torch.equal(sd_m[k], sd_a[k]) for k in sd_m)
+    # switched off: the reference's protocol, one library crossing sequence per member, same bits
+    MixedQLinear.fuse_shared_groups = False
+    try:
+        outs2 = [m(xt) for m in members]
+    finally:
+        MixedQLinear.fuse_shared_groups = True
+    assert all(torch.equal(_bits(o), _bits(o2)) for o, o2 in zip(outs, outs2))
+
+
+def test_shared_input_group_with_different_outlier_columns_is_not_fused():
+    """Members whose outlier columns differ cannot share one GEMM: the group falls back to the reference's protocol
+    (which shares the first member's quantized activation, whatever the later members' columns are)."""
+    from quik_amd.qlinear import MixedQLinear, SharedQuantizedInput
+    rng = np.random.default_rng(5)
+    n_in, F, bits = 512 + 32, 32, 4
+    shared = SharedQuantizedInput(2)
+    mods = []
+    for k in range(2):
+        W, s_w, fi = _layer(rng, 96, n_in, F, bits)
+        lin = torch.nn.Linear(n_in, 96, bias=False)
+        mods.append(MixedQLinear.from_float(lin, torch.from_numpy(W), torch.from_numpy(s_w), shared,
+                                            torch.from_numpy(fi), bits=bits).to(DEV))
+    xt = torch.from_numpy(rng.standard_normal((40, n_in)).astype(np.float16)).to(DEV)
+    outs = [m(xt) for m in mods]
+    assert shared._fused is False and shared.cur_group_elem == 0
+    assert all(torch.isfinite(o).all() for o in outs)
