@@ -530,7 +530,7 @@ def main():
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             step()
-        for _ in range(3):
+        for _ in range(max(20, args.warmup)):   # past the clock transient that follows the idle gap of the capture
             graph.replay()
         torch.cuda.synchronize()
         g0, g1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -627,7 +627,7 @@ def main():
                      if mod.fused and traffic.get("gemm6" if six else "gemm") else None,
                      "avg_ms": round(g_avg, 4), "median_ms": round(g_ms[len(g_ms) // 2], 4),
                      "timed_launches": len(g_ms), "algorithmic_ops": int_ops},
-        "roofline_quantize": {"kernel": ("quantize_fp6_wave_kernel (one wave per token row, 6-bit operand output)" if six and bits == 4
+        "roofline_quantize": {"kernel": ("quantize_fp6_wave_kernel (one wave per token row, eight rows per workgroup, 6-bit operand output)" if six and bits == 4
                                          else "asym_quantize_stream_kernel" + (" (tile-ordered operand output)" if six else "")),
                               "bound": "hbm",
                               "achieved": round(quant_gbps, 1),
