@@ -20,6 +20,8 @@ inline hipStream_t as_stream(void *s) { return reinterpret_cast<hipStream_t>(s);
 // QUIK_ERR_COLMAP when the word is not known yet and `st` is being captured (no synchronisation possible there).
 constexpr uint32_t kColmapStreams = 1u, kColmapInPlace = 2u;
 int colmap_flags(const void *colmap, int64_t cols, int64_t num_int, int64_t num_fp, hipStream_t st, uint32_t *flags);
+// all four flag words of the map (flags, number of dirty groups, number of holes, reserved), same look-up
+int colmap_words(const void *colmap, int64_t cols, int64_t num_int, int64_t num_fp, hipStream_t st, uint32_t (&out)[4]);
 void colmap_forget(const void *colmap);
 // QUIK_OK when the column map has all bits of `need` set, QUIK_ERR_COLMAP when not (or an error of colmap_flags)
 inline int colmap_require(const void *colmap, int64_t cols, int64_t num_int, int64_t num_fp, hipStream_t st,

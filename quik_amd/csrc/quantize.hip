@@ -855,13 +855,14 @@ __device__ __forceinline__ uint32_t level_pair_fast(uint32_t w, const RQ &rq) {
 template <bool BF16, bool SYM, int JT, int W>
 __global__ __launch_bounds__(64 * W) void quantize_fp6_wave_kernel(
     const uint16_t *__restrict__ x, int64_t rows, int cols, const uint32_t *__restrict__ patch,
-    const uint16_t *__restrict__ fp_col, const uint32_t *__restrict__ flags, int num_int, int num_fp,
+    const uint16_t *__restrict__ fp_col, int nholes, int num_int, int num_fp,
     uint8_t *__restrict__ dst, uint16_t *__restrict__ meta, float sym_divisor) {
   static_assert(!(BF16 && SYM), "symmetric activations are fp16");
   constexpr int kTogether = 2;  // waves that issue their copies at the same time (measured: 1, 2, 4 and all 8)
   extern __shared__ __align__(16) uint8_t images[];
   __shared__ int turn_s;
-  if (!(flags[0] & 2u)) return;  // no in-place order: nothing to write (the entry points refuse such a map before launching)
+  // (nholes: the column map's count of holes, which the host knows: the entry points look the map's flag words up
+  // before launching, and refuse a map without the in-place order; the kernel starts without a dependent load)
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
   const int frags_all = cols >> 5, frags = num_int >> 5, nchunk = num_fp >> 3;
@@ -869,7 +870,6 @@ __global__ __launch_bounds__(64 * W) void quantize_fp6_wave_kernel(
   uint8_t *row_img = images + wave * (J * 4096);
   if (threadIdx.x == 0) turn_s = 0;
   __syncthreads();
-  const int nholes = static_cast<int>(flags[2]);
   const Fp6Layout l6 = fp6_layout(rows, num_int, num_fp);
   const uint32_t lds0 = lds_address(row_img);
 
@@ -1051,6 +1051,9 @@ __global__ __launch_bounds__(64 * W) void quantize_fp6_wave_kernel(
           uint32_t o[6];
           fp6_pack_fragment(b, o);
           const uint32_t unit = static_cast<uint32_t>(f >> 1) * 3072u, h = static_cast<uint32_t>(f & 1);
+          // (default cache policy: a 128-byte line of the operand buffer takes pieces of 4 (heads) or 16 (tails) rows,
+          // which meet in the XCD's L2; as streaming stores every piece went to memory on its own and the launch
+          // took 29 us instead of 12)
           *reinterpret_cast<uint4 *>(head_row + unit + ((h << 4) ^ swap16)) = make_uint4(o[0], o[1], o[2], o[3]);
           *reinterpret_cast<uint2 *>(tail_row + unit + h * 512u) = make_uint2(o[4], o[5]);
         }
@@ -1363,6 +1366,10 @@ int launch_asym(const void *x, int64_t rows, int64_t cols, const uint8_t *cm, co
 template <bool BF16, bool SYM>
 int launch_fp6_wave(const void *x, int64_t rows, int64_t cols, const uint8_t *cm, const ColmapLayout &l, int64_t num_int,
                     int64_t num_fp, void *dst, void *meta, hipStream_t st, float sym_divisor = 1.0f) {
+  uint32_t words[4];
+  if (int rc = colmap_words(cm, cols, num_int, num_fp, st, words)) return rc;
+  if ((words[0] & (kColmapStreams | kColmapInPlace)) != (kColmapStreams | kColmapInPlace)) return QUIK_ERR_COLMAP;
+  const int nholes = static_cast<int>(words[2]);
   const int J = static_cast<int>((cols / 32 + 63) / 64);
   // one workgroup per CU: as many waves as their row images fit (160 KB of LDS), at most 8 (two per SIMD)
   const int per_cu = 156 / (J * 4) < 8 ? 156 / (J * 4) : 8;
@@ -1380,7 +1387,7 @@ int launch_fp6_wave(const void *x, int64_t rows, int64_t cols, const uint8_t *cm
     const int grid = static_cast<int>(groups < resident ? groups : resident);
     hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * W), static_cast<size_t>(lds), st, static_cast<const uint16_t *>(x), rows,
                        static_cast<int>(cols), reinterpret_cast<const uint32_t *>(cm + l.off_patch),
-                       reinterpret_cast<const uint16_t *>(cm + l.off_fp), reinterpret_cast<const uint32_t *>(cm + l.off_flags),
+                       reinterpret_cast<const uint16_t *>(cm + l.off_fp), nholes,
                        static_cast<int>(num_int), static_cast<int>(num_fp), static_cast<uint8_t *>(dst),
                        static_cast<uint16_t *>(meta), sym_divisor);
     return check_launch();

@@ -44,7 +44,7 @@ int num_cus() {
 namespace {
 struct ColmapFlags {
   int64_t cols, num_int, num_fp;
-  uint32_t flags;
+  uint32_t words[4];  // the map's four flag words (colmap.h): flags, dirty groups, holes, reserved
 };
 std::mutex g_colmap_mutex;
 std::unordered_map<const void *, ColmapFlags> g_colmap_flags;
@@ -57,12 +57,19 @@ void colmap_forget(const void *colmap) {
 }
 
 int colmap_flags(const void *colmap, int64_t cols, int64_t num_int, int64_t num_fp, hipStream_t st, uint32_t *flags) {
+  uint32_t words[4];
+  if (int rc = colmap_words(colmap, cols, num_int, num_fp, st, words)) return rc;
+  *flags = words[0];
+  return QUIK_OK;
+}
+
+int colmap_words(const void *colmap, int64_t cols, int64_t num_int, int64_t num_fp, hipStream_t st, uint32_t (&out)[4]) {
   {
     std::lock_guard<std::mutex> lock(g_colmap_mutex);
     auto it = g_colmap_flags.find(colmap);
     if (it != g_colmap_flags.end() && it->second.cols == cols && it->second.num_int == num_int &&
         it->second.num_fp == num_fp) {
-      *flags = it->second.flags;
+      for (int i = 0; i < 4; ++i) out[i] = it->second.words[i];
       return QUIK_OK;
     }
   }
@@ -73,8 +80,8 @@ int colmap_flags(const void *colmap, int64_t cols, int64_t num_int, int64_t num_
   }
   if (capture != hipStreamCaptureStatusNone) return QUIK_ERR_COLMAP;
   const ColmapLayout l = colmap_layout(cols, num_int, num_fp);
-  uint32_t word = 0;
-  if (hipMemcpyAsync(&word, static_cast<const uint8_t *>(colmap) + l.off_flags, sizeof(word), hipMemcpyDeviceToHost,
+  uint32_t word[4] = {0, 0, 0, 0};
+  if (hipMemcpyAsync(word, static_cast<const uint8_t *>(colmap) + l.off_flags, sizeof(word), hipMemcpyDeviceToHost,
                      st) != hipSuccess ||
       hipStreamSynchronize(st) != hipSuccess) {
     set_last_hip_error(hipGetLastError());
@@ -83,9 +90,9 @@ int colmap_flags(const void *colmap, int64_t cols, int64_t num_int, int64_t num_
   {
     std::lock_guard<std::mutex> lock(g_colmap_mutex);
     if (g_colmap_flags.size() >= kMaxKnownColmaps) g_colmap_flags.clear();
-    g_colmap_flags[colmap] = ColmapFlags{cols, num_int, num_fp, word};
+    g_colmap_flags[colmap] = ColmapFlags{cols, num_int, num_fp, {word[0], word[1], word[2], word[3]}};
   }
-  *flags = word;
+  for (int i = 0; i < 4; ++i) out[i] = word[i];
   return QUIK_OK;
 }
 

@@ -522,11 +522,20 @@ def test_shared_quantized_input_group():
         omods.append(qo.from_float(W, s_w, fi, bits))
     x = _acts(rng, M, n_in, fi).astype(np.float16)
     xt = _t(x)
-    for i, (m, om) in enumerate(zip(mods, omods)):
-        out = m(xt)[0].float().cpu().numpy()
-        want, _ = qo.mixed_qlinear_forward(x, om, bits)
-        assert np.abs(out - want).max() <= 1e-2 * np.sqrt((want.astype(np.float64) ** 2).mean())
-        assert (shared.qint_x is None) == (i == 2)
+    from quik_amd.qlinear import MixedQLinear
+    # the reference's protocol (the shared quantized activation is held until the last member has run), and the
+    # default here: one quantize + one GEMM for the group, the other members' columns held instead
+    for fuse in (False, True):
+        MixedQLinear.fuse_shared_groups = fuse
+        try:
+            for i, (m, om) in enumerate(zip(mods, omods)):
+                out = m(xt)[0].float().cpu().numpy()
+                want, _ = qo.mixed_qlinear_forward(x, om, bits)
+                assert np.abs(out - want).max() <= 1e-2 * np.sqrt((want.astype(np.float64) ** 2).mean())
+                held = shared._outs if fuse else shared.qint_x
+                assert (held is None) == (i == 2)
+        finally:
+            MixedQLinear.fuse_shared_groups = True
 
 
 @pytest.mark.parametrize("tokens,bits", [(300, 4), (8, 4), (40, 8)])
@@ -1303,17 +1312,30 @@ def test_six_bit_path_shared_input_and_fallbacks():
         single.six_bit_path = False
         singles.append(single)
     xt = _t(_acts(rng, M, n_in, fi).astype(np.float16))
-    for i, (m, s) in enumerate(zip(mods, singles)):
+    from quik_amd.qlinear import MixedQLinear
+    for i, (m, s) in enumerate(zip(mods, singles)):            # the default: one GEMM for the group
         out = m(xt)
-        assert (shared.x6 is None) == (i == 2) and shared.qint_x is None
+        assert (shared._outs is None) == (i == 2) and shared.x6 is None and shared.qint_x is None
         assert torch.equal(out, s(xt))
-    mods[1].six_bit_path = False                               # mixed group: member 1 re-quantizes to int4
+    MixedQLinear.fuse_shared_groups = False                    # member by member, as the reference runs a group
+    try:
+        for i, (m, s) in enumerate(zip(mods, singles)):
+            out = m(xt)
+            assert (shared.x6 is None) == (i == 2) and shared.qint_x is None
+            assert torch.equal(out, s(xt))
+        mods[1].six_bit_path = False                           # mixed group: member 1 re-quantizes to int4
+        for i, (m, s) in enumerate(zip(mods, singles)):
+            assert torch.equal(m(xt), s(xt))
+        assert shared.x6 is None and shared.qint_x is None
+        small = xt[:20].contiguous()                           # decode size: int4 path, weight-streaming kernel
+        assert torch.equal(mods[0](small), singles[0](small))
+        shared.finish(), shared.finish()
+    finally:
+        MixedQLinear.fuse_shared_groups = True
+    # a group whose members disagree about the tile-ordered path is not fused, and still gives the members' bits
     for i, (m, s) in enumerate(zip(mods, singles)):
         assert torch.equal(m(xt), s(xt))
-    assert shared.x6 is None and shared.qint_x is None
-    small = xt[:20].contiguous()                               # decode size: int4 path, weight-streaming kernel
-    assert torch.equal(mods[0](small), singles[0](small))
-    shared.finish(), shared.finish()
+    assert shared._fused is False and shared.x6 is None and shared.qint_x is None
 
 
 def test_tile_ordered_paths_random_shapes():
