@@ -247,7 +247,9 @@ struct Fp6Pipe {
     // Block scales of 2^0.  Written as scale operands 0, 0 the compiler emits the plain v_mfma_f32_32x32x64_f8f6f4,
     // whose scales are 1.0 by definition; with the equivalent E8M0 value 127 spelled out it emits the scaled form,
     // a scale-load instruction in front of every MFMA, which costs an issue slot each (measured on chains of
-    // dependent MFMAs: identical results, 21 % more time).
+    // dependent MFMAs: identical results, 21 % more time).  Were a compiler to keep the scaled form WITH operands 0,
+    // every product would be scaled by 2^-127: the Makefile's check-mfma target reads the mnemonics of the built
+    // object and fails the build on a scaled f8f6f4 MFMA.
     acc[mi][ni] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(w, x, acc[mi][ni], 2, 2, 0, 0, 0, 0);
   }
   template <bool BF16, int I>
