@@ -9,7 +9,8 @@ namespace quik {
 
 // column map layout: [src_col: num_int idx][fp_col: num_fp idx][mask: ceil(cols/32) u32]
 //                    [grp: ceil(cols/8) u32][dirty: min(num_fp, ceil(cols/8)) u32][dirty_grp: same count, u16]
-//                    [kperm: num_int u16][patch: num_fp u32][flags: 4 u32]
+//                    [kperm: num_int u16][patch: num_fp u32]
+//                    [unit: ceil(num_int/16) u16][gather_unit: num_fp u16][gather_cols: num_fp x 16 u16][flags: 4 u32]
 // idx is uint16_t when cols <= 65536, else uint32_t.  Section offsets are 16-byte aligned.
 // A "group" is 8 consecutive source columns (one 16-byte load).  A group without outliers is
 // clean, one with outliers is dirty; dirty groups are numbered in ascending order (slots).
@@ -20,7 +21,14 @@ namespace quik {
 //   flags[0] bit 0: int_indices ascending, the two lists partition the columns and the shape
 //            fits the streaming kernel;  flags[1] = number of dirty groups.
 //   flags[0] bit 1: the in-place order below exists; flags[2] = its number of holes.
-// grp, dirty, dirty_grp, kperm and patch exist only when cols <= kStreamMaxCols.
+//   flags[3] = number of gathered units (below), when the map streams and num_int % 16 == 0.
+// grp, dirty, dirty_grp, kperm, patch, unit, gather_unit and gather_cols exist only when cols <= kStreamMaxCols.
+//
+// Units (int8 operand buffers in tile order): unit u is the 16 integer columns int_indices[16 u .. 16 u + 15], one
+// 16-byte chunk of a row of the buffer.
+//   unit[u]          the first of those columns when the 16 are consecutive source columns, else 0xFFFF
+//   gather_unit[i]   the i-th unit (ascending) whose columns are not consecutive; at most one per outlier column
+//   gather_cols[i]   its 16 source columns
 //
 // In-place order of the integer columns (operand buffers of the 6-bit path).  With num_int and num_fp
 // multiples of 32, the first num_int source columns keep their places: position k holds source column k.
@@ -32,7 +40,8 @@ namespace quik {
 //   [patch: num_fp u32]   hole column | filler column << 16, flags[2] entries
 struct ColmapLayout {
   bool idx16;
-  int64_t off_fp, off_mask, off_grp, off_dirty, off_slot, off_kperm, off_patch, off_flags, bytes;
+  int64_t off_fp, off_mask, off_grp, off_dirty, off_slot, off_kperm, off_patch, off_unit, off_gunit, off_gcols, off_flags,
+      bytes;
 };
 
 __host__ __device__ inline int64_t align16(int64_t v) { return (v + 15) & ~int64_t(15); }
@@ -58,7 +67,10 @@ __host__ __device__ inline ColmapLayout colmap_layout(int64_t cols, int64_t num_
   l.off_slot = l.off_dirty + align16(stream ? max_dirty_groups(cols, num_fp) * 4 : 0);
   l.off_kperm = l.off_slot + align16(stream ? max_dirty_groups(cols, num_fp) * 2 : 0);
   l.off_patch = l.off_kperm + align16(stream ? num_int * 2 : 0);
-  l.off_flags = l.off_patch + align16(stream ? num_fp * 4 : 0);
+  l.off_unit = l.off_patch + align16(stream ? num_fp * 4 : 0);
+  l.off_gunit = l.off_unit + align16(stream ? ((num_int + 15) / 16) * 2 : 0);
+  l.off_gcols = l.off_gunit + align16(stream ? num_fp * 2 : 0);
+  l.off_flags = l.off_gcols + (stream ? num_fp * 32 : 0);
   l.bytes = l.off_flags + 16;
   return l;
 }

@@ -50,6 +50,8 @@ __global__ __launch_bounds__(1024) void colmap_build_kernel(const int64_t *__res
                                                             uint32_t *__restrict__ grp, uint32_t *__restrict__ dirty,
                                                             uint16_t *__restrict__ dirty_grp,
                                                             uint16_t *__restrict__ kperm, uint32_t *__restrict__ patch,
+                                                            uint16_t *__restrict__ unit, uint16_t *__restrict__ gather_unit,
+                                                            uint16_t *__restrict__ gather_cols,
                                                             uint32_t *__restrict__ flags) {
   // single workgroup: the mask is cleared before any bit is set
   __shared__ int ascending;
@@ -154,6 +156,27 @@ __global__ __launch_bounds__(1024) void colmap_build_kernel(const int64_t *__res
           dirty_grp[slot] = static_cast<uint16_t>(g);
         }
       }
+    }
+  }
+  // 16-column units of the tile-ordered int8 operand buffers (colmap.h)
+  if (cols <= kStreamMaxCols && (flags[0] & 1u) && num_int % 16 == 0) {
+    const int64_t units = num_int / 16;
+    for (int64_t u = threadIdx.x; u < units; u += blockDim.x) {
+      const uint32_t c0 = src_col[16 * u], c15 = src_col[16 * u + 15];
+      unit[u] = c15 - c0 == 15u ? static_cast<uint16_t>(c0) : uint16_t(0xFFFF);
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      uint32_t n = 0;
+      for (int64_t u = 0; u < units; ++u) {
+        if (unit[u] != 0xFFFFu) continue;
+        if (n < num_fp) {  // (always: an outlier column lies inside the span of at most one unit)
+          gather_unit[n] = static_cast<uint16_t>(u);
+          for (int t = 0; t < 16; ++t) gather_cols[16 * n + t] = static_cast<uint16_t>(src_col[16 * u + t]);
+        }
+        ++n;
+      }
+      flags[3] = n;
     }
   }
 }
@@ -468,25 +491,35 @@ __device__ __forceinline__ void stream_rows(const uint16_t *__restrict__ x, int6
   const int tid = threadIdx.x;
   const int nvec = static_cast<int>(cols >> 3);
   const float inf = __builtin_inff();
+  // Row-invariant tables in registers.  Every load is unconditional, from an address that always exists (lanes
+  // without an entry read the first words of grp): behind a condition each load sits in a branch of its own with
+  // its own wait, and the kernel starts with one round trip to the L2 after the other.
   uint32_t g[NV];
 #pragma unroll
-  for (int i = 0; i < NV; ++i) g[i] = tid + i * TPR < nvec ? grp[tid + i * TPR] : 0xFFFFFFFFu;
-  // row-invariant tables of this lane's first ND dirty groups and outliers, kept in registers so
-  // that the per-row loops below wait on no global load
+  for (int i = 0; i < NV; ++i) g[i] = grp[tid + i * TPR < nvec ? tid + i * TPR : 0];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) g[i] = tid + i * TPR < nvec ? g[i] : 0xFFFFFFFFu;
+  // this lane's first ND dirty groups and outliers, so that the per-row loops below wait on no global load
   constexpr int ND = TPR >= 256 ? 1 : 256 / TPR;
   uint32_t my_dirty[ND], my_dgrp[ND], my_fpcol[ND];
+  const uint16_t *spare16 = reinterpret_cast<const uint16_t *>(grp);
 #pragma unroll
   for (int k = 0; k < ND; ++k) {
-    my_dirty[k] = tid + k * TPR < ndirty ? dirty[tid + k * TPR] : 0u;
-    my_dgrp[k] = tid + k * TPR < ndirty ? dirty_grp[tid + k * TPR] : 0u;
-    my_fpcol[k] = tid + k * TPR < num_fp ? fp_col[tid + k * TPR] : 0u;
+    const bool has_d = tid + k * TPR < ndirty, has_f = tid + k * TPR < num_fp;
+    my_dirty[k] = *(has_d ? dirty + tid + k * TPR : grp);
+    my_dgrp[k] = *(has_d ? dirty_grp + tid + k * TPR : spare16);
+    my_fpcol[k] = *(has_f ? fp_col + tid + k * TPR : spare16);
+  }
+#pragma unroll
+  for (int k = 0; k < ND; ++k) {
+    if (!(tid + k * TPR < ndirty)) my_dirty[k] = my_dgrp[k] = 0u;
+    if (!(tid + k * TPR < num_fp)) my_fpcol[k] = 0u;
   }
 
   auto load_row = [&](int64_t row, uint4 (&v)[NV]) {
     const uint4 *xv = reinterpret_cast<const uint4 *>(x + row * cols);
 #pragma unroll
-    for (int i = 0; i < NV; ++i)
-      if (tid + i * TPR < nvec) v[i] = xv[tid + i * TPR];
+    for (int i = 0; i < NV; ++i) v[i] = xv[tid + i * TPR < nvec ? tid + i * TPR : nvec - 1];  // (past the end: any group; its g[i] says "not clean")
   };
 
   // min/max of one dirty group.  fp16: the outlier halves are overwritten with 0xFFFF, a quiet NaN,
@@ -807,6 +840,322 @@ __device__ __forceinline__ uint32_t pk_max_f16(uint32_t a, uint32_t b) {
   return r;
 }
 
+// The IEEE bit of the MODE register makes v_pk_min_f16 / v_pk_max_f16 answer a SIGNALLING NaN operand with a quiet
+// NaN instead of the other operand, which would then be lost from a running minimum.  Kernels that use the two
+// helpers above on raw input clear the bit for themselves: every NaN is skipped alike, as __hmin / __hmax and fminf
+// skip it.  (Nothing else in these kernels depends on the bit: it only selects how signalling NaNs are treated.)
+__device__ __forceinline__ void treat_all_nans_alike() {
+  asm volatile("s_setreg_imm32_b32 hwreg(HW_REG_MODE, 9, 1), 0");
+}
+
+// ---------------------------------------------------------------------------------------
+// Rows of more than 8192 columns (the down_proj inputs) -> int8 operand buffer in tile order, fp16 input.
+//
+// One workgroup of eight waves per CU (two where two rings fit the LDS) walks over its rows; a row is copied global -> LDS with direct copies (no
+// registers, so two rows are in flight while a third is worked on) into a ring of two slots.  Per row:
+//   wait for this wave's copies of the row, barrier (the row is in LDS)
+//   every lane reads its NV groups of 8 columns (and, lanes 0 .. ndirty-1, one group that holds outlier columns;
+//   lanes 0 .. num_fp-1 one outlier value, which goes straight to the staging area); barrier (the slot is free)
+//   the copies of the row after the next are issued into the slot
+//   min / max, barrier, scale and zero
+//   8 codes per group -> staging area in SOURCE order (one byte per column, 8 aligned bytes per group; the bytes
+//   at outlier columns mean nothing), barrier
+//   staging area -> operand buffer in 16-byte units: a unit takes 16 consecutive integer columns, which are 16
+//   consecutive staged bytes from an offset that depends on the unit only (the outlier columns in front of it) unless
+//   outlier columns lie between them; lanes 0 .. (such units) - 1 gather one of those byte by byte.  The outlier
+//   values follow the codes and leave as 16-byte units as well.
+// Squeezing the outlier columns out on the way OUT of the staging area keeps every LDS access aligned: 8-byte
+// writes at byte offsets that are not multiples of 8 (the compacted position of a group) cost about twice the
+// time of aligned ones here, and were half of this kernel's time per row.
+// The arithmetic of a row takes less time than its bytes need, so the copies never wait for it; with registers as
+// the prefetch target (asym_quantize_stream_kernel's persistent form) two workgroups of four waves fit a CU, a wave
+// stalls in the issue of 16 loads per lane while the memory queue is full, and transfer and arithmetic add up.
+// Groups past the row's end read 16 bytes of NaN kept behind the slot (min / max skip them).
+constexpr int kRingThreads = 512;
+
+// LDS bytes of the ring kernel (host and device agree through these functions)
+__host__ __device__ inline int64_t ring_groups_per_lane(int64_t cols) { return (cols / 8 + kRingThreads - 1) / kRingThreads; }
+__host__ __device__ inline int64_t ring_slot_bytes(int64_t cols) { return ((cols * 2 + 1023) / 1024) * 1024 + 16; }
+__host__ __device__ inline int64_t ring_lds_bytes(int64_t cols, int64_t num_fp) {
+  return 2 * ring_slot_bytes(cols) + ring_groups_per_lane(cols) * kRingThreads * 8 + 2 * num_fp + 32 +
+         4 * (kRingThreads / 64) * sizeof(float);
+}
+
+// codes of the two halves of w in bytes 0 and 2 (int8: code = level - 128 mod 256), rows on the fast path
+__device__ __forceinline__ uint32_t ring_code_pair(uint32_t w, h2 zero2, float rcp, uint32_t maxq2) {
+  const uint32_t d = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, w) - zero2);
+  uint32_t tb;
+  asm("v_fma_mixlo_f16 %0, %1, %2, 0 op_sel_hi:[1,0,0]\n\t"
+      "v_fma_mixhi_f16 %0, %1, %2, 0 op_sel:[1,0,0] op_sel_hi:[1,0,0]"
+      : "=&v"(tb)
+      : "v"(d), "v"(rcp));
+  tb = pk_min_f16(pk_max_f16(tb, 0u), maxq2);  // NaN -> 0
+  constexpr _Float16 magic = static_cast<_Float16>(1024 + 128);
+  return __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, tb) + h2{magic, magic});
+}
+
+template <int NV>
+__global__ __launch_bounds__(kRingThreads) void quantize_tile8_ring_kernel(
+    const uint16_t *__restrict__ x, int64_t rows, int64_t cols, const uint16_t *__restrict__ fp_col,
+    const uint32_t *__restrict__ grp, const uint32_t *__restrict__ dirty, const uint16_t *__restrict__ dirty_grp,
+    const uint16_t *__restrict__ unit, const uint16_t *__restrict__ gather_unit,
+    const uint16_t *__restrict__ gather_cols, int ndirty, int ngather, int64_t num_int, int64_t num_fp,
+    uint8_t *__restrict__ dst, uint16_t *__restrict__ meta) {
+  constexpr int T = kRingThreads, NW = T / 64;
+  constexpr int NU = NV / 2 + 1;  // 16-byte units per lane: (codes + outlier values) / 16 / T, at most 512 outliers
+  extern __shared__ __align__(16) uint8_t ring_s[];
+  treat_all_nans_alike();
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int nvec = static_cast<int>(cols >> 3);
+  const uint32_t row_bytes = static_cast<uint32_t>(cols) * 2u;
+  const uint32_t pieces = (row_bytes + 1023u) >> 10;  // direct copies move 1 KB each
+  const uint32_t nan_off = pieces << 10;              // inside a slot: 16 bytes of NaN behind the row
+  const uint32_t slot_stride = nan_off + 16u;
+  // LDS: slot 0 | slot 1 | codes in source order (8 NV T bytes) | outlier values | 32 spare bytes (the units' second
+  // 16-byte read may start there) | reduction slots
+  uint8_t *codes_s = ring_s + 2 * slot_stride;
+  const uint32_t fp_off = NV * T * 8;
+  float *red_s = reinterpret_cast<float *>(codes_s + fp_off + 2 * num_fp + 32);  // [2][2 NW]
+  const Tile8Layout l8 = tile8_layout(rows, num_int, num_fp);
+
+  // rows of this workgroup: workgroups are dealt round-robin to the 8 XCDs and the four rows that share the cache
+  // lines of the operand buffer should meet in one L2, so XCD k takes the k-th eighth of the rows
+  const int64_t per_xcd = (rows + 7) >> 3, stride = gridDim.x >> 3;
+  auto row_at = [&](int64_t i) -> int64_t {
+    const int64_t idx = (blockIdx.x >> 3) + i * stride;
+    const int64_t r = (blockIdx.x & 7) * per_xcd + idx;
+    return idx < per_xcd && r < rows ? r : -1;
+  };
+  const uint32_t ring_lds = lds_address(ring_s);
+  // copy k of this wave for a row (every wave issues NV copies per row, the count the waits below rely on: a piece
+  // past the last is the last once more)
+  auto issue_one = [&](int64_t row, int slot, int k) {
+    const uint8_t *src = reinterpret_cast<const uint8_t *>(x + row * cols);
+    const uint32_t base = ring_lds + static_cast<uint32_t>(slot) * slot_stride;
+    uint32_t piece = static_cast<uint32_t>(wave + NW * k);
+    piece = piece < pieces ? piece : pieces - 1u;
+    uint32_t off = (piece << 10) + static_cast<uint32_t>(lane) * 16u;
+    off = off < row_bytes - 16u ? off : row_bytes - 16u;  // lanes past the row's end repeat its last 16 bytes
+    dma_load16(src, off, base + (piece << 10));
+  };
+  auto issue = [&](int64_t row, int slot) {
+#pragma unroll
+    for (int k = 0; k < NV; ++k) issue_one(row, slot, k);
+  };
+
+  int64_t row = row_at(0);
+  if (row < 0) return;
+  issue(row, 0);
+
+  // ---- row-invariant tables of this lane, in registers
+  // groups: where to read (the NaN block for groups past the row's end) and whether min / max take the group as it
+  // is (a group with outlier columns is taken by one of the lanes 0 .. ndirty-1 instead, with those columns masked)
+  // (every load is unconditional, from a clamped index: behind a condition each would sit in a branch of its own
+  // with its own wait, one round trip to the L2 after the other)
+  uint32_t gsrc[NV], keep[NV];
+  uint32_t info[NV];
+#pragma unroll
+  for (int k = 0; k < NV; ++k) {
+    const int gi = tid + k * T;
+    info[k] = grp[gi < nvec ? gi : nvec - 1];
+  }
+  const bool has_dirty = tid < ndirty, has_fp = tid < num_fp;
+  // (lanes without an entry read the first words of grp, which always exist: the other tables may be empty)
+  const uint16_t *spare = reinterpret_cast<const uint16_t *>(grp);
+  const uint32_t d_info = *(has_dirty ? dirty + tid : grp);
+  const uint32_t d_grp = *(has_dirty ? dirty_grp + tid : spare);
+  const uint32_t f_col = *(has_fp ? fp_col + tid : spare);
+  // units (colmap.h): consecutive columns are 16 consecutive staged bytes from the unit's first column on ("plain");
+  // the others are gathered byte by byte, one unit per lane of the first `ngather` lanes
+  const int nu_int = static_cast<int>(num_int >> 4), nu = nu_int + static_cast<int>(num_fp >> 3);
+  uint32_t ubase[NU], ushift[NU];  // 16-byte-aligned offset into the staging area, byte shift; 0xFFFFFFFF: not plain
+  uint32_t ucol[NU];
+#pragma unroll
+  for (int j = 0; j < NU; ++j) {
+    const int u = tid + j * T;
+    ucol[j] = unit[u < nu_int ? u : nu_int - 1];  // (num_int >= 64: at least four units)
+  }
+  const bool has_gather = tid < ngather;
+  uint32_t goff[8];  // staged byte offsets (= columns) of the 16 codes of this lane's gathered unit, two per register
+  const int gunit = *(has_gather ? gather_unit + tid : spare);
+  {
+    const uint4 *c = reinterpret_cast<const uint4 *>(has_gather ? gather_cols + 16 * tid : spare);
+    const uint4 a = c[0], b = c[1];
+    goff[0] = a.x, goff[1] = a.y, goff[2] = a.z, goff[3] = a.w;
+    goff[4] = b.x, goff[5] = b.y, goff[6] = b.z, goff[7] = b.w;
+  }
+#pragma unroll
+  for (int k = 0; k < NV; ++k) {
+    const int gi = tid + k * T;
+    gsrc[k] = gi < nvec ? static_cast<uint32_t>(gi) * 16u : nan_off;
+    keep[k] = gi >= nvec || (info[k] & 0xFFu) == 0u ? 0xFFFFFFFFu : 0u;
+  }
+  const uint32_t d_mask = has_dirty ? d_info & 0xFFu : 0xFFu;
+  const uint32_t d_src = has_dirty ? d_grp * 16u : nan_off;
+  const uint32_t f_src = has_fp ? f_col * 2u : 0u;
+#pragma unroll
+  for (int j = 0; j < NU; ++j) {
+    const int u = tid + j * T;
+    uint32_t off = 0xFFFFFFFFu;
+    if (u < nu_int) {
+      if (ucol[j] != 0xFFFFu) off = ucol[j];
+    } else if (u < nu) {
+      off = fp_off + static_cast<uint32_t>(u - nu_int) * 16u;
+    }
+    ubase[j] = off == 0xFFFFFFFFu ? off : off & ~15u;
+    ushift[j] = off & 15u;
+  }
+  if (tid < 4) {
+    reinterpret_cast<uint32_t *>(ring_s + nan_off)[tid] = 0xFFFFFFFFu;
+    reinterpret_cast<uint32_t *>(ring_s + slot_stride + nan_off)[tid] = 0xFFFFFFFFu;
+  }
+  // the tables are complete here (this also waits for the first row), not at their first use inside the loop,
+  // where a wait for them would wait for the copies in flight as well
+#pragma unroll
+  for (int k = 0; k < NV; ++k) asm volatile("" ::"v"(gsrc[k]), "v"(keep[k]));
+#pragma unroll
+  for (int j = 0; j < NU; ++j) asm volatile("" ::"v"(ubase[j]), "v"(ushift[j]));
+#pragma unroll
+  for (int j = 0; j < 8; ++j) asm volatile("" ::"v"(goff[j]));
+  asm volatile("" ::"v"(d_mask), "v"(d_src), "v"(f_src), "v"(gunit));
+  {
+    const int64_t r1 = row_at(1);
+    if (r1 >= 0) issue(r1, 1);
+  }
+
+  const uint32_t maxq2 = 0x5BF85BF8u;  // 255.0 in both halves
+  for (int64_t i = 0; row >= 0; ++i) {
+    const int slot = static_cast<int>(i & 1);
+    const int64_t row1 = row_at(i + 1), row2 = row_at(i + 2);
+    // This wave's copies of the row have landed.  Memory operations complete in the order of their issue; the NV
+    // newest at this point are stores of the last row and, before them, copies of the next row, so "at most NV
+    // outstanding" covers the NV copies of this row, which are older than all of those.
+    if (row1 >= 0) {
+      __builtin_amdgcn_s_waitcnt(vmcnt_imm(NV));
+    } else {
+      __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+    }
+    __syncthreads();
+    const uint8_t *slot_s = ring_s + static_cast<uint32_t>(slot) * slot_stride;
+    uint4 v[NV];
+#pragma unroll
+    for (int k = 0; k < NV; ++k) v[k] = *reinterpret_cast<const uint4 *>(slot_s + gsrc[k]);
+    const uint4 dv = *reinterpret_cast<const uint4 *>(slot_s + d_src);
+    const uint16_t fpv = *reinterpret_cast<const uint16_t *>(slot_s + f_src);
+    // (the staging area is free: every wave has finished the last row's stores before the barrier above)
+    if (has_fp) reinterpret_cast<uint16_t *>(codes_s + fp_off)[tid] = fpv;
+    __syncthreads();
+
+    // ---- min / max; the copies of the row after the next go out between the groups (the address unit takes a
+    // copy every 16 cycles: issued in one run, the eight waves would queue behind each other for half a microsecond)
+    uint32_t pmn_b = 0x7C007C00u, pmx_b = 0xFC00FC00u;  // +inf / -inf in both halves
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+      if (row2 >= 0) issue_one(row2, slot, k);
+      const uint32_t lo = pk_min_f16(pk_min_f16(v[k].x, v[k].y), pk_min_f16(v[k].z, v[k].w));
+      const uint32_t hi = pk_max_f16(pk_max_f16(v[k].x, v[k].y), pk_max_f16(v[k].z, v[k].w));
+      pmn_b = pk_min_f16(pmn_b, (lo & keep[k]) | (0x7C007C00u & ~keep[k]));
+      pmx_b = pk_max_f16(pmx_b, (hi & keep[k]) | (0xFC00FC00u & ~keep[k]));
+    }
+    if (has_dirty) {
+      // outlier halves become 0xFFFF, a quiet NaN, which min / max skip
+      const uint32_t w[4] = {dv.x, dv.y, dv.z, dv.w};
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const uint32_t lo = static_cast<uint32_t>(__builtin_amdgcn_sbfe(static_cast<int>(d_mask), 2 * k, 1));
+        const uint32_t hi = static_cast<uint32_t>(__builtin_amdgcn_sbfe(static_cast<int>(d_mask), 2 * k + 1, 1));
+        const uint32_t m = w[k] | __builtin_amdgcn_perm(hi, lo, 0x07060100u);
+        pmn_b = pk_min_f16(pmn_b, m);
+        pmx_b = pk_max_f16(pmx_b, m);
+      }
+    }
+    const h2 pmn = __builtin_bit_cast(h2, pmn_b), pmx = __builtin_bit_cast(h2, pmx_b);
+    float mn = fminf(static_cast<float>(pmn.x), static_cast<float>(pmn.y));
+    float mx = fmaxf(static_cast<float>(pmx.x), static_cast<float>(pmx.y));
+    mn = wave_min(mn);
+    mx = wave_max(mx);
+    float *r = red_s + slot * 2 * NW;  // two sets: the next row's writes cannot overtake this row's reads
+    if (lane == 0) {
+      r[wave] = mn;
+      r[NW + wave] = mx;
+    }
+    __syncthreads();
+    mn = r[0];
+    mx = r[NW];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) {
+      mn = fminf(mn, r[w]);
+      mx = fmaxf(mx, r[NW + w]);
+    }
+    RowQuant<false> rq;
+    rq.init(mn, mx, 8);
+    if (tid == 0) {
+      meta[2 * row] = rq.scale_bits;
+      meta[2 * row + 1] = rq.zero_bits;
+    }
+
+    // ---- codes -> staging area, source order
+    uint2 *stage8 = reinterpret_cast<uint2 *>(codes_s) + tid;
+    if (__builtin_amdgcn_readfirstlane(rq.slow ? 1 : 0)) {
+#pragma unroll
+      for (int k = 0; k < NV; ++k) stage8[k * T] = group_codes<8, false, true>(v[k], rq);
+    } else {
+      const _Float16 zh = static_cast<_Float16>(rq.zero);
+      const h2 zero2 = h2{zh, zh};
+#pragma unroll
+      for (int k = 0; k < NV; ++k) {
+        const uint32_t p0 = ring_code_pair(v[k].x, zero2, rq.rcp, maxq2), p1 = ring_code_pair(v[k].y, zero2, rq.rcp, maxq2);
+        const uint32_t p2 = ring_code_pair(v[k].z, zero2, rq.rcp, maxq2), p3 = ring_code_pair(v[k].w, zero2, rq.rcp, maxq2);
+        stage8[k * T] = make_uint2(__builtin_amdgcn_perm(p1, p0, 0x06040200u), __builtin_amdgcn_perm(p3, p2, 0x06040200u));
+      }
+    }
+    __syncthreads();
+
+    // ---- staging area -> operand buffer, 16 bytes per lane and unit
+    // chunk (step, h) of the row is at + 2048 step + 16 (h ^ bit 3 of the row) from here (tile8_offset)
+    uint8_t *drow = dst + (row >> 6) * l8.block_bytes + ((row >> 5) & 1) * 1024 + (row & 31) * 32;
+    const uint32_t swap16 = static_cast<uint32_t>((row >> 3) & 1) << 4;
+    auto unit_at = [&](int u) -> uint4 * {
+      return reinterpret_cast<uint4 *>(drow + ((static_cast<uint32_t>(u >> 1) << 11) | ((static_cast<uint32_t>(u & 1) << 4) ^ swap16)));
+    };
+#pragma unroll
+    for (int j = 0; j < NU; ++j) {
+      if (ubase[j] != 0xFFFFFFFFu) {
+        // 16 bytes from byte offset ubase + ushift: two aligned 16-byte reads, then a shift by whole words (two
+        // levels of selects) and by bytes
+        const uint4 a = *reinterpret_cast<const uint4 *>(codes_s + ubase[j]);
+        const uint4 b = *reinterpret_cast<const uint4 *>(codes_s + ubase[j] + 16);
+        uint32_t w[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+        // (selects written as bit masks: as conditional moves between array elements the compiler turns them into
+        // one dynamically indexed array in scratch memory, whose loads would wait for the copies in flight)
+        const uint32_t by2 = 0u - ((ushift[j] >> 3) & 1u), by1 = 0u - ((ushift[j] >> 2) & 1u);
+#pragma unroll
+        for (int t = 0; t < 6; ++t) w[t] = (w[t + 2] & by2) | (w[t] & ~by2);
+#pragma unroll
+        for (int t = 0; t < 5; ++t) w[t] = (w[t + 1] & by1) | (w[t] & ~by1);
+        uint4 c;
+        c.x = __builtin_amdgcn_alignbyte(w[1], w[0], ushift[j]);
+        c.y = __builtin_amdgcn_alignbyte(w[2], w[1], ushift[j]);
+        c.z = __builtin_amdgcn_alignbyte(w[3], w[2], ushift[j]);
+        c.w = __builtin_amdgcn_alignbyte(w[4], w[3], ushift[j]);
+        *unit_at(tid + j * T) = c;
+      }
+    }
+    if (has_gather) {
+      uint32_t c[4];
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const uint32_t b0 = codes_s[goff[2 * t] & 0xFFFFu], b1 = codes_s[goff[2 * t] >> 16];
+        const uint32_t b2 = codes_s[goff[2 * t + 1] & 0xFFFFu], b3 = codes_s[goff[2 * t + 1] >> 16];
+        c[t] = b0 | (b1 << 8) | (b2 << 16) | (b3 << 24);
+      }
+      *unit_at(gunit) = make_uint4(c[0], c[1], c[2], c[3]);
+    }
+    row = row1;
+  }
+}
+
 // 4-bit LEVELS (code + 8, 0 .. 15) of the two fp16 halves of w in bytes 0 and 2 of the result, for rows on the fast
 // path (finite range, scale >= 1e-6; RowQuant::slow == false); same levels as code_pair gives.
 //   asymmetric: d = fp16(x - zero); t = fp16(f32(d) * rcp); t = max(t, 0) (a NaN element becomes 0, as the
@@ -861,6 +1210,7 @@ __global__ __launch_bounds__(64 * W) void quantize_fp6_wave_kernel(
   constexpr int kTogether = 2;  // waves that issue their copies at the same time (measured: 1, 2, 4 and all 8)
   extern __shared__ __align__(16) uint8_t images[];
   __shared__ int turn_s;
+  if constexpr (!BF16 && !SYM) treat_all_nans_alike();  // pass 1 uses pk_min_f16 / pk_max_f16 on the raw row
   // (nholes: the column map's count of holes, which the host knows: the entry points look the map's flag words up
   // before launching, and refuse a map without the in-place order; the kernel starts without a dependent load)
   const int lane = threadIdx.x & 63;
@@ -1309,9 +1659,62 @@ int launch_sym_stream(const void *x, int64_t rows, int64_t cols, const uint8_t *
 #undef QUIK_SYM_STREAM
 }
 
+// Long fp16 rows -> int8 operand buffer through the LDS ring (quantize_tile8_ring_kernel).  `ndirty`: groups of 8
+// columns that hold outlier columns, from the host's copy of the column map's flag words.
+constexpr int64_t kLdsPerCu = 160 * 1024;
+// rows of more than 8192 columns: measured against the streaming kernel at 2048 rows, kernel time from a cold
+// cache: 8192 columns 17.4 against 16.8 us, 11008 19.9 against 20.9, 13824 23.7 against 26.3, 28672 41.6 against 51.0
+constexpr int64_t kRingMinGroups = 2 * kRingThreads + 1;
+bool ring_fits(int64_t cols, int64_t num_int, int64_t num_fp, int64_t ndirty) {
+  const int64_t groups = cols / 8;
+  return groups >= kRingMinGroups && groups <= 8 * kRingThreads && ndirty >= 0 && ndirty <= kRingThreads &&
+         num_fp <= kRingThreads && num_int % 16 == 0 && ring_lds_bytes(cols, num_fp) <= kLdsPerCu;
+}
+template <int NV>
+int launch_tile8_ring_nv(const void *x, int64_t rows, int64_t cols, const uint8_t *cm, const ColmapLayout &l,
+                         int64_t num_int, int64_t num_fp, int ndirty, int ngather, void *dst, void *meta,
+                         hipStream_t st) {
+  auto kern = quantize_tile8_ring_kernel<NV>;
+  const int64_t lds = ring_lds_bytes(cols, num_fp);
+  if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+      e != hipSuccess) {
+    set_last_hip_error(e);
+    return QUIK_ERR_LAUNCH;
+  }
+  const int64_t per_xcd = (rows + 7) / 8;
+  // one workgroup per CU when the ring takes most of its LDS, two when two fit; a multiple of the XCDs
+  int64_t grid = num_cus() / 8 * 8 * (2 * lds + 1024 <= kLdsPerCu ? 2 : 1);
+  if (grid < 8) grid = 8;
+  if (grid > per_xcd * 8) grid = per_xcd * 8;
+  hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(grid)), dim3(kRingThreads), static_cast<size_t>(lds), st,
+                     static_cast<const uint16_t *>(x), rows, cols, reinterpret_cast<const uint16_t *>(cm + l.off_fp),
+                     reinterpret_cast<const uint32_t *>(cm + l.off_grp),
+                     reinterpret_cast<const uint32_t *>(cm + l.off_dirty),
+                     reinterpret_cast<const uint16_t *>(cm + l.off_slot),
+                     reinterpret_cast<const uint16_t *>(cm + l.off_unit),
+                     reinterpret_cast<const uint16_t *>(cm + l.off_gunit),
+                     reinterpret_cast<const uint16_t *>(cm + l.off_gcols), ndirty, ngather, num_int, num_fp,
+                     static_cast<uint8_t *>(dst), static_cast<uint16_t *>(meta));
+  return check_launch();
+}
+int launch_tile8_ring(const void *x, int64_t rows, int64_t cols, const uint8_t *cm, const ColmapLayout &l,
+                      int64_t num_int, int64_t num_fp, int ndirty, int ngather, void *dst, void *meta,
+                      hipStream_t st) {
+  switch ((cols / 8 + kRingThreads - 1) / kRingThreads) {
+    case 3: return launch_tile8_ring_nv<3>(x, rows, cols, cm, l, num_int, num_fp, ndirty, ngather, dst, meta, st);
+    case 4: return launch_tile8_ring_nv<4>(x, rows, cols, cm, l, num_int, num_fp, ndirty, ngather, dst, meta, st);
+    case 5: return launch_tile8_ring_nv<5>(x, rows, cols, cm, l, num_int, num_fp, ndirty, ngather, dst, meta, st);
+    case 6: return launch_tile8_ring_nv<6>(x, rows, cols, cm, l, num_int, num_fp, ndirty, ngather, dst, meta, st);
+    case 7: return launch_tile8_ring_nv<7>(x, rows, cols, cm, l, num_int, num_fp, ndirty, ngather, dst, meta, st);
+    default: return launch_tile8_ring_nv<8>(x, rows, cols, cm, l, num_int, num_fp, ndirty, ngather, dst, meta, st);
+  }
+}
+
 template <typename IdxT, int BITS, bool BF16>
 int launch_asym(const void *x, int64_t rows, int64_t cols, const uint8_t *cm, const ColmapLayout &l, int64_t num_int,
-                int64_t num_fp, void *dst, void *meta, void *fp_x, hipStream_t st, bool tiled = false) {
+                int64_t num_fp, void *dst, void *meta, void *fp_x, hipStream_t st, bool tiled = false,
+                int64_t ndirty = -1, int64_t ngather = 0) {
   const IdxT *src_col = reinterpret_cast<const IdxT *>(cm);
   const IdxT *fp_col = reinterpret_cast<const IdxT *>(cm + l.off_fp);
   const uint32_t *mask = reinterpret_cast<const uint32_t *>(cm + l.off_mask);
@@ -1321,9 +1724,16 @@ int launch_asym(const void *x, int64_t rows, int64_t cols, const uint8_t *cm, co
     const int64_t groups = cols / 8;
 #define QUIK_STREAM(NV) \
   return launch_stream<IdxT, BITS, BF16, NV, kThreads>(x, rows, cols, cm, l, num_int, num_fp, dst, meta, fp_x, st, tiled)
-    // rows beyond 16384 columns with tile-ordered int8 output (Llama-2-70B down_proj): 180 registers per lane leave
-    // room for two workgroups per CU, so the launch is persistent and prefetches the next row (measured at 2048 x
-    // 28672: 67 -> 61 us inside the forward; at 2048 x 11008, where three workgroups fit, it is slower)
+    // fp16 rows beyond 8192 columns with tile-ordered int8 output: the LDS ring kernel
+    if constexpr (BITS == 8 && !BF16) {
+      if (tiled && ring_fits(cols, num_int, num_fp, ndirty) && ngather <= kRingThreads)
+        return launch_tile8_ring(x, rows, cols, cm, l, num_int, num_fp, static_cast<int>(ndirty),
+                                 static_cast<int>(ngather), dst, meta, st);
+    }
+    // bf16 rows beyond 16384 columns (and fp16 ones the ring kernel does not take: more than 512 outlier columns):
+    // 180 registers per lane leave room for two workgroups per CU, so the launch is persistent and prefetches the
+    // next row (measured at 2048 x 28672: 67 -> 61 us inside the forward; at 2048 x 11008, where three workgroups
+    // fit, it is slower)
     if constexpr (BITS == 8) {
       if (tiled && groups > 2048)
         return launch_stream<IdxT, BITS, BF16, 16, kThreads, false, true>(x, rows, cols, cm, l, num_int, num_fp, dst, meta,
@@ -1430,14 +1840,16 @@ extern "C" int quik_colmap_build(const int64_t *int_indices, int64_t num_int, co
                        reinterpret_cast<uint16_t *>(cm + l.off_fp), mask, reinterpret_cast<uint32_t *>(cm + l.off_grp),
                        reinterpret_cast<uint32_t *>(cm + l.off_dirty), reinterpret_cast<uint16_t *>(cm + l.off_slot),
                        reinterpret_cast<uint16_t *>(cm + l.off_kperm), reinterpret_cast<uint32_t *>(cm + l.off_patch),
-                       reinterpret_cast<uint32_t *>(cm + l.off_flags));
+                       reinterpret_cast<uint16_t *>(cm + l.off_unit), reinterpret_cast<uint16_t *>(cm + l.off_gunit),
+                       reinterpret_cast<uint16_t *>(cm + l.off_gcols), reinterpret_cast<uint32_t *>(cm + l.off_flags));
   } else {
     hipLaunchKernelGGL(colmap_build_kernel<uint32_t>, dim3(1), dim3(1024), 0, as_stream(stream), int_indices,
                        num_int, fp_indices, num_fp, cols, reinterpret_cast<uint32_t *>(cm),
                        reinterpret_cast<uint32_t *>(cm + l.off_fp), mask, reinterpret_cast<uint32_t *>(cm + l.off_grp),
                        reinterpret_cast<uint32_t *>(cm + l.off_dirty), reinterpret_cast<uint16_t *>(cm + l.off_slot),
                        reinterpret_cast<uint16_t *>(cm + l.off_kperm), reinterpret_cast<uint32_t *>(cm + l.off_patch),
-                       reinterpret_cast<uint32_t *>(cm + l.off_flags));
+                       reinterpret_cast<uint16_t *>(cm + l.off_unit), reinterpret_cast<uint16_t *>(cm + l.off_gunit),
+                       reinterpret_cast<uint16_t *>(cm + l.off_gcols), reinterpret_cast<uint32_t *>(cm + l.off_flags));
   }
   return check_launch();
 }
@@ -1504,13 +1916,16 @@ extern "C" int quik_asym_quantize_tile8(const void *x, int dtype, int64_t rows, 
   if (rows == 0) return QUIK_OK;
   if (!x || !colmap || !out8 || !meta) return QUIK_ERR_NULL;
   if (reinterpret_cast<uintptr_t>(x) % 16 != 0 || reinterpret_cast<uintptr_t>(out8) % 256 != 0) return QUIK_ERR_ALIGN;
-  if (int rc = colmap_require(colmap, cols, num_int, num_fp, as_stream(stream), kColmapStreams)) return rc;
+  uint32_t words[4];
+  if (int rc = colmap_words(colmap, cols, num_int, num_fp, as_stream(stream), words)) return rc;
+  if (!(words[0] & kColmapStreams)) return QUIK_ERR_COLMAP;
   const ColmapLayout l = colmap_layout(cols, num_int, num_fp);
   const uint8_t *cm = static_cast<const uint8_t *>(colmap);
   hipStream_t st = as_stream(stream);
-  return dtype == QUIK_F16
-             ? launch_asym<uint16_t, 8, false>(x, rows, cols, cm, l, num_int, num_fp, out8, meta, nullptr, st, true)
-             : launch_asym<uint16_t, 8, true>(x, rows, cols, cm, l, num_int, num_fp, out8, meta, nullptr, st, true);
+  return dtype == QUIK_F16 ? launch_asym<uint16_t, 8, false>(x, rows, cols, cm, l, num_int, num_fp, out8, meta, nullptr,
+                                                            st, true, words[1], words[3])
+                           : launch_asym<uint16_t, 8, true>(x, rows, cols, cm, l, num_int, num_fp, out8, meta, nullptr,
+                                                           st, true, words[1], words[3]);
 }
 
 extern "C" int quik_sym_quantize_mapped(const void *x, int64_t rows, int64_t cols, const void *colmap, int64_t num_int,

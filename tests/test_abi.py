@@ -39,8 +39,11 @@ def test_argument_validation_without_gpu():
     assert lib.quik_colmap_bytes(8192, 7936, 255) == 0
     # idx16 layout: src_col (2 B each), fp_col, one mask bit per column, one u32 per 8-column group, one u32 per
     # possible dirty group (at most one per outlier), one u16 per possible dirty group, the in-place order (one u16
-    # per integer column) and its patch list (one u32 per outlier column), flags; every section 16-byte aligned
-    assert lib.quik_colmap_bytes(8192, 7936, 256) == 7936 * 2 + 512 + 1024 + 4096 + 1024 + 512 + 7936 * 2 + 1024 + 16
+    # per integer column) and its patch list (one u32 per outlier column), the 16-column units of the int8 operand
+    # buffers (one u16 per unit, one u16 and 16 source columns per unit that may need a gather: at most one per
+    # outlier column), flags; every section 16-byte aligned
+    assert lib.quik_colmap_bytes(8192, 7936, 256) == (7936 * 2 + 512 + 1024 + 4096 + 1024 + 512 + 7936 * 2 + 1024 +
+                                                      7936 // 16 * 2 + 512 + 256 * 32 + 16)
     a16 = lambda v: (v + 15) // 16 * 16
     assert lib.quik_colmap_bytes(70000, 69000, 1000) == 69000 * 4 + a16(4000) + a16((70000 + 31) // 32 * 4) + 16
     assert lib.quik_asym_quantize(one, 0, 4, 64, one, 62, 2, 5, one, one, one, null) == -1
