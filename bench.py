@@ -60,7 +60,7 @@ PEAK_HBM_GBPS = 8000.0    # MI355X HBM3E, published
 # (`traffic_source`).  (gemm6 / quantize6: the kernels of the 6-bit matrix-core path, the default; gemm / quantize:
 # --int8-mfma)
 MEASURED_TRAFFIC_BYTES = {
-    "llama2-70b.gate_proj": {"gemm": 809.4e6, "quantize": 43.0e6, "gemm6": 758.4e6, "quantize6": 47.1e6},
+    "llama2-70b.gate_proj": {"gemm": 809.4e6, "quantize": 43.0e6, "gemm6": 757.0e6, "quantize6": 47.1e6},
 }
 TRAFFIC_SOURCE = {
     "gemm6": "offline: profiles/gemm_fused6_split_kernel__llama2-70b.gate_proj.md (rocprofv3 --pmc FETCH_SIZE / "
@@ -628,6 +628,8 @@ def main():
                      "avg_ms": round(g_avg, 4), "median_ms": round(g_ms[len(g_ms) // 2], 4),
                      "timed_launches": len(g_ms), "algorithmic_ops": int_ops},
         "roofline_quantize": {"kernel": ("quantize_fp6_wave_kernel (one wave per token row, eight rows per workgroup, 6-bit operand output)" if six and bits == 4
+                                         else "quantize_tile8_ring_kernel (row copied into an LDS ring, int8 operand output in tile order)"
+                                         if six and bits == 8 and n_in > 8192 and str(x.dtype) == "torch.float16"
                                          else "asym_quantize_stream_kernel" + (" (tile-ordered operand output)" if six else "")),
                               "bound": "hbm",
                               "achieved": round(quant_gbps, 1),
