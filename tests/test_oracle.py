@@ -444,6 +444,42 @@ def test_sim_path_agrees_to_quantisation_noise():
     assert q[0, 1] == 0 and abs(q[0, 0] + 1.0) < 1e-6
 
 
+def test_sim_quantiser_on_half_input_is_a_float32_evaluation():
+    """The reference's fake-quant runs on half tensors, but not in half arithmetic: find_params compares the row
+    minima with `torch.zeros(rows)`, a float32 tensor (experiments/quant_sim.py:178-180), so xmin, xmax, scale and
+    zero are float32 by type promotion, and `x / scale` in asymmetric_quantize (:5-7) promotes the half input as
+    well; the only rounding to half is the `.to(x_dtype)` of ActQuantWrapper.forward (:248).  The op sequence is
+    spelled out here on a half input, dtype for dtype, and must equal the oracle's float32 evaluation rounded
+    once, bit for bit (edge rows: all zero, all positive, all negative, ties at .5 of the grid)."""
+    from oracle import sim_path
+    g = torch.Generator().manual_seed(3)
+    for bits in (4, 8):
+        x = (torch.randn(64, 256, generator=g) * 3).half()
+        x[0] = 0
+        x[1] = x[1].abs() + 1
+        x[2] = -x[2].abs() - 1
+        x[3, :16] = torch.arange(16).half() * 0.5          # scale 0.5 for 4 bits: every second value is a tie
+        x[3, 16:] = 0
+        x[3, 16] = 7.5
+        maxq = torch.tensor(2 ** bits - 1)
+        tmp = torch.zeros(x.shape[0])                       # float32, as in the reference
+        xmin = torch.minimum(x.min(1)[0], tmp)
+        xmax = torch.maximum(x.max(1)[0], tmp)
+        assert xmin.dtype == torch.float32
+        both = (xmin == 0) & (xmax == 0)
+        xmin[both] = -1
+        xmax[both] = +1
+        scale = (xmax - xmin) / maxq
+        zero = torch.round(-xmin / scale)
+        scale = scale.unsqueeze(1).repeat(1, x.shape[-1]).reshape(x.shape)
+        zero = zero.unsqueeze(1).repeat(1, x.shape[-1]).reshape(x.shape)
+        q = torch.clamp(torch.round(x / scale) + zero, 0, maxq)
+        assert q.dtype == torch.float32
+        literal = (scale * (q - zero)).to(x.dtype)
+        ours = sim_path.act_fake_quant(x.float(), bits).to(x.dtype)
+        assert torch.equal(literal.view(torch.int16), ours.view(torch.int16))
+
+
 # ---------------------------------------------------------------------------- fused dequantize ops
 @pytest.mark.parametrize("spread", [3, 8, 128])
 def test_fused_dequantize_epilogues_vs_reference_known_answer_formula(spread):
