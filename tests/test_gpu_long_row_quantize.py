@@ -119,6 +119,28 @@ def test_long_rows_against_the_oracle(rows, n_in, F):
     _check(x, ii, fi, n_in)
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_long_rows_random_shapes(seed):
+    """Seeded random shapes over the kernel's whole range: 8224 .. 31744 columns in steps of 32, 0 .. 512 outlier
+    columns (in runs, clustered at one end, or spread), 1 .. 300 rows."""
+    rng = np.random.default_rng(1000 + seed)
+    F = 32 * int(rng.integers(0, 17))
+    k64 = int(rng.integers((8224 - F + 63) // 64, (31744 - F) // 64 + 1))
+    n_in = 64 * k64 + F
+    rows = int(rng.integers(9, 300))
+    kind = seed % 3
+    if kind == 0 or F == 0:
+        fi = rng.permutation(n_in)[:F]
+    elif kind == 1:                                        # runs of adjacent outlier columns
+        starts = rng.permutation(n_in // 64)[:F // 8] * 64 + rng.integers(0, 50, F // 8)
+        fi = (starts[:, None] + np.arange(8)[None, :]).ravel()
+    else:                                                  # all of them in the last columns of the row
+        fi = n_in - 1 - rng.permutation(2 * F)[:F]
+    assert len(np.unique(fi)) == F
+    x, ii, fi = _case(rng, rows, n_in, fi)
+    _check(x, ii, fi, n_in)
+
+
 def test_every_group_holds_an_outlier_column_falls_back():
     """More groups with outlier columns than the ring kernel keeps per lane (512): the streaming kernel serves the
     shape, same results."""
