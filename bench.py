@@ -44,6 +44,10 @@ WORKLOADS = {
     "llama2-13b.gate_proj.t128": (128, 5120, 13824, 256, 4),
     "llama2-13b.gate_proj.t16": (16, 5120, 13824, 256, 4),
     "llama2-13b.gate_proj.t1": (1, 5120, 13824, 256, 4),
+    "llama2-13b.gate_proj.t2": (2, 5120, 13824, 256, 4),
+    "llama2-13b.gate_proj.t4": (4, 5120, 13824, 256, 4),
+    "llama2-70b.gate_proj.t1": (1, 8192, 28672, 256, 4),
+    "llama2-70b.down_proj.int8.t1": (1, 28672, 8192, 256, 8),
     "llama2-13b.down_proj.int8.t16": (16, 13824, 5120, 256, 8),
     "llama2-70b.gate_proj.t64": (64, 8192, 28672, 256, 4),
     "llama2-70b.gate_proj.t32": (32, 8192, 28672, 256, 4),          # weight-streaming kernel, token rows in LDS

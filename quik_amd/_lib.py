@@ -48,6 +48,7 @@ SIGNATURES = {
                                               _vp]),
     "quik_layer_workspace_bytes": (_i64, [_vp, _i64]),
     "quik_layer_forward": (_int, [_vp, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp]),
+    "quik_layer_set_one_launch": (None, [_int]),
     "quik_sim_act_fake_quant": (_int, [_vp, _int, _i64, _i64, _vp, _int, _vp, _vp]),
     "quik_mixed_linear_fwd_tile8_noalloc": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _i64, _vp, _vp]),
     "quik_int4_matmul": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),

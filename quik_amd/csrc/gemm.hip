@@ -4,7 +4,12 @@
 #include <cstdint>
 #include <mutex>
 
+#include "colmap.h"
 #include "gemm_decode.h"
+#include "gemm_gemv.h"
+#ifndef GEMV_MAX_ROWS
+#define GEMV_MAX_ROWS 2
+#endif
 #include "gemm_tile8.h"
 #include "gemm_kernels.h"
 
@@ -174,8 +179,46 @@ bool decode_x_fits(const FusedArgs &p) {
          (p.N + 31) / 32 > num_cus();
 }
 
+// At most kGemvMaxRows token rows (fused form): one wave per output column, gemm_gemv.h.  Needs 16-byte aligned rows
+// of both weight arrays and room in LDS for the token rows.
+constexpr int kGemvMaxRows = GEMV_MAX_ROWS;
+bool gemv_ok(const FusedArgs &p, bool quant = false) {
+  const auto aligned = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
+  const int mt = p.M <= 1 ? 1 : p.M <= 2 ? 2 : 4;
+  return p.M >= 1 && p.M <= kGemvMaxRows && p.kbytes >= 16 && p.kbytes % 16 == 0 && p.F % 8 == 0 &&
+         (quant || aligned(p.qx)) && aligned(p.qw) && (p.F == 0 || ((quant || aligned(p.fp_x)) && aligned(p.fp_w))) &&
+         gemv_smem(mt, p.kbytes, p.F) + gemv_table_bytes((p.N + kGemvWaves * num_cus() - 1) / (kGemvWaves * num_cus())) <=
+             kLdsBytes;
+}
+template <int MODE, bool BF16, int MT, bool QUANT>
+int launch_gemv_mt(const FusedArgs &p, const GemvQuant &q, hipStream_t st) {
+  auto kern = gemv_decode_kernel<MODE, BF16, MT, QUANT>;
+  if (int rc = prepare(kern, kLdsBytes)) return rc;  // (the size varies with the layer: set once to the most)
+  // persistent waves, one column at a time each: two workgroups per CU when their LDS fits twice
+  const int64_t fixed = gemv_smem(MT, p.kbytes, p.F) + (QUANT ? gemv_quant_lds(q.cols, q.num_int).bytes : 0);
+  const int64_t per_cu = 2 * (fixed + 4096) <= kLdsBytes ? 2 : 1;
+  int64_t grid = (p.N + kGemvWaves - 1) / kGemvWaves;
+  if (grid > per_cu * num_cus()) grid = per_cu * num_cus();
+  const int64_t smem = fixed + gemv_table_bytes((p.N + kGemvWaves * grid - 1) / (kGemvWaves * grid));
+  if (smem > kLdsBytes) return kChainNotHandled;
+  hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(grid)), dim3(kGemvWaves * 64), static_cast<size_t>(smem), st, p, q);
+  return check_launch();
+}
+template <int MODE, bool BF16, bool QUANT = false>
+int launch_gemv(const FusedArgs &p, const GemvQuant &q, hipStream_t st) {
+  if (p.M <= 1) return launch_gemv_mt<MODE, BF16, 1, QUANT>(p, q, st);
+  if (p.M <= 2) return launch_gemv_mt<MODE, BF16, 2, QUANT>(p, q, st);
+  return launch_gemv_mt<MODE, BF16, 4, QUANT>(p, q, st);
+}
+
 template <int MODE, bool BF16, bool FUSED>
 int launch_decode(const FusedArgs &p, int32_t *C, int ldc, hipStream_t st) {
+  if constexpr (FUSED) {
+    if (gemv_ok(p)) {
+      const int rc = launch_gemv<MODE, BF16>(p, GemvQuant{}, st);
+      if (rc != kChainNotHandled) return rc;
+    }
+  }
   if (decode_x_fits<8, FUSED>(p)) return launch_decode_w<MODE, BF16, FUSED, 8, true>(p, C, ldc, st);
   if (decode_waves(p.N, p.kbytes) == 8) return launch_decode_w<MODE, BF16, FUSED, 8, false>(p, C, ldc, st);
   return launch_decode_w<MODE, BF16, FUSED, 4, false>(p, C, ldc, st);
@@ -571,6 +614,51 @@ extern "C" int quik_int8_matmul(const int8_t *A, const int8_t *B, int32_t *C, in
   if (M == 0 || N == 0) return QUIK_OK;
   return run_i32<kInt8>(reinterpret_cast<const uint8_t *>(A), reinterpret_cast<const uint8_t *>(B), C, M, N, K,
                         as_stream(stream));
+}
+
+// MixedQLinear forward (asymmetric activations) for at most kGemvMaxRows token rows in ONE launch: the kernel of
+// gemm_gemv.h quantises the rows itself.  kChainNotHandled: the shape is left to the two-launch path.
+int quik::gemv_forward_one_launch(const void *x, int dtype, int64_t rows, int64_t cols, const void *colmap,
+                                  int64_t num_int, int64_t num_fp, int bits, const void *qw, const void *s_col,
+                                  const void *w_red, const void *fp_w, const void *bias, int64_t N, void *out,
+                                  hipStream_t st) {
+  // (cols % 32, num_int % 128: the column map's group and unit tables arrive as whole 16-byte pieces)
+  if (rows < 1 || rows > kGemvMaxRows || !w_red || cols % 32 != 0 || cols > kStreamMaxCols || num_int % 128 != 0 ||
+      num_fp > kGemvWaves * 64 ||
+      (reinterpret_cast<uintptr_t>(x) & 15) != 0 || N > (1 << 30))
+    return kChainNotHandled;
+  uint32_t words[4];
+  if (int rc = colmap_words(colmap, cols, num_int, num_fp, st, words)) return rc == QUIK_ERR_COLMAP ? kChainNotHandled : rc;
+  if (!(words[0] & kColmapStreams)) return kChainNotHandled;
+  const ColmapLayout l = colmap_layout(cols, num_int, num_fp);
+  const uint8_t *cm = static_cast<const uint8_t *>(colmap);
+  FusedArgs p{};
+  p.qw = static_cast<const uint8_t *>(qw);
+  p.s_col = static_cast<const uint16_t *>(s_col);
+  p.w_red = static_cast<const uint16_t *>(w_red);
+  p.fp_w = static_cast<const uint16_t *>(fp_w);
+  p.bias = static_cast<const uint16_t *>(bias);
+  p.out = static_cast<uint16_t *>(out);
+  p.M = static_cast<int>(rows);
+  p.N = static_cast<int>(N);
+  p.ldo = static_cast<int>(N);
+  p.kbytes = static_cast<int>(bits == 4 ? num_int / 2 : num_int);
+  p.F = static_cast<int>(num_fp);
+  p.meta_stride = 2;
+  p.shift = bits == 4 ? 8.0f : 128.0f;
+  if (!gemv_ok(p, true)) return kChainNotHandled;
+  GemvQuant q{};
+  q.x = static_cast<const uint16_t *>(x);
+  q.fp_col = reinterpret_cast<const uint16_t *>(cm + l.off_fp);
+  q.grp = reinterpret_cast<const uint32_t *>(cm + l.off_grp);
+  q.unit = reinterpret_cast<const uint16_t *>(cm + l.off_unit);
+  q.gather_unit = reinterpret_cast<const uint16_t *>(cm + l.off_gunit);
+  q.gather_cols = reinterpret_cast<const uint16_t *>(cm + l.off_gcols);
+  q.cols = static_cast<int>(cols), q.num_int = static_cast<int>(num_int), q.num_fp = static_cast<int>(num_fp);
+  q.ngather = static_cast<int>(words[3]);
+  if (q.ngather > kGemvWaves * 64) return kChainNotHandled;  // (one gathered unit per thread)
+  if (bits == 4) return dtype == QUIK_F16 ? launch_gemv<kInt4, false, true>(p, q, st) : launch_gemv<kInt4, true, true>(p, q, st);
+  return dtype == QUIK_F16 ? launch_gemv<kInt8, false, true>(p, q, st) : launch_gemv<kInt8, true, true>(p, q, st);
 }
 
 extern "C" int quik_mixed_linear_fwd(const void *qx, const void *qw, const void *meta, const void *s_col,

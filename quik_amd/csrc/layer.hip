@@ -10,6 +10,9 @@ namespace {
 
 inline int64_t align256(int64_t v) { return (v + 255) & ~int64_t(255); }
 
+// quik_layer_set_one_launch: tests and measurements switch the one-launch form of small calls off to compare
+bool layer_one_launch = true;
+
 struct LayerPlan {
   bool tiled;
   int64_t off_q, off_meta, off_fp, bytes;
@@ -55,6 +58,8 @@ LayerPlan plan_layer(const quik_layer *l, int64_t rows) {
 
 using namespace quik;
 
+extern "C" void quik_layer_set_one_launch(int on) { layer_one_launch = on != 0; }
+
 extern "C" int64_t quik_layer_workspace_bytes(const quik_layer *layer, int64_t rows) {
   if (!layer_valid(layer) || rows <= 0) return 0;
   return plan_layer(layer, rows).bytes;
@@ -78,6 +83,21 @@ extern "C" int quik_layer_forward(const quik_layer *layer, const void *x, int64_
   uint8_t *ws = static_cast<uint8_t *>(workspace);
   void *q = ws + p.off_q, *meta = ws + p.off_meta, *fp_x = l.num_fp > 0 ? ws + p.off_fp : nullptr;
   const void *w_red = l.symmetric ? nullptr : l.reduced_w;
+  if (!l.symmetric && !p.tiled && l.colmap_streams && layer_one_launch) {
+    // one or two token rows: one launch, the quantize inside the weight-streaming kernel (the workspace is not used)
+    const int rc = gemv_forward_one_launch(x, l.dtype, rows, l.in_features, l.colmap, l.num_int, l.num_fp, l.bits,
+                                           l.int_weight, l.weights_scales, w_red, l.fp_weight, l.bias, l.out_features,
+                                           out, as_stream(stream));
+    if (rc != kChainNotHandled) {
+      if (rc == QUIK_OK && mid_event) {  // (profiling hook: there is no second launch to mark)
+        if (hipError_t e = hipEventRecord(static_cast<hipEvent_t>(mid_event), as_stream(stream)); e != hipSuccess) {
+          set_last_hip_error(e);
+          return QUIK_ERR_LAUNCH;
+        }
+      }
+      return rc;
+    }
+  }
   if (l.symmetric) {
     if (l.dtype != QUIK_F16 || !l.colmap_streams) return QUIK_ERR_DTYPE;  // the caller's op sequence serves these
     if (int rc = quik_sym_quantize_mapped(x, rows, l.in_features, l.colmap, l.num_int, l.num_fp, l.bits, l.sym_divisor,
