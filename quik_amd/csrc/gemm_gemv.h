@@ -170,18 +170,28 @@ __device__ __forceinline__ void gemv_quantize_row(const uint8_t *raw, const uint
   __syncthreads();  // (the raw row, the staging area and the reduction slots are free for the next row)
 }
 
-// sum over the wave in a fixed order (every lane active): four DPP steps, then the four rows of 16
-__device__ __forceinline__ float wave_sum_f(float v) {
+// Sums over the wave in a fixed order (every lane active), result in every lane: four DPP steps make each row of 16
+// uniform, two row broadcasts (lane 15 of a row into the next row, lane 31 into the upper half) leave the total in
+// the last row, one scalar read hands it out.  (Four scalar reads and three scalar adds instead of the broadcasts
+// cost more here: every read of a vector register that a DPP instruction has just written waits out a hazard.)
+constexpr int kDppRowBcast15 = 0x142, kDppRowBcast31 = 0x143;
+__device__ __forceinline__ int32_t wave_total(int32_t v) {
+  v += dpp_move_i<kDppSwap1>(v);
+  v += dpp_move_i<kDppSwap2>(v);
+  v += dpp_move_i<kDppHalfMirror>(v);
+  v += dpp_move_i<kDppMirror>(v);
+  v += __builtin_amdgcn_update_dpp(0, v, kDppRowBcast15, 0xA, 0xF, false);
+  v += __builtin_amdgcn_update_dpp(0, v, kDppRowBcast31, 0xC, 0xF, false);
+  return __builtin_amdgcn_readlane(v, 63);
+}
+__device__ __forceinline__ float wave_total(float v) {
   v += dpp_move<kDppSwap1>(v);
   v += dpp_move<kDppSwap2>(v);
   v += dpp_move<kDppHalfMirror>(v);
   v += dpp_move<kDppMirror>(v);
-  const int b = __builtin_bit_cast(int, v);
-  const float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 0));
-  const float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 16));
-  const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 32));
-  const float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 48));
-  return (r0 + r1) + (r2 + r3);
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), kDppRowBcast15, 0xA, 0xF, false));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), kDppRowBcast31, 0xC, 0xF, false));
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
 
 template <int MODE, bool BF16, int MT, bool QUANT = false>
@@ -358,8 +368,8 @@ __global__ __launch_bounds__(kGemvWaves * 64) void gemv_decode_kernel(FusedArgs 
       float tf = 0.0f;
 #pragma unroll
       for (int m = 0; m < MT; ++m) {
-        const int32_t si = wave_sum(acc[m]);
-        const float sf = wave_sum_f(accf[m]);
+        const int32_t si = wave_total(acc[m]);
+        const float sf = wave_total(accf[m]);
         ti = lane == m ? si : ti;
         tf = lane == m ? sf : tf;
         acc[m] = 0;
