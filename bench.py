@@ -595,9 +595,11 @@ def main():
             "gemm_fused8t_split_kernel / gemm_fused8t_kernel (tile-ordered int8 operands, one launch per step)"
         dtype = "int8"
     elif mod.fused:
-        gemm_kernel = "gemm_decode_kernel (weight streaming, one launch per step)" if M <= 32 else \
+        gemm_kernel = "gemv_decode_kernel (one or two token rows: quantize and weight-streaming matrix-vector product " \
+            "in ONE launch; avg_ms below is the interval behind it, the launch itself is in roofline_quantize.avg_ms)" \
+            if M <= 2 else "gemm_decode_kernel (weight streaming, one launch per step)" if M <= 32 else \
             "gemm_fused_split_kernel / gemm_fused_kernel (one launch per step)"
-        dtype = "int8" if bits == 8 else "int4 (on int8 MFMA)"
+        dtype = "int8" if bits == 8 else "int4 (dot-product instructions)" if M <= 2 else "int4 (on int8 MFMA)"
     else:
         gemm_kernel = "gemm_i32_split_kernel + dequantize + F.linear"
         dtype = "int8" if bits == 8 else "int4 (on int8 MFMA)"
