@@ -625,12 +625,14 @@ def test_kernel_path_vs_simulated_path(bits, bf16):
     assert e_ker < (0.2 if bits == 4 else 0.02), e_ker
 
 
-@pytest.mark.parametrize("tokens", [300, 40, 4])     # 6-bit matrix-core path (two tile plans), decode kernel
-def test_forward_under_hip_graph_replays(tokens):
+# 6-bit matrix-core path (two tile plans), weight-streaming MFMA kernel, matrix-vector kernel behind a quantize
+# launch (K = 960 is not a multiple of 128) and with the quantize inside (one launch)
+@pytest.mark.parametrize("tokens,n_in", [(300, 1024), (40, 1024), (4, 1024), (2, 1024), (1, 1088), (2, 1088)])
+def test_forward_under_hip_graph_replays(tokens, n_in):
     """The forward (quantize + GEMM, no allocation or synchronisation inside the library) captured in a
     HIP graph: every replay, with new input contents and eager work in between, equals the eager result."""
     rng = np.random.default_rng(60 + tokens)
-    N, n_in, F, bits = 384, 1024, 64, 4
+    N, F, bits = 384, 64, 4
     W, s_w, ii, fi = _layer(rng, N, n_in, F, bits)
     mod = _module(W, s_w, fi, bits, rng.standard_normal(N).astype(np.float16))
     static_x = _t(_acts(rng, tokens, n_in, fi).astype(np.float16))
