@@ -86,6 +86,9 @@ CASES = [
     (1, 2048, 4096 + 128, 128, 4, torch.bfloat16, True),
     (2, 1024, 2048 + 64, 64, 8, torch.bfloat16, False),
     (1, 8192, 28672, 256, 8, torch.float16, False),      # 70B down_proj: the longest rows
+    (2, 1001, 1024 + 64, 64, 4, torch.float16, False),   # ragged N: odd row stride of the output
+    (1, 5, 128 + 32, 32, 4, torch.float16, False),       # fewer columns than waves, the shortest K
+    (2, 77, 256 + 32, 32, 8, torch.bfloat16, True),
 ]
 
 
