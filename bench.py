@@ -12,7 +12,8 @@ columns, W4A4 asymmetric activations.
 Prints ONE JSON line.  value = 2*M*N*K / t_step in TOPS (the integer GEMM's operations over the
 whole forward time; the outlier GEMM's 2*M*N*F flops are not counted).  `roofline` is for the
 dominant kernel (the fused GEMM, priced against the peak of the MFMA instructions it issues: 10.1 POP/s
-for the 6-bit path, 5.0 POP/s for int8); `roofline_quantize` for the
+for the 6-bit path, 5.0 POP/s for int8; for the workloads of at most 32 token rows the weight-streaming
+kernel, priced against the HBM peak); `roofline_quantize` for the
 quantize kernel (bounded by HBM).  Kernel durations are measured with HIP events recorded on
 the stream the kernels run on, inside the timed region.  `cpu_baseline` times the CPU
 restatement of the reference's fake-quant path (oracle/sim_path.py) on the host cores.
@@ -596,13 +597,36 @@ def main():
         dtype = "int8"
     elif mod.fused:
         gemm_kernel = "gemv_decode_kernel (one or two token rows: quantize and weight-streaming matrix-vector product " \
-            "in ONE launch; avg_ms below is the interval behind it, the launch itself is in roofline_quantize.avg_ms)" \
+            "in ONE launch)" \
             if M <= 2 else "gemm_decode_kernel (weight streaming, one launch per step)" if M <= 32 else \
             "gemm_fused_split_kernel / gemm_fused_kernel (one launch per step)"
         dtype = "int8" if bits == 8 else "int4 (dot-product instructions)" if M <= 2 else "int4 (on int8 MFMA)"
     else:
         gemm_kernel = "gemm_i32_split_kernel + dequantize + F.linear"
         dtype = "int8" if bits == 8 else "int4 (on int8 MFMA)"
+
+    roofline = {"kernel": gemm_kernel,
+                "bound": "mfma", "achieved": round(gemm_tops, 2), "peak": peak,
+                "unit": "TOP/s", "frac": round(gemm_tops / peak, 4),
+                "frac_of_int8_peak": round(gemm_tops / PEAK_INT8_TOPS, 4),
+                "traffic": traffic.get("gemm6" if six else "gemm") if mod.fused else None,
+                "traffic_source": TRAFFIC_SOURCE["gemm6" if six else "gemm"]
+                if mod.fused and traffic.get("gemm6" if six else "gemm") else None,
+                "avg_ms": round(g_avg, 4), "median_ms": round(g_ms[len(g_ms) // 2], 4),
+                "timed_launches": len(g_ms), "algorithmic_ops": int_ops}
+    one_launch = mod.fused and not six and M <= 2
+    if mod.fused and not six and M <= 32:
+        # the weight-streaming kernels are bound by HBM: every weight byte once, plus the small operands
+        stream_bytes = N * K * bits // 8 + N * F * 2 + 3 * N * 2 + M * n_in * 2 + M * N * 2
+        launch_ms = q_avg if one_launch else g_avg       # (one launch: it ends at the event the library records)
+        launch_med = (q_ms if one_launch else g_ms)[len(g_ms) // 2]
+        gbps = stream_bytes / (launch_ms * 1e-3) / 1e9
+        roofline = {"kernel": gemm_kernel, "bound": "hbm", "achieved": round(gbps, 1), "peak": PEAK_HBM_GBPS,
+                    "unit": "GB/s", "frac": round(gbps / PEAK_HBM_GBPS, 4), "traffic": None,
+                    "avg_ms": round(launch_ms, 4), "median_ms": round(launch_med, 4), "timed_launches": len(g_ms),
+                    "algorithmic_bytes": stream_bytes,
+                    "note": "avg_ms includes the cost of one event record (several us); kernel-trace durations of "
+                            "the launch alone: profiles/"}
 
     res = {
         "metric": "MixedQLinear fwd TOPS (2*M*N*K / forward time), 1 GPU",
@@ -624,16 +648,8 @@ def main():
         "resident_weight_bytes": mod.weight_bytes(),
         "verified_vs_oracle": None if spot is None else {"tiles": 3, "max_abs_err_over_rms": round(spot, 6),
                                                          "tolerance": 1e-2},
-        "roofline": {"kernel": gemm_kernel,
-                     "bound": "mfma", "achieved": round(gemm_tops, 2), "peak": peak,
-                     "unit": "TOP/s", "frac": round(gemm_tops / peak, 4),
-                     "frac_of_int8_peak": round(gemm_tops / PEAK_INT8_TOPS, 4),
-                     "traffic": traffic.get("gemm6" if six else "gemm") if mod.fused else None,
-                     "traffic_source": TRAFFIC_SOURCE["gemm6" if six else "gemm"]
-                     if mod.fused and traffic.get("gemm6" if six else "gemm") else None,
-                     "avg_ms": round(g_avg, 4), "median_ms": round(g_ms[len(g_ms) // 2], 4),
-                     "timed_launches": len(g_ms), "algorithmic_ops": int_ops},
-        "roofline_quantize": {"kernel": ("quantize_fp6_wave_kernel (one wave per token row, eight rows per workgroup, 6-bit operand output)" if six and bits == 4
+        "roofline": roofline,
+        "roofline_quantize": None if one_launch else {"kernel": ("quantize_fp6_wave_kernel (one wave per token row, eight rows per workgroup, 6-bit operand output)" if six and bits == 4
                                          else "quantize_tile8_ring_kernel (row copied into an LDS ring, int8 operand output in tile order)"
                                          if six and bits == 8 and n_in > 8192 and str(x.dtype) == "torch.float16"
                                          else "asym_quantize_stream_kernel" + (" (tile-ordered operand output)" if six else "")),
