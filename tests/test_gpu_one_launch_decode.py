@@ -160,3 +160,43 @@ def test_three_rows_and_symmetric_layers_keep_two_launches():
     xt = torch.from_numpy(rng.standard_normal((3, 1088)).astype(np.float16)).to(DEV)
     _, ws = _call(mod, xt, 0x5A)
     assert not bool((ws == 0x5A).all())
+
+
+def test_decode_sizes_random_shapes_against_the_oracle():
+    """Seeded sweep over calls of 1 .. 32 rows: ragged N and K, with and without outlier columns and bias, both
+    widths.  Whatever kernel the library picks (matrix-vector kernel in one or two launches, MFMA weight-streaming
+    kernel with the token rows streamed or resident in LDS), the module's output stays within the fused forward's
+    tolerance of the oracle, and equals the two-launch form bit for bit where the one-launch form applies."""
+    from quik_amd import _lib as L
+    lib = L.load()
+    rng = np.random.default_rng(777)
+    for it in range(28):
+        bits = int(rng.choice([4, 8]))
+        rows = int(rng.choice([1, 1, 2, 2, 3, 4, 5, 8, 13, 16, 17, 31, 32]))
+        F = int(rng.choice([0, 8, 16, 32, 64, 72, 256]))
+        K = int(rng.choice([32, 64, 96, 128, 256, 384, 640, 992, 1024, 2048, 4864]))    # (K % 32 == 0 and F % 8 == 0: the GEMM's row alignment)
+        N = int(rng.choice([1, 7, 8, 33, 100, 256, 513, 1000, 2048, 8200, 9000]))
+        n_in = K + F
+        with_bias = bool(rng.integers(0, 2))
+        case = (it, rows, N, n_in, F, bits, with_bias)
+        mod, W, s_w, fi, ii, bias = _layer(rng, N, n_in, F, bits, torch.float16, bool(rng.integers(0, 2)) and F >= 8 and n_in >= 8 * F + 64)
+        if not with_bias:
+            mod.bias = None
+            bias = None
+        x = rng.standard_normal((rows, n_in)).astype(np.float32)
+        x[:, fi] *= 50
+        xt = torch.from_numpy(x).to(DEV, torch.float16)
+        lib.quik_layer_set_one_launch(1)
+        out1 = mod(xt)[0]
+        lib.quik_layer_set_one_launch(0)
+        out2 = mod(xt)[0]
+        lib.quik_layer_set_one_launch(1)
+        if rows <= 2:
+            assert torch.equal(out1.view(torch.int16), out2.view(torch.int16)), case
+        omod = qo.from_float(W, s_w, fi, bits)
+        want, _ = qo.mixed_qlinear_forward(xt.cpu().numpy(), omod, bits, bias=bias)
+        w64 = want.astype(np.float64)
+        rms = float(np.sqrt((w64 ** 2).mean())) + 1e-30
+        for got in (out1, out2):
+            err = np.abs(got.float().cpu().numpy() - w64).max()
+            assert err <= 1e-2 * rms, (case, err, rms)
