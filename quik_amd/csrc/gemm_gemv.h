@@ -1,7 +1,7 @@
-// MixedQLinear forward for at most four token rows (single-stream decode): a matrix-vector product per token row,
-// bound by one pass over the weights.
+// MixedQLinear forward for very few token rows (single-stream decode; the host uses it for one and two): a
+// matrix-vector product per token row, bound by one pass over the weights.
 //
-// With one to four token rows a 32-row MFMA block is mostly padding, and what the weight-streaming MFMA kernel
+// With so few token rows a 32-row MFMA block is mostly padding, and what the weight-streaming MFMA kernel
 // (gemm_decode.h) does around the MFMAs (LDS transpose of every weight chunk, partial sums of eight waves meeting
 // in LDS at every slab end, four barriers per slab) costs more than the products.  Here a WAVE owns whole output
 // columns: it streams a column's weight row with 16-byte loads (1 KB per instruction, whole lines), multiplies with
@@ -10,7 +10,7 @@
 // keeps in LDS (at most 4 x K bytes, copied once), and sums over the wave at the column's end.  No barrier after the
 // copy of the token rows, no cross-wave sums.  The outlier columns (fp16 / bf16 weights and values) travel through
 // the same stream of loads as further 16-byte pieces of the column, kGemvPieces pieces ahead, across column
-// boundaries; a column's three epilogue scalars come through the scalar cache, requested when the column starts.
+// boundaries; a column's three epilogue scalars wait in a small LDS table that the workgroup fills at the start.
 // Integer sums are exact; the fp32 outlier sum is taken in lane order, then over the wave.  Epilogue as in the other
 // fused kernels: (f32(acc) (s_row s_col) + outliers) + (zs w_red + bias).
 //
@@ -219,7 +219,7 @@ __global__ __launch_bounds__(kGemvWaves * 64) void gemv_decode_kernel(FusedArgs 
   const int pieces = ipieces + fpieces;
   uint8_t *xs = smem, *fs = smem + MT * xstride;
 
-  // ---- the stream's first loads go out before anything else: they do not depend on the token rows
+  // ---- the stream's first loads go out before anything that waits: they do not depend on the token rows
   const int step = gridDim.x * kGemvWaves;
   const int n_first = blockIdx.x * kGemvWaves + wave;
   const uint8_t *fw = fbytes > 0 ? reinterpret_cast<const uint8_t *>(p.fp_w) : p.qw;
@@ -241,13 +241,18 @@ __global__ __launch_bounds__(kGemvWaves * 64) void gemv_decode_kernel(FusedArgs 
     }
   };
   v4i buf[kGemvPieces];
-  static_for<kGemvPieces - 1>([&](auto I) __attribute__((always_inline)) { issue(buf[I.value]); });
+  auto first_pieces = [&]() __attribute__((always_inline)) {
+    static_for<kGemvPieces - 1>([&](auto I) __attribute__((always_inline)) { issue(buf[I.value]); });
+  };
 
   float srow = 0.0f, zs = 0.0f;  // lane m keeps token row m's scale and zero-point term
   if constexpr (QUANT) {
     // ---- token rows -> codes and outlier values in LDS, quantised here.  The first row and the column map's
     // tables arrive together as direct copies; this thread's gathered unit and outlier column go to registers
     // (unconditional loads from clamped indices: under conditions each would wait for the one before it).
+    // These few kilobytes are requested IN FRONT of the first weight pieces: a wave's loads are counted in the
+    // order of issue, and behind the pieces (32 KB per workgroup, every workgroup of the launch at once) the row
+    // would count as landed only after that whole burst, with the quantize work still to come.
     uint8_t *area = smem + MT * (xstride + fstride) + gemv_table_bytes((p.N + step - 1) / step);
     const GemvQuantLds ql = gemv_quant_lds(quant.cols, quant.num_int);
     const uint32_t area_lds = lds_address(area);
@@ -261,9 +266,16 @@ __global__ __launch_bounds__(kGemvWaves * 64) void gemv_decode_kernel(FusedArgs 
     const uint4 gb = reinterpret_cast<const uint4 *>(has_g ? quant.gather_cols + 16 * tid : spare)[1];
     const uint32_t goff[8] = {ga.x, ga.y, ga.z, ga.w, gb.x, gb.y, gb.z, gb.w};
     const int fcol = *(has_f ? quant.fp_col + tid : spare);
+    __builtin_amdgcn_sched_barrier(0);
+    first_pieces();
+    __builtin_amdgcn_sched_barrier(0);
     for (int m = 0; m < p.M; ++m) {
+      // A second row takes the first one's place (both requested at once at the start were no faster, measured, and
+      // cost a second row of LDS); it sits behind the weight pieces, which have long landed by then.
       if (m > 0) gemv_copy_in(quant.x + int64_t(m) * quant.cols, quant.cols * 2, area_lds + ql.raw, wave, lane);
-      __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+      // the first row: everything but the weight pieces, which were issued last
+      if (m == 0) __builtin_amdgcn_s_waitcnt(vmcnt_imm(kGemvPieces - 1));
+      else __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
       __syncthreads();
       float sc, zr;
       gemv_quantize_row<MODE == kInt4 ? 4 : 8, BF16>(area + ql.raw, reinterpret_cast<const uint32_t *>(area + ql.grp),
@@ -276,6 +288,7 @@ __global__ __launch_bounds__(kGemvWaves * 64) void gemv_decode_kernel(FusedArgs 
       }
     }
   } else {
+    first_pieces();
     // ---- token rows -> LDS (codes, outlier values) with direct copies, 1 KB each.  Rows past M repeat the last one
     // (their results are never stored); lanes past a row's end repeat its last 16 bytes (the weight pieces that
     // stand against them are masked to zero where they are used).
