@@ -87,9 +87,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_decode_kernel(FusedArgs args,
   };
   // ---- XLDS: copy the token rows into LDS, 16-byte unit u = ((chunk step) * 2 + K half) * M + row
   const uint8_t *x_lds = smem + decode_smem<WAVES, FUSED, XLDS>();
-  if constexpr (XLDS) {
+  auto copy_token_rows = [&]() __attribute__((always_inline)) {
     const int units = nchunks * kDecodeSteps * 2 * p.M;
-    const uint32_t lds_base = lds_address(x_lds);
+    const uint32_t lds_base = lds_address(smem + decode_smem<WAVES, FUSED, XLDS>());
     for (int u0 = __builtin_amdgcn_readfirstlane(wave) * 64; u0 < units; u0 += WAVES * 64) {
       const int u = u0 + lane < units ? u0 + lane : units - 1;  // the last copy is padded with a valid unit
       const int cs = u / (2 * p.M), rem = u - cs * 2 * p.M;
@@ -98,8 +98,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_decode_kernel(FusedArgs args,
       off = off < kbytes ? off : 0;  // past the row's end: the weights of these positions are zeroed below
       dma_load16(p.qx, static_cast<uint32_t>(row * kbytes + off), lds_base + u0 * 16);
     }
-    x_lds += (h * p.M + mrow) * 16;  // this lane's unit inside a step
-  }
+  };
+  if constexpr (XLDS) x_lds += (h * p.M + mrow) * 16;  // this lane's unit inside a step
   const int x_step = 2 * p.M * 16;
   // ---- loader: item (ld_slab, ld_c) -> b, then advance to this wave's next item
   int ld_slab = blockIdx.x, ld_c = wave;
@@ -322,7 +322,12 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_decode_kernel(FusedArgs args,
   int slab = blockIdx.x, c = wave;  // the item being multiplied
   slab_begin(slab);
   static_for<NB - 1>([&](auto I) __attribute__((always_inline)) { issue(buf[I.value]); });
-  if constexpr (XLDS) {  // every wave's share of the token rows has landed (with the first weight chunks)
+  if constexpr (XLDS) {
+    // The copy of the token rows (up to 128 KB out of L2) is requested BEHIND the first weight chunks: issuing it
+    // takes the workgroup about a microsecond, in which the weight requests are already on their way to HBM.
+    __builtin_amdgcn_sched_barrier(0);
+    copy_token_rows();
+    // every wave's share of the token rows has landed (with the first weight chunks)
     __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
     __syncthreads();
   }
