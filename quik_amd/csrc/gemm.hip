@@ -207,8 +207,10 @@ int launch_gemv_mt(const FusedArgs &p, const GemvQuant &q, hipStream_t st) {
 template <int MODE, bool BF16, bool QUANT = false>
 int launch_gemv(const FusedArgs &p, const GemvQuant &q, hipStream_t st) {
   if (p.M <= 1) return launch_gemv_mt<MODE, BF16, 1, QUANT>(p, q, st);
-  if (p.M <= 2) return launch_gemv_mt<MODE, BF16, 2, QUANT>(p, q, st);
-  return launch_gemv_mt<MODE, BF16, 4, QUANT>(p, q, st);
+  if constexpr (kGemvMaxRows > 2) {  // (only built when the row limit is raised: gemv_ok() admits no such call otherwise)
+    if (p.M > 2) return launch_gemv_mt<MODE, BF16, 4, QUANT>(p, q, st);
+  }
+  return launch_gemv_mt<MODE, BF16, 2, QUANT>(p, q, st);
 }
 
 template <int MODE, bool BF16, bool FUSED>
