@@ -495,6 +495,31 @@ def main():
     e1.record()
     torch.cuda.synchronize()
     q_b2b = e0.elapsed_time(e1) / 50
+    # ... and the same 20 launches replayed from a HIP graph: no host time and no event records between them, so
+    # the period per launch is the kernel plus the gap between two dependent launches
+    q_graph = None
+    try:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            quantize_only()
+        torch.cuda.current_stream().wait_stream(side)
+        qg = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(qg):
+            for _ in range(20):
+                quantize_only()
+        for _ in range(3):
+            qg.replay()
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(5):
+            qg.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        q_graph = e0.elapsed_time(e1) / 100
+        del qg
+    except Exception as exc:   # noqa: BLE001  (an extra figure: the benchmark does not depend on it)
+        print(f"bench: quantize graph timing skipped: {exc}", file=sys.stderr)
     traffic = MEASURED_TRAFFIC_BYTES.get(name, {})
 
     # the same forward without the two event records per step: the figure a caller of the module sees
@@ -662,11 +687,15 @@ def main():
                               "avg_ms": round(q_avg, 5),
                               "median_ms": round(q_ms[len(q_ms) // 2], 5), "algorithmic_bytes": quant_bytes,
                               "back_to_back_ms": round(q_b2b, 5),
+                              "graph_back_to_back_ms": None if q_graph is None else round(q_graph, 5),
+                              "frac_by_graph_period": None if q_graph is None
+                              else round(quant_bytes / (q_graph * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4),
                               "note": "avg_ms: from the event behind the previous forward to the event the library "
                                       "records between the quantize launch and the GEMM launch (the launch plus the "
                                       "cost of one event record, several us); back_to_back_ms: per launch over 50 consecutive "
                                       "launches after the timed region (bound by the host: ~14 us of Python per "
-                                      "call); kernel-trace durations of the launch alone: profiles/"},
+                                      "call); graph_back_to_back_ms: period per launch of 20 launches replayed from a "
+                                      "HIP graph (kernel + the gap between dependent launches); kernel-trace durations of the launch alone: profiles/"},
     }
     if not args.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline(name, x_cpu, W_cpu, int_idx, fp_idx)
