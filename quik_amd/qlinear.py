@@ -248,6 +248,15 @@ class MixedQLinear(torch.nn.Module):
         if shared_input is not None and hasattr(shared_input, "register"):
             shared_input.register(self)
 
+    def _apply(self, fn, recurse=True):
+        """`.to()` / `.half()` / `.bfloat16()` convert the floating-point buffers; `dtype` (a plain attribute in the
+        reference, qlinear.py:52, fixed at construction) follows them, so that a converted module computes in the
+        type its buffers now have instead of failing on the mismatch."""
+        out = super()._apply(fn, recurse)
+        if self.weights_scales.dtype in (torch.float16, torch.bfloat16):
+            self.dtype = self.weights_scales.dtype
+        return out
+
     # -- cached column map: rebuilt when the index buffers move or are written in place
     def _column_map(self):
         key = (self.int_indices.data_ptr(), self.fp_indices.data_ptr(), self.int_indices._version,

@@ -195,6 +195,12 @@ def test_from_float_buffers_on_cpu():
         assert set(mod.state_dict()) == {"weights_scales", "int_weight", "int_indices", "fp_indices", "fp_weight",
                                          "reduced_w"}
     assert pack_to_i4(torch.tensor([[-8, 7]])).tolist() == [[0x78]]
+    # a converted module computes in the type its buffers now have (the integer buffers keep theirs)
+    assert mod.dtype == torch.float16
+    mod = mod.to(torch.bfloat16)
+    assert mod.dtype == torch.bfloat16 and mod.weights_scales.dtype == torch.bfloat16
+    assert mod.int_weight.dtype == torch.int8 and mod.int_indices.dtype == torch.int64
+    assert mod.half().dtype == torch.float16
     with pytest.raises(AssertionError, match="duplication"):
         MixedQLinear.from_float(lin, torch.from_numpy(W), torch.from_numpy(s_w), None, torch.tensor([1, 1]), bits=4)
 
