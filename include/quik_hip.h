@@ -270,8 +270,9 @@ int64_t quik_layer_workspace_bytes(const quik_layer *layer, int64_t rows);
 int quik_layer_forward(const quik_layer *layer, const void *x, int64_t rows, void *workspace,
                        int64_t workspace_bytes, void *splitk_workspace, int64_t splitk_bytes, void *out,
                        void *mid_event, void *stream);
-/* Calls of one or two token rows (asymmetric activations, a column map that streams) take ONE launch: the
- * weight-streaming kernel quantises the rows itself, with the arithmetic of quik_asym_quantize, and the workspace
+/* Calls of one or two token rows (a column map that streams; symmetric activations: fp16) take ONE launch: the
+ * weight-streaming kernel quantises the rows itself, with the arithmetic of quik_asym_quantize /
+ * quik_sym_quantize_mapped, and the workspace
  * stays untouched; mid_event is then recorded behind that launch.  quik_layer_set_one_launch(0) switches this off
  * for the process (the two-launch form; same output bits), 1 switches it on again (the default).  No counterpart in
  * the reference. */

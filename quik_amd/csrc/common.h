@@ -31,11 +31,13 @@ inline int colmap_require(const void *colmap, int64_t cols, int64_t num_int, int
   return (flags & need) == need ? QUIK_OK : QUIK_ERR_COLMAP;
 }
 
-// gemm.hip: MixedQLinear forward (asymmetric activations) for one or two token rows in ONE launch, the quantize
-// inside the kernel.  Returns kChainNotHandled (below) for shapes it leaves to the two-launch path.
+// gemm.hip: MixedQLinear forward for one or two token rows in ONE launch, the quantize inside the kernel
+// (w_red == NULL: symmetric activations with scale = max |x| / sym_divisor, fp16 only).  Returns kChainNotHandled
+// (below) for shapes it leaves to the two-launch path.
 int gemv_forward_one_launch(const void *x, int dtype, int64_t rows, int64_t cols, const void *colmap, int64_t num_int,
                             int64_t num_fp, int bits, const void *qw, const void *s_col, const void *w_red,
-                            const void *fp_w, const void *bias, int64_t N, void *out, hipStream_t st);
+                            const void *fp_w, const void *bias, int64_t N, void *out, float sym_divisor,
+                            hipStream_t st);
 
 // gemm.hip: integer GEMM + the fp16-arithmetic epilogue of the reference's fused ops in one launch (zero_row ==
 // NULL: symmetric form).  Returns kChainNotHandled for shapes it leaves to the two-launch path.

@@ -190,12 +190,12 @@ bool gemv_ok(const FusedArgs &p, bool quant = false) {
          gemv_smem(mt, p.kbytes, p.F) + gemv_table_bytes((p.N + kGemvWaves * num_cus() - 1) / (kGemvWaves * num_cus())) <=
              kLdsBytes;
 }
-template <int MODE, bool BF16, int MT, bool QUANT>
+template <int MODE, bool BF16, int MT, int QUANT>
 int launch_gemv_mt(const FusedArgs &p, const GemvQuant &q, hipStream_t st) {
   auto kern = gemv_decode_kernel<MODE, BF16, MT, QUANT>;
   if (int rc = prepare(kern, kLdsBytes)) return rc;  // (the size varies with the layer: set once to the most)
   // persistent waves, one column at a time each: two workgroups per CU when their LDS fits twice
-  const int64_t fixed = gemv_smem(MT, p.kbytes, p.F) + (QUANT ? gemv_quant_lds(q.cols, q.num_int).bytes : 0);
+  const int64_t fixed = gemv_smem(MT, p.kbytes, p.F) + (QUANT != kGemvNoQuant ? gemv_quant_lds(q.cols, q.num_int).bytes : 0);
   const int64_t per_cu = 2 * (fixed + 4096) <= kLdsBytes ? 2 : 1;
   int64_t grid = (p.N + kGemvWaves - 1) / kGemvWaves;
   if (grid > per_cu * num_cus()) grid = per_cu * num_cus();
@@ -204,7 +204,7 @@ int launch_gemv_mt(const FusedArgs &p, const GemvQuant &q, hipStream_t st) {
   hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(grid)), dim3(kGemvWaves * 64), static_cast<size_t>(smem), st, p, q);
   return check_launch();
 }
-template <int MODE, bool BF16, bool QUANT = false>
+template <int MODE, bool BF16, int QUANT = kGemvNoQuant>
 int launch_gemv(const FusedArgs &p, const GemvQuant &q, hipStream_t st) {
   if (p.M <= 1) return launch_gemv_mt<MODE, BF16, 1, QUANT>(p, q, st);
   if constexpr (kGemvMaxRows > 2) {  // (only built when the row limit is raised: gemv_ok() admits no such call otherwise)
@@ -618,14 +618,16 @@ extern "C" int quik_int8_matmul(const int8_t *A, const int8_t *B, int32_t *C, in
                         as_stream(stream));
 }
 
-// MixedQLinear forward (asymmetric activations) for at most kGemvMaxRows token rows in ONE launch: the kernel of
-// gemm_gemv.h quantises the rows itself.  kChainNotHandled: the shape is left to the two-launch path.
+// MixedQLinear forward for at most kGemvMaxRows token rows in ONE launch: the kernel of gemm_gemv.h quantises the
+// rows itself (asymmetric activations, or symmetric ones when w_red is NULL: fp16 only, scale = max |x| /
+// sym_divisor).  kChainNotHandled: the shape is left to the two-launch path.
 int quik::gemv_forward_one_launch(const void *x, int dtype, int64_t rows, int64_t cols, const void *colmap,
                                   int64_t num_int, int64_t num_fp, int bits, const void *qw, const void *s_col,
                                   const void *w_red, const void *fp_w, const void *bias, int64_t N, void *out,
-                                  hipStream_t st) {
+                                  float sym_divisor, hipStream_t st) {
+  const bool sym = w_red == nullptr;
   // (cols % 32, num_int % 128: the column map's group and unit tables arrive as whole 16-byte pieces)
-  if (rows < 1 || rows > kGemvMaxRows || !w_red || cols % 32 != 0 || cols > kStreamMaxCols || num_int % 128 != 0 ||
+  if (rows < 1 || rows > kGemvMaxRows || (sym && dtype != QUIK_F16) || cols % 32 != 0 || cols > kStreamMaxCols || num_int % 128 != 0 ||
       num_fp > kGemvWaves * 64 ||
       (reinterpret_cast<uintptr_t>(x) & 15) != 0 || N > (1 << 30))
     return kChainNotHandled;
@@ -646,7 +648,7 @@ int quik::gemv_forward_one_launch(const void *x, int dtype, int64_t rows, int64_
   p.ldo = static_cast<int>(N);
   p.kbytes = static_cast<int>(bits == 4 ? num_int / 2 : num_int);
   p.F = static_cast<int>(num_fp);
-  p.meta_stride = 2;
+  p.meta_stride = sym ? 1 : 2;
   p.shift = bits == 4 ? 8.0f : 128.0f;
   if (!gemv_ok(p, true)) return kChainNotHandled;
   GemvQuant q{};
@@ -658,9 +660,12 @@ int quik::gemv_forward_one_launch(const void *x, int dtype, int64_t rows, int64_
   q.gather_cols = reinterpret_cast<const uint16_t *>(cm + l.off_gcols);
   q.cols = static_cast<int>(cols), q.num_int = static_cast<int>(num_int), q.num_fp = static_cast<int>(num_fp);
   q.ngather = static_cast<int>(words[3]);
+  q.sym_divisor = sym_divisor;
   if (q.ngather > kGemvWaves * 64) return kChainNotHandled;  // (one gathered unit per thread)
-  if (bits == 4) return dtype == QUIK_F16 ? launch_gemv<kInt4, false, true>(p, q, st) : launch_gemv<kInt4, true, true>(p, q, st);
-  return dtype == QUIK_F16 ? launch_gemv<kInt8, false, true>(p, q, st) : launch_gemv<kInt8, true, true>(p, q, st);
+  if (sym) return bits == 4 ? launch_gemv<kInt4, false, kGemvSym>(p, q, st) : launch_gemv<kInt8, false, kGemvSym>(p, q, st);
+  if (bits == 4)
+    return dtype == QUIK_F16 ? launch_gemv<kInt4, false, kGemvAsym>(p, q, st) : launch_gemv<kInt4, true, kGemvAsym>(p, q, st);
+  return dtype == QUIK_F16 ? launch_gemv<kInt8, false, kGemvAsym>(p, q, st) : launch_gemv<kInt8, true, kGemvAsym>(p, q, st);
 }
 
 extern "C" int quik_mixed_linear_fwd(const void *qx, const void *qw, const void *meta, const void *s_col,

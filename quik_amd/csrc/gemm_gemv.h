@@ -20,7 +20,9 @@
 // min / max over the integer columns, scale, zero, the codes of every group of 8 source columns written to a staging
 // area in source order, then squeezed into the compact order of the weights' K axis through the column map's unit
 // tables (colmap.h); outlier values in the caller's order.  Codes and scales are bit-identical to the quantize
-// kernels', so the output is bit-identical to the two-launch form.
+// kernels', so the output is bit-identical to the two-launch form.  Symmetric activations (fp16): the largest |x|
+// in place of min / max, scale = fp16(max |x| / divisor), codes rne(fp16(x / scale)), no zero-point term
+// (reference: experiments/qlinear.py:97-103, src/symmetric/symmetric.cu:6-61).
 #pragma once
 #include "gemm_kernels.h"
 #include "quantize_math.h"
@@ -47,6 +49,7 @@ struct GemvQuant {
   const uint16_t *x, *fp_col, *unit, *gather_unit, *gather_cols;
   const uint32_t *grp;
   int cols, num_int, num_fp, ngather;
+  float sym_divisor;  // symmetric activations only: scale = fp16(max |x| / sym_divisor)
 };
 // LDS of the QUANT form behind the token rows' codes and the scalars' table: the raw row (2 bytes per column), the
 // column map's group words (4 bytes per 8 columns) and unit words (2 bytes per 16 integer columns), each in whole
@@ -81,7 +84,7 @@ __device__ __forceinline__ void gemv_copy_in(const void *src, int bytes, uint32_
 // values (fs_row), by all threads of the workgroup; returns the row's scale and zero as the kernels read them from
 // `meta`.  grp_s / unit_s: the column map's tables in LDS; goff / gunit / fcol: this thread's gathered unit (its 16
 // source columns, two per register) and outlier column.
-template <int BITS, bool BF16>
+template <int BITS, bool BF16, bool SYM>
 __device__ __forceinline__ void gemv_quantize_row(const uint8_t *raw, const uint32_t *grp_s, const uint16_t *unit_s,
                                                   const GemvQuant &q, const uint32_t (&goff)[8], int gunit, int fcol,
                                                   uint8_t *xs_row, uint8_t *fs_row, uint8_t *stage, float *red,
@@ -98,10 +101,17 @@ __device__ __forceinline__ void gemv_quantize_row(const uint8_t *raw, const uint
     const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      const float f = to_f32<BF16>(static_cast<uint16_t>(w[e >> 1] >> (16 * (e & 1))));
+      const uint16_t hbits = static_cast<uint16_t>(w[e >> 1] >> (16 * (e & 1)));
       const bool out = (skip >> e) & 1u;
-      mn = fminf(mn, out ? inf : f);
-      mx = fmaxf(mx, out ? -inf : f);
+      if constexpr (SYM) {
+        // largest |x| as a bit pattern (non-negative fp16 patterns order like integers, NaN patterns above infinity);
+        // a 15-bit integer is exact as a float, so the float reductions below carry it
+        mx = fmaxf(mx, out ? 0.0f : static_cast<float>(hbits & 0x7FFFu));
+      } else {
+        const float f = to_f32<BF16>(hbits);
+        mn = fminf(mn, out ? inf : f);
+        mx = fmaxf(mx, out ? -inf : f);
+      }
     }
   }
   mn = wave_min(mn);
@@ -119,14 +129,18 @@ __device__ __forceinline__ void gemv_quantize_row(const uint8_t *raw, const uint
     mx = fmaxf(mx, red[kGemvWaves + w]);
   }
   RowQuant<BF16> rq;
-  rq.init(mn, mx, BITS);
+  if constexpr (SYM) {
+    rq.init_sym(static_cast<uint32_t>(mx), q.sym_divisor);
+  } else {
+    rq.init(mn, mx, BITS);
+  }
   scale_out = to_f32<BF16>(rq.scale_bits);
   zero_out = to_f32<BF16>(rq.zero_bits);
   // codes of every group, source order; outlier values in the caller's order
   const bool slow = __builtin_amdgcn_readfirstlane(rq.slow ? 1 : 0);
   for (int g = tid; g < nvec; g += T) {
     const uint4 v = *reinterpret_cast<const uint4 *>(raw + g * 16);
-    const uint2 c = slow ? group_codes<BITS, BF16, true>(v, rq) : group_codes<BITS, BF16, false>(v, rq);
+    const uint2 c = slow ? group_codes<BITS, BF16, true, SYM>(v, rq) : group_codes<BITS, BF16, false, SYM>(v, rq);
     *reinterpret_cast<uint2 *>(stage + g * 8) = c;
   }
   if (tid < q.num_fp) reinterpret_cast<uint16_t *>(fs_row)[tid] = reinterpret_cast<const uint16_t *>(raw)[fcol];
@@ -196,9 +210,12 @@ __device__ __forceinline__ float wave_total(float v) {
   return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
 
-template <int MODE, bool BF16, int MT, bool QUANT = false>
+// QUANT: kGemvNoQuant (the token rows' codes come from a quantize launch), kGemvAsym / kGemvSym (quantised here)
+constexpr int kGemvNoQuant = 0, kGemvAsym = 1, kGemvSym = 2;
+template <int MODE, bool BF16, int MT, int QUANT = kGemvNoQuant>
 __global__ __launch_bounds__(kGemvWaves * 64) void gemv_decode_kernel(FusedArgs args, GemvQuant quant) {
   static_assert(MODE == kInt4 || MODE == kInt8, "integer codes");
+  static_assert(QUANT != kGemvSym || !BF16, "symmetric activations are fp16");
   struct {
     const uint8_t *qx, *qw;
     const uint16_t *meta, *s_col, *w_red, *fp_x, *fp_w, *bias;
@@ -246,7 +263,7 @@ __global__ __launch_bounds__(kGemvWaves * 64) void gemv_decode_kernel(FusedArgs 
   };
 
   float srow = 0.0f, zs = 0.0f;  // lane m keeps token row m's scale and zero-point term
-  if constexpr (QUANT) {
+  if constexpr (QUANT != kGemvNoQuant) {
     // ---- token rows -> codes and outlier values in LDS, quantised here.  The first row and the column map's
     // tables arrive together as direct copies; this thread's gathered unit and outlier column go to registers
     // (unconditional loads from clamped indices: under conditions each would wait for the one before it).
@@ -278,13 +295,13 @@ __global__ __launch_bounds__(kGemvWaves * 64) void gemv_decode_kernel(FusedArgs 
       else __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
       __syncthreads();
       float sc, zr;
-      gemv_quantize_row<MODE == kInt4 ? 4 : 8, BF16>(area + ql.raw, reinterpret_cast<const uint32_t *>(area + ql.grp),
+      gemv_quantize_row<MODE == kInt4 ? 4 : 8, BF16, QUANT == kGemvSym>(area + ql.raw, reinterpret_cast<const uint32_t *>(area + ql.grp),
                                                      reinterpret_cast<const uint16_t *>(area + ql.unit), quant, goff,
                                                      gunit, fcol, xs + m * xstride, fs + m * fstride, area + ql.stage,
                                                      reinterpret_cast<float *>(area + ql.red), sc, zr);
       if (lane == m) {
         srow = sc;
-        zs = zr + p.shift * sc;
+        zs = QUANT == kGemvSym ? 0.0f : zr + p.shift * sc;  // (symmetric: no zero-point term)
       }
     }
   } else {

@@ -83,11 +83,11 @@ extern "C" int quik_layer_forward(const quik_layer *layer, const void *x, int64_
   uint8_t *ws = static_cast<uint8_t *>(workspace);
   void *q = ws + p.off_q, *meta = ws + p.off_meta, *fp_x = l.num_fp > 0 ? ws + p.off_fp : nullptr;
   const void *w_red = l.symmetric ? nullptr : l.reduced_w;
-  if (!l.symmetric && !p.tiled && l.colmap_streams && layer_one_launch) {
+  if (!p.tiled && l.colmap_streams && layer_one_launch && (!l.symmetric || l.dtype == QUIK_F16)) {
     // one or two token rows: one launch, the quantize inside the weight-streaming kernel (the workspace is not used)
     const int rc = gemv_forward_one_launch(x, l.dtype, rows, l.in_features, l.colmap, l.num_int, l.num_fp, l.bits,
                                            l.int_weight, l.weights_scales, w_red, l.fp_weight, l.bias, l.out_features,
-                                           out, as_stream(stream));
+                                           out, l.sym_divisor, as_stream(stream));
     if (rc != kChainNotHandled) {
       if (rc == QUIK_OK && mid_event) {  // (profiling hook: there is no second launch to mark)
         if (hipError_t e = hipEventRecord(static_cast<hipEvent_t>(mid_event), as_stream(stream)); e != hipSuccess) {

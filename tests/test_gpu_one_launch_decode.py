@@ -1,5 +1,6 @@
 """MixedQLinear forward for one or two token rows: ONE launch (the weight-streaming matrix-vector kernel quantises
-the rows itself) against the two-launch form (quik_asym_quantize + quik_mixed_linear_fwd) and against the oracle.
+the rows itself) against the two-launch form (quik_asym_quantize / quik_sym_quantize_mapped + quik_mixed_linear_fwd)
+and against the oracle.
 
 The one-launch form uses the quantize kernels' own arithmetic on the same inputs, so codes and scales, and with them
 the outputs, must be bit-identical to the two-launch form; that form is switched on through
@@ -30,7 +31,7 @@ def _lib():
     lib.quik_layer_set_one_launch(1)
 
 
-def _layer(rng, N, n_in, F, bits, dtype, runs):
+def _layer(rng, N, n_in, F, bits, dtype, runs, symm=False):
     from quik_amd.qlinear import MixedQLinear
     if runs and F:
         starts = rng.permutation(n_in // 32)[:F // 4] * 32 + rng.integers(0, 20, F // 4)
@@ -53,7 +54,7 @@ def _layer(rng, N, n_in, F, bits, dtype, runs):
     lin = torch.nn.Linear(n_in, N, bias=True)
     lin.bias.data = torch.from_numpy(bias.astype(np.float32))
     mod = MixedQLinear.from_float(lin, torch.from_numpy(W), torch.from_numpy(s_w), None, torch.from_numpy(fi),
-                                  bits=bits).to(DEV)
+                                  symm=symm, bits=bits).to(DEV)
     if dtype == torch.bfloat16:
         mod = mod.to(torch.bfloat16)
     return mod, W, s_w, fi, ii, bias
@@ -152,7 +153,48 @@ def test_edge_rows_in_one_launch():
         assert torch.equal(out1.view(torch.int16), out2.view(torch.int16)), (a, b)
 
 
-def test_three_rows_and_symmetric_layers_keep_two_launches():
+@pytest.mark.parametrize("rows,N,n_in,F", [(1, 13824, 5120, 256), (2, 1000, 1024 + 64, 64), (1, 520, 2048, 0),
+                                           (2, 77, 256 + 32, 32)])
+def test_symmetric_layer_in_one_launch(rows, N, n_in, F):
+    """Symmetric activations (fp16, 4 bits: scale = max |x| / 4 as the reference's expression evaluates,
+    experiments/qlinear.py:97-103) take the same single launch: bit-identical to quik_sym_quantize_mapped + the fused
+    GEMM, within the fused forward's tolerance of the oracle's fp16-chain result; rows that hold a NaN, an infinity
+    or nothing but zeros included."""
+    from quik_amd import _lib as L
+    lib = L.load()
+    rng = np.random.default_rng(rows + N + n_in + F)
+    mod, W, s_w, fi, ii, bias = _layer(rng, N, n_in, F, 4, torch.float16, F > 0, symm=True)
+    x = rng.standard_normal((rows, n_in)).astype(np.float32)
+    x[:, fi] *= 50
+    variants = [x.astype(np.float16)]
+    for kind in range(3):
+        y = x.astype(np.float16).copy()
+        if kind == 0:
+            y[0, ii[3]] = np.nan
+        elif kind == 1:
+            y[rows - 1, ii[5]] = np.inf
+        else:
+            y[0, :] = 0
+        variants.append(y)
+    for k, xv in enumerate(variants):
+        xt = torch.from_numpy(xv).to(DEV)
+        lib.quik_layer_set_one_launch(1)
+        out1, ws1 = _call(mod, xt, 0x5A)
+        assert bool((ws1 == 0x5A).all()), "the one-launch form does not touch the workspace"
+        lib.quik_layer_set_one_launch(0)
+        out2, ws2 = _call(mod, xt, 0x5A)
+        lib.quik_layer_set_one_launch(1)
+        assert not bool((ws2 == 0x5A).all())
+        assert torch.equal(out1.view(torch.int16), out2.view(torch.int16)), k
+        if k == 0:
+            omod = qo.from_float(W, s_w, fi, 4, symm=True)
+            want, _ = qo.mixed_qlinear_forward(xv, omod, 4, bias=bias, symm=True)
+            w64 = want.astype(np.float64)
+            rms = float(np.sqrt((w64 ** 2).mean()))
+            assert np.abs(out1.float().cpu().numpy() - w64).max() <= 1e-2 * rms
+
+
+def test_three_rows_keep_two_launches():
     from quik_amd import _lib as L
     lib = L.load()
     rng = np.random.default_rng(12)
