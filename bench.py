@@ -560,7 +560,7 @@ def main():
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             step()
-        for _ in range(max(20, args.warmup)):   # past the clock transient that follows the idle gap of the capture
+        for _ in range(max(60, args.warmup)):   # past the clock transient (about 12 ms) that follows the idle gap of the capture
             graph.replay()
         torch.cuda.synchronize()
         g0, g1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
