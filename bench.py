@@ -173,6 +173,7 @@ BLOCK_WORKLOADS = {
     # name: (batch, new tokens per sequence, tokens already in the KV cache)
     "llama2-70b.decoder_block.prefill": (16, 512, 0),
     "llama2-70b.decoder_block.decode": (64, 1, 512),
+    "llama2-70b.decoder_block.decode1": (1, 1, 512),     # single-stream decode: every linear is one launch
 }
 BLOCK_DIMS = dict(hidden=8192, heads=64, kv_heads=8, head_dim=128, mlp=28672, F=256)
 
@@ -345,8 +346,49 @@ def bench_block(args):
     block_f_ms = timed(lambda: blk.forward(x, True, cache))
     lin_ms = timed(lambda: linears(False))
     lin_f_ms = timed(lambda: linears(True))
+    # the linears of the block (fused groups) replayed from a HIP graph: what a serving loop that captures the
+    # layer sees; every replay is checked against the eager outputs
+    lin_graph_ms = None
+    try:
+        outs = {}
+
+        def linears_out():
+            outs["qkv"] = blk.g_qkv(h_in)
+            outs["o"] = L["o"](a_in)
+            outs["mlp"] = blk.g_mlp(h_in)
+            outs["down"] = L["down"](m_in)
+
+        linears_out()
+        want = {k: [t.clone() for t in (v if isinstance(v, (tuple, list)) else [v])] for k, v in outs.items()}
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            linears_out()
+        torch.cuda.current_stream().wait_stream(side)
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            linears_out()
+        for _ in range(3):
+            g.replay()
+            torch.cuda.synchronize()
+            for k, v in outs.items():
+                for t, w in zip(v if isinstance(v, (tuple, list)) else [v], want[k]):
+                    assert torch.equal(t, w), f"graph replay of {k} differs from the eager result"
+        for _ in range(max(20, args.warmup)):
+            g.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(args.steps):
+            g.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        lin_graph_ms = e0.elapsed_time(e1) / args.steps
+    except Exception as exc:   # noqa: BLE001  (an extra figure)
+        print(f"bench.py: graph replay of the linears skipped: {exc}", file=sys.stderr)
     M = B * S
     ops = sum(2.0 * M * m.out_features * m.int_features_num for m in L.values())
+    weight_bytes = sum(m.out_features * (m.int_features_num * m.bits // 8 + m.fp_features_num * 2) for m in L.values())
     res = {
         "metric": "decoder block latency, Llama-2-70B dims, 7 MixedQLinear + PyTorch norm/attention, 1 GPU",
         "value": round(block_f_ms, 4), "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -355,7 +397,10 @@ def bench_block(args):
         "config": {"workload": f"{args.workload}: batch {B} x {S} new tokens, {past} cached; q/k/v and gate/up as "
                                f"one GEMM each (FusedMixedQLinearGroup)", "tokens": M, **d},
         "block_ms_seven_modules_shared_input": round(block_ms, 4),
-        "linears_only_ms": {"seven_modules_shared_input": round(lin_ms, 4), "fused_groups": round(lin_f_ms, 4)},
+        "linears_only_ms": {"seven_modules_shared_input": round(lin_ms, 4), "fused_groups": round(lin_f_ms, 4),
+                            "fused_groups_graph_replay": None if lin_graph_ms is None else round(lin_graph_ms, 4)},
+        "linears_weight_bytes_reference_layout": weight_bytes,
+        "linears_weight_stream_gbps": round(weight_bytes / (min(lin_graph_ms or lin_f_ms, lin_f_ms) * 1e-3) / 1e9, 1),
         "linears_int_tops": round(ops / (lin_f_ms * 1e-3) / 1e12, 1),
         "linears_pct_int8_mfma_peak": round(100.0 * ops / (lin_f_ms * 1e-3) / 1e12 / PEAK_INT8_TOPS, 2),
     }
