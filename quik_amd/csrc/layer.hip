@@ -5,13 +5,15 @@
 // of the reference, for callers that want one boundary crossing per layer.)
 #include "common.h"
 
+#include <atomic>
+
 namespace quik {
 namespace {
 
 inline int64_t align256(int64_t v) { return (v + 255) & ~int64_t(255); }
 
 // quik_layer_set_one_launch: tests and measurements switch the one-launch form of small calls off to compare
-bool layer_one_launch = true;
+std::atomic<bool> layer_one_launch{true};  // (read by every forward, possibly from several host threads)
 
 struct LayerPlan {
   bool tiled;
@@ -58,7 +60,7 @@ LayerPlan plan_layer(const quik_layer *l, int64_t rows) {
 
 using namespace quik;
 
-extern "C" void quik_layer_set_one_launch(int on) { layer_one_launch = on != 0; }
+extern "C" void quik_layer_set_one_launch(int on) { layer_one_launch.store(on != 0, std::memory_order_relaxed); }
 
 extern "C" int64_t quik_layer_workspace_bytes(const quik_layer *layer, int64_t rows) {
   if (!layer_valid(layer) || rows <= 0) return 0;
@@ -83,7 +85,7 @@ extern "C" int quik_layer_forward(const quik_layer *layer, const void *x, int64_
   uint8_t *ws = static_cast<uint8_t *>(workspace);
   void *q = ws + p.off_q, *meta = ws + p.off_meta, *fp_x = l.num_fp > 0 ? ws + p.off_fp : nullptr;
   const void *w_red = l.symmetric ? nullptr : l.reduced_w;
-  if (!p.tiled && l.colmap_streams && layer_one_launch && (!l.symmetric || l.dtype == QUIK_F16)) {
+  if (!p.tiled && l.colmap_streams && layer_one_launch.load(std::memory_order_relaxed) && (!l.symmetric || l.dtype == QUIK_F16)) {
     // one or two token rows: one launch, the quantize inside the weight-streaming kernel (the workspace is not used)
     const int rc = gemv_forward_one_launch(x, l.dtype, rows, l.in_features, l.colmap, l.num_int, l.num_fp, l.bits,
                                            l.int_weight, l.weights_scales, w_red, l.fp_weight, l.bias, l.out_features,
