@@ -131,6 +131,7 @@ class SharedQuantizedInput:
         fused.six_bit_path = first.six_bit_path
         fused.six_bit_min_rows, fused.tile8_min_rows = first.six_bit_min_rows, first.tile8_min_rows
         fused.sym_divisor = first.sym_divisor
+        fused.transient_tiled_copy = first.transient_tiled_copy
         # the members' buffers become row slices (contiguous) of the concatenated ones: no second copy
         lo = 0
         for m in mods:
@@ -209,6 +210,12 @@ class MixedQLinear(torch.nn.Module):
     six_bit_min_rows = 33    # up to 32 rows the weight-streaming decode kernel on the packed int4 weights is the right one
     tile8_min_rows = 33      # the same switch for 8 bits (the tile-ordered kernel itself takes any row count)
     fuse_shared_groups = True   # members of a SharedQuantizedInput group run as one quantize + one GEMM (see there)
+    # Memory policy: True = the tile-ordered weight copy is NOT kept.  Every call of more than 32 rows repacks the
+    # reference's buffers into a temporary operand buffer (one launch, the buffer goes back to torch's allocator
+    # behind the GEMM, so consecutive layers reuse the same block) and runs the same tile-ordered GEMM: output bits
+    # unchanged, weights resident once (the reference's layout), each such call longer by the repacking
+    # (see weight_bytes(); set on the class for every layer or on single modules).
+    transient_tiled_copy = False
 
     def __init__(self, in_features, out_features, shared_input=None,
                  fp_features_num=0, symm=False, bits=4, dtype=torch.float16, fused=True, allocate=True):
@@ -287,6 +294,11 @@ class MixedQLinear(torch.nn.Module):
             return self._w6
         fp_w = self.fp_weight if self.fp_features_num > 0 else \
             torch.empty((self.out_features, 0), dtype=self.dtype, device=self.int_weight.device)
+        if self.transient_tiled_copy:    # a fresh buffer per call, never kept
+            self._w6 = self._w6_key = None
+            if self.bits == 4:
+                return matmul.pack_weight_fp6(self.int_weight, fp_w, self._column_map())
+            return matmul.pack_weight_tile8(self.int_weight, fp_w)
         key = (self.int_weight.data_ptr(), self.int_weight._version, fp_w.data_ptr(), fp_w._version,
                self.int_weight.device, self._column_map().data_ptr())
         if self._w6 is None or self._w6_key != key:
@@ -320,6 +332,11 @@ class MixedQLinear(torch.nn.Module):
         self._descs.clear()
 
     def release_row_major_weights(self):
+        if self.transient_tiled_copy:
+            raise RuntimeError("transient_tiled_copy repacks the row-major weights on every call: they cannot be released")
+        return self._release_row_major_weights()
+
+    def _release_row_major_weights(self):
         """Keep only the tile-ordered copy: int_weight and fp_weight become empty tensors and EVERY call, down to
         one row, takes the tile-ordered path (same output bits above 32 rows; up to 32 rows equal within rounding
         of the fp32 sums, and slower than the weight-streaming kernel, which reads the packed nibbles).  The
@@ -359,6 +376,15 @@ class MixedQLinear(torch.nn.Module):
         # (the scalar switches below are baked into the descriptor too: changing one after a forward rebuilds it)
         key = tuple((b.data_ptr(), b._version) if b is not None else None for b in bufs) + \
             (self.six_bit_min_rows, self.tile8_min_rows, float(self.sym_divisor), bool(self.six_bit_path))
+        transient = tiled and self.transient_tiled_copy and not self._row_major_released
+        if transient:
+            # the cached descriptor of the row-major form, copied, with this call's temporary operand buffer
+            base, sizes = self._descriptor(False)
+            d = L.QuikLayer.from_buffer_copy(base)
+            w6 = self._weight6()
+            d.tiled_weight = w6.data_ptr()
+            d._keep = w6     # (alive until the caller drops the descriptor, i.e. behind the launch)
+            return d, self._descs.setdefault("transient_sizes", {})
         entry = self._descs.get(tiled)
         if entry is None or entry[0] != key:
             w6 = self._weight6() if tiled else None

@@ -227,6 +227,57 @@ def test_one_resident_copy_of_the_weights(bits, symm, n_in, F):
         tiled_only.release_tiled_weights()
 
 
+@pytest.mark.parametrize("bits,symm,n_in,F", [(4, False, 2048 + 64, 64), (8, False, 1280 + 256, 256),
+                                              (4, True, 1024 + 32, 32)])
+def test_transient_tile_ordered_copy(bits, symm, n_in, F, monkeypatch):
+    """transient_tiled_copy: calls of more than 32 rows repack the reference's buffers into a temporary operand
+    buffer and run the same tile-ordered GEMM.  Same output bits as the default module at every row count (the
+    small calls are untouched), nothing tile-ordered kept between calls, one packing launch per large call; the
+    same under HIP graph replays."""
+    from quik_amd import matmul
+    N = 384
+    rng = np.random.default_rng(bits + F + 1)
+    W, s_w, fi = _layer(rng, N, n_in, F, bits)
+    bias = rng.standard_normal(N).astype(np.float16)
+    both = _module(W, s_w, fi, bits, bias, symm)
+    lean = _module(W, s_w, fi, bits, bias, symm)
+    lean.transient_tiled_copy = True
+    packs = []
+    for name in ("pack_weight_fp6", "pack_weight_tile8"):
+        orig = getattr(matmul, name)
+        monkeypatch.setattr(matmul, name, lambda *a, _o=orig, **k: (packs.append(1), _o(*a, **k))[1])
+    for M in (1, 32, 33, 200, 33):
+        x = rng.standard_normal((M, n_in)).astype(np.float32)
+        x[:, fi] *= 50
+        xt = torch.from_numpy(x.astype(np.float16)).to(DEV)
+        want = both(xt)
+        n0 = len(packs)
+        got = lean(xt)
+        assert torch.equal(_bits(got), _bits(want)), M
+        assert len(packs) - n0 == (1 if M > 32 else 0)
+        wb = lean.weight_bytes()
+        assert wb["tiled"] == 0 and wb["row_major"] == wb["reference_layout"] and lean._w6 is None
+    with pytest.raises(RuntimeError):
+        lean.release_row_major_weights()
+    # graph replays: the packing launch is part of the graph
+    xt = torch.from_numpy((rng.standard_normal((70, n_in)) * 1.0).astype(np.float16)).to(DEV)
+    want = both(xt).clone()
+    lean(xt)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        lean(xt)
+    torch.cuda.current_stream().wait_stream(side)
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        out = lean(xt)
+    for _ in range(3):
+        out.zero_()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(_bits(out), _bits(want))
+
+
 # ------------------------------------------------------------------------------ shared-input groups
 @pytest.mark.parametrize("rows,bits,symm,bias", [(200, 4, False, False), (16, 4, False, True), (72, 4, True, False),
                                                  (130, 8, False, False), (1, 8, False, False)])
