@@ -144,6 +144,70 @@ def test_default_route_at_benchmark_shapes(case):
     check_against_oracle(out, x, W, s_w, fi, bits, symm, spot_tiles(M, N))
 
 
+def test_default_route_random_shapes_against_the_oracle():
+    """Seeded sweep over module calls of any size: row counts on both sides of every switch of kernels, ragged N,
+    K and F at the granularity the GEMM's row alignment allows (shapes the tile-ordered paths refuse included),
+    W4A4 / W8A8 / symmetric, fp16 against the oracle's forward on the whole output, bf16 against the row-major
+    route of the same module bit for bit.  Elementwise bound: 1e-2 x output RMS, or two fp16 ulps of the element
+    where that is larger (heavy-tailed outputs)."""
+    from quik_amd.qlinear import MixedQLinear
+    rng = np.random.default_rng(4242)
+    done = 0
+    while done < 40:
+        bits = int(rng.choice([4, 8]))
+        symm = bits == 4 and rng.random() < 0.2
+        bf16 = (not symm) and rng.random() < 0.25
+        M = int(rng.choice([1, 2, 3, 16, 32, 33, 48, 64, 65, 100, 128, 129, 256, 257, 300, 511, 700, 1100]))
+        K = (32 if bits == 4 else 16) * int(rng.choice([1, 2, 3, 4, 6, 8, 12, 16, 31, 32, 40, 64, 77, 128]))
+        F = 8 * int(rng.choice([0, 0, 1, 2, 4, 8, 9, 16, 32, 33]))
+        N = int(rng.choice([5, 8, 31, 64, 100, 130, 256, 513, 1000, 2048, 4100]))
+        if M * N < 64 or M * N * K > 2e9:
+            continue
+        done += 1
+        n_in = K + F
+        fi = rng.permutation(n_in)[:F].astype(np.int64)
+        keep = np.ones(n_in, bool)
+        keep[fi] = False
+        ii = np.arange(n_in)[keep]
+        lo, hi = (-8, 8) if bits == 4 else (-127, 128)
+        s_w = rng.uniform(0.001, 0.01, (N, 1)).astype(np.float16)
+        W = np.zeros((N, n_in), np.float16)
+        W[:, ii] = (rng.integers(lo, hi, (N, K)) * s_w.astype(np.float32)).astype(np.float16)
+        W[:, fi] = (0.02 * rng.standard_normal((N, F))).astype(np.float16)
+        bias = (0.1 * rng.standard_normal(N)).astype(np.float16) if rng.random() < 0.5 else None
+        lin = torch.nn.Linear(n_in, N, bias=bias is not None)
+        if bias is not None:
+            lin.bias.data = torch.from_numpy(bias.astype(np.float32))
+        x = rng.standard_normal((M, n_in)).astype(np.float32)
+        if rng.random() < 0.5:
+            x[:, fi] *= 50
+        elif F:
+            x[:, fi] = np.clip(20 * rng.standard_t(3, (M, F)), -6e4, 6e4)
+        x = x.astype(np.float16)
+        case = (done, M, N, K, F, bits, bool(symm), bool(bf16), bias is not None)
+        mod = MixedQLinear.from_float(lin, torch.from_numpy(W), torch.from_numpy(s_w), None,
+                                      torch.from_numpy(fi) if F else None, symm=bool(symm), bits=bits).to(DEV)
+        if bf16:
+            mod = mod.to(torch.bfloat16)
+            xt = torch.from_numpy(x).to(DEV).to(torch.bfloat16)
+            out = mod(xt)[0]
+            mod.six_bit_path = False
+            assert torch.equal(_bits(out), _bits(mod(xt)[0])), case
+            continue
+        omod = qo.from_float(W, s_w, fi, bits, symm=bool(symm))
+        want, _ = qo.mixed_qlinear_forward(x, omod, bits, bias, symm=bool(symm))
+        w64 = want.astype(np.float64)
+        fin = np.isfinite(w64)
+        rms = np.sqrt((w64[fin] ** 2).mean()) + 1e-30
+        xt = torch.from_numpy(x).to(DEV)
+        got = mod(xt)[0]
+        d = np.abs(got.float().cpu().numpy().astype(np.float64) - w64)[fin]
+        assert not (d > np.maximum(1e-2 * rms, 2.0 ** -9 * np.abs(w64[fin]))).any(), (case, d.max(), rms)
+        if M > 32 and not symm:
+            mod.six_bit_path = False
+            assert torch.equal(_bits(got), _bits(mod(xt)[0])), case
+
+
 def test_default_route_three_dimensional_prefill_input():
     """The decoder block's prefill hands (16, 512, 8192); the module flattens it and returns (16, 512, N)."""
     M, n_in, N, F, bits = 8192, 8192, 1024, 256, 4
