@@ -1610,6 +1610,18 @@ int launch_fp6_wave(const void *x, int64_t rows, int64_t cols, const uint8_t *cm
                        static_cast<uint16_t *>(meta), sym_divisor);
     return check_launch();
   };
+  // Few rows: workgroups of two waves, so that the launch still reaches every CU (512 rows in workgroups of eight
+  // are 64 workgroups, a quarter of the CUs, each taking eight rows in turn).
+  if (rows * 2 <= int64_t(8) * num_cus()) {
+    switch (J) {
+      case 1: return go(quantize_fp6_wave_kernel<BF16, SYM, 1, 2>, 2);
+      case 2: return go(quantize_fp6_wave_kernel<BF16, SYM, 2, 2>, 2);
+      case 3: return go(quantize_fp6_wave_kernel<BF16, SYM, 3, 2>, 2);
+      case 4: return go(quantize_fp6_wave_kernel<BF16, SYM, 4, 2>, 2);
+      case 5: return go(quantize_fp6_wave_kernel<BF16, SYM, 5, 2>, 2);
+      default: break;
+    }
+  }
   switch (J) {  // fragments per lane known at compile time: the loops over them unroll
     case 1: return go(quantize_fp6_wave_kernel<BF16, SYM, 1, 8>, 8);
     case 2: return go(quantize_fp6_wave_kernel<BF16, SYM, 2, 8>, 8);
