@@ -719,7 +719,7 @@ def main():
         "verified_vs_oracle": None if spot is None else {"tiles": 3, "max_abs_err_over_rms": round(spot, 6),
                                                          "tolerance": 1e-2},
         "roofline": roofline,
-        "roofline_quantize": None if one_launch else {"kernel": (f"quantize_fp6_wave_kernel (one wave per token row, {'two' if M <= 1024 else 'eight'} rows per workgroup, 6-bit operand output)" if six and bits == 4
+        "roofline_quantize": None if one_launch else {"kernel": (f"quantize_fp6_wave_kernel (one wave per token row, {'two' if M <= 1536 else 'eight'} rows per workgroup, 6-bit operand output)" if six and bits == 4
                                          else "quantize_tile8_ring_kernel (row copied into an LDS ring, int8 operand output in tile order)"
                                          if six and bits == 8 and n_in > 8192 and str(x.dtype) == "torch.float16"
                                          else "asym_quantize_stream_kernel" + (" (tile-ordered operand output)" if six else "")),

@@ -1611,8 +1611,10 @@ int launch_fp6_wave(const void *x, int64_t rows, int64_t cols, const uint8_t *cm
     return check_launch();
   };
   // Few rows: workgroups of two waves, so that the launch still reaches every CU (512 rows in workgroups of eight
-  // are 64 workgroups, a quarter of the CUs, each taking eight rows in turn).
-  if (rows * 2 <= int64_t(8) * num_cus()) {
+  // are 64 workgroups, a quarter of the CUs, each taking eight rows in turn).  Measured at 8192 columns, period per
+  // launch with two / eight waves: 1280 rows 8.7 / 9.1 us, 1536 rows 9.4 / 9.7, 1792 rows 10.5 / 10.4, 2048 rows
+  // 11.7 / 11.5: the switch is at six rows per CU.
+  if (rows <= int64_t(6) * num_cus()) {
     switch (J) {
       case 1: return go(quantize_fp6_wave_kernel<BF16, SYM, 1, 2>, 2);
       case 2: return go(quantize_fp6_wave_kernel<BF16, SYM, 2, 2>, 2);
