@@ -65,7 +65,7 @@ PEAK_HBM_GBPS = 8000.0    # MI355X HBM3E, published
 # (`traffic_source`).  (gemm6 / quantize6: the kernels of the 6-bit matrix-core path, the default; gemm / quantize:
 # --int8-mfma)
 MEASURED_TRAFFIC_BYTES = {
-    "llama2-70b.gate_proj": {"gemm": 809.4e6, "quantize": 43.0e6, "gemm6": 757.0e6, "quantize6": 47.1e6},
+    "llama2-70b.gate_proj": {"gemm": 809.4e6, "quantize": 43.0e6, "gemm6": 754.7e6, "quantize6": 47.1e6},
 }
 TRAFFIC_SOURCE = {
     "gemm6": "offline: profiles/gemm_fused6_split_kernel__llama2-70b.gate_proj.md (rocprofv3 --pmc FETCH_SIZE / "
